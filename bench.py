@@ -1,0 +1,306 @@
+"""Decode throughput of the FP8 + KV-cache path on one MI355X, at the headline shape.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[3]): nanochat d26 (n_embd 1664, 13 heads, head_dim 128, 26 layers,
+vocab 32768, window pattern SSSL), bf16 weights with FP8 linears, random init seed 2; one prompt of
+random token ids is prefilled at batch 1, the KV cache is replicated to 64 rows, and greedy decoding
+runs through Engine.generate until the context reaches 2048 tokens.  A "step" is one iteration of that
+loop: sample for all 64 rows + one GPT.forward(ids[64,1], kv_cache).  The prompt length is chosen so
+that the last timed step ends at context 2048 (1792 prompt tokens for the default 8 + 248 steps).
+
+One JSON line is printed with tokens/s, the roofline of the dominant kernel (decode attention, HBM
+bound; its time is measured with HIP events on the launch stream in extra steps right after the timed
+region), FP8 GEMM rates at the isolated Float8Linear shapes, and a CPU baseline (the CPU oracle, a
+port of the reference's CPU behaviour, timed on this box's host cores on a bounded sample).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12
+FP8_PEAK = 5.0e15
+D26 = dict(sequence_len=2048, vocab_size=32768, n_layer=26, n_head=13, n_kv_head=13, n_embd=1664, window_pattern="SSSL")
+BATCH = 64
+CONTEXT = 2048
+
+
+class RangeTokenizer:
+    """Engine needs four tokenizer methods; specials are placed outside the vocabulary so that random
+    greedy decoding never terminates a row early."""
+
+    def encode_special(self, s):
+        return 1 << 30
+
+    def get_bos_token_id(self):
+        return (1 << 30) + 1
+
+    def encode(self, s, prepend=None):
+        return []
+
+    def decode(self, tokens):
+        return ""
+
+
+def build_model(device, seed=2):
+    """Random init of the d26 architecture directly on the GPU (same distributions as the reference's
+    init_weights, with non-zero projections so every kernel does real work)."""
+    from nanochat_amd.fp8 import convert_to_float8_training, fp8_module_filter
+    from nanochat_amd.gpt import GPT, GPTConfig
+    cfg = GPTConfig(**D26)
+    with torch.device("meta"):
+        model = GPT(cfg)
+    model.to_empty(device=device)
+    g = torch.Generator(device=device).manual_seed(seed)
+    s = 3 ** 0.5 * cfg.n_embd ** -0.5
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("wte.weight"):
+                p.normal_(0.0, 0.8, generator=g)
+            elif name == "lm_head.weight":
+                p.normal_(0.0, 0.03, generator=g)
+            elif "value_embeds" in name or "c_q" in name or "c_k" in name or "c_v" in name or "attn.c_proj" in name:
+                p.uniform_(-s, s, generator=g)
+            elif "c_fc" in name:
+                p.uniform_(-0.4 * s, 0.4 * s, generator=g)
+            elif "mlp.c_proj" in name:
+                p.uniform_(-0.5 * s, 0.5 * s, generator=g)
+            elif "gate" in name:
+                p.uniform_(-0.5, 0.5, generator=g)
+            elif name == "resid_lambdas":
+                p.copy_(torch.linspace(1.15, 1.05, cfg.n_layer))
+            elif name == "x0_lambdas":
+                p.copy_(torch.linspace(0.20, 0.05, cfg.n_layer))
+            elif name == "smear_lambda":
+                p.fill_(0.35)
+            elif name == "backout_lambda":
+                p.fill_(0.2)
+            else:
+                raise RuntimeError(f"unhandled parameter {name}")
+        # bf16 weights with FP8 linears
+        model.to(torch.bfloat16)
+    convert_to_float8_training(model, module_filter_fn=fp8_module_filter)
+    return model
+
+
+def attention_bytes_per_step(model, batch, context):
+    """Algorithmic KV bytes one decode step reads at this context: per layer B * 2 * Hkv * D * 2 bytes
+    per visible key, min(context, window + 1) visible keys."""
+    cfg = model.config
+    per_key = batch * 2 * cfg.n_kv_head * 128 * 2
+    return sum(per_key * min(context, w + 1) for w, _ in model.window_sizes)
+
+
+def read_profile(lib, cls):
+    ms, units, n = C.c_double(), C.c_double(), C.c_int64()
+    rc = lib.nc_profile_read(cls, C.byref(ms), C.byref(units), C.byref(n))
+    assert rc == 0
+    return ms.value, units.value, n.value
+
+
+def gemm_rates(device):
+    """FP8 GEMM TFLOP/s at the isolated Float8Linear shapes (M=8192), kernel time by HIP events."""
+    from nanochat_amd import _lib, ops
+    lib = _lib.lib()
+    out = {}
+    g = torch.Generator(device=device).manual_seed(0)
+    for K, N in [(1664, 4992), (1664, 1664), (1664, 6656), (6656, 1664)]:
+        M = 8192
+        a = torch.randn(M, K, device=device, generator=g).bfloat16()
+        w = ((torch.rand(N, K, device=device, generator=g) * 2 - 1) * (3.0 / K) ** 0.5).bfloat16()
+        a8, ia, _ = ops.fp8_quantize(a)
+        w8, iw, _ = ops.fp8_quantize(w)
+        iw = iw.reshape(1)
+        res = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+        for _ in range(3):
+            ops.fp8_gemm(a8, w8, ia, iw, out=res)
+        torch.cuda.synchronize()
+        lib.nc_profile_enable(1)
+        for _ in range(20):
+            ops.fp8_gemm(a8, w8, ia, iw, out=res)
+        torch.cuda.synchronize()
+        ms, flops, n = read_profile(lib, 1)
+        lib.nc_profile_enable(0)
+        # quantize (amax + convert) of the activation, 3 bytes per element algorithmic
+        lib.nc_profile_enable(1)
+        for _ in range(20):
+            ops.fp8_quantize(a)
+        torch.cuda.synchronize()
+        qms, qbytes, qn = read_profile(lib, 2)
+        lib.nc_profile_enable(0)
+        tf = flops / (ms * 1e-3) / 1e12
+        out[f"K{K}_N{N}"] = {"us": round(ms / n * 1e3, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
+                             "quantize_us": round(qms / qn * 1e3, 2),
+                             "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1)}
+    return out
+
+
+def cpu_baseline(budget_s=25.0):
+    """One decode step of the CPU oracle at the same shape (d26, 64 rows, context 1792), bf16 with
+    fp8-emulated linears, weights re-quantized on every call as the reference does (fp8.py:136)."""
+    from oracle import decode_ref, gpt_ref
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    cfg = gpt_ref.GPTConfig(**D26)
+    t0 = time.time()
+    g = torch.Generator().manual_seed(2)
+    E, L, V = cfg.n_embd, cfg.n_layer, cfg.vocab_size
+    s = 3 ** 0.5 * E ** -0.5
+    p = {}
+
+    # one random matrix per shape, cloned per layer: distinct memory (no cache reuse across layers) without
+    # paying the host RNG for 1.9e9 elements; timing does not depend on the values
+    def u(*shape, a):
+        return (torch.rand(*shape, generator=g) * 2 * a - a).bfloat16()
+    w_ee, w_fc, w_pr, w_ve = u(E, E, a=s), u(4 * E, E, a=0.4 * s), u(E, 4 * E, a=0.5 * s), u(V, E, a=s)
+    p["transformer.wte.weight"] = torch.randn(V, E, generator=g).bfloat16()
+    p["lm_head.weight"] = (torch.randn(V, E, generator=g) * 0.03).bfloat16()
+    for i in range(L):
+        pre = f"transformer.h.{i}."
+        for nm in ("attn.c_q", "attn.c_k", "attn.c_v", "attn.c_proj"):
+            p[pre + nm + ".weight"] = w_ee.clone()
+        p[pre + "mlp.c_fc.weight"] = w_fc.clone()
+        p[pre + "mlp.c_proj.weight"] = w_pr.clone()
+        if gpt_ref.has_ve(i, L):
+            p[f"value_embeds.{i}.weight"] = w_ve.clone()
+            p[pre + "attn.ve_gate.weight"] = torch.rand(cfg.n_kv_head, 12, generator=g) - 0.5
+    p["resid_lambdas"] = torch.linspace(1.15, 1.05, L)
+    p["x0_lambdas"] = torch.linspace(0.20, 0.05, L)
+    p["smear_lambda"] = torch.full((1,), 0.35)
+    p["backout_lambda"] = torch.full((1,), 0.2)
+    p["smear_gate.weight"] = torch.rand(1, 24, generator=g) - 0.5
+    rt = gpt_ref.Runtime(cfg, p, compute_dtype=torch.bfloat16, fp8=True, cache_weights=False)
+    ctx = 1792
+    cache = decode_ref.new_cache(cfg, BATCH, ctx + 8, torch.bfloat16)
+    # a filled cache without paying for a CPU prefill: random keys/values of the right magnitude
+    kblk = (torch.randn(1, 1, ctx, cfg.n_kv_head, 128, generator=g) * 1.2).bfloat16()
+    vblk = (torch.randn(1, 1, ctx, cfg.n_kv_head, 128, generator=g) * 0.5).bfloat16()
+    cache.k_cache[:, :, :ctx] = kblk
+    cache.v_cache[:, :, :ctx] = vblk
+    cache.cache_seqlens.fill_(ctx)
+    cache.prev_embedding = torch.randn(BATCH, 1, E, generator=g).bfloat16()
+    setup_s = time.time() - t0
+    ids = torch.randint(0, V, (BATCH, 1), generator=g)
+    steps, spent = 0, 0.0
+    while steps < 1 or (spent < budget_s and steps < 4):
+        t1 = time.time()
+        logits = gpt_ref.forward(rt, ids, cache)
+        ids = logits[:, -1].argmax(-1, keepdim=True)
+        spent += time.time() - t1
+        steps += 1
+    return {"value": round(BATCH * steps / spent, 3), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{steps} decode step(s) of the CPU oracle at d26, 64 rows, context {ctx} (random-filled cache), bf16 + "
+                      f"fp8-emulated linears with per-call weight quantization as in the reference; setup {setup_s:.0f}s not timed",
+            "s_per_step": round(spent / steps, 3)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=248)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--profile-steps", type=int, default=16)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (decode shards by batch row; see DESIGN.md). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    from nanochat_amd import _lib
+    from nanochat_amd.engine import Engine
+    lib = _lib.lib()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    K, W, P = args.steps, args.warmup, args.profile_steps
+    total_new = W + K + P
+    prompt_len = CONTEXT - (W + K)            # the last timed step brings the context to 2048
+    assert prompt_len >= 1, "steps + warmup must stay below the 2048-token context"
+    model = build_model(device)
+    engine = Engine(model, RangeTokenizer())
+    g = torch.Generator().manual_seed(2)
+    prompt = torch.randint(0, D26["vocab_size"], (prompt_len,), generator=g).tolist()
+
+    # Engine.generate sizes the decode cache as prompt + max_tokens; the profiled extra steps run past the
+    # timed region, so the rotary/cache bound is 2048 + P (the rotary table covers 10x the context).
+    gen = engine.generate(prompt, num_samples=BATCH, max_tokens=total_new + 1, temperature=0.0)
+    t_pre = time.perf_counter()
+    next(gen)                                  # prefill + cache replication + first sample + first forward
+    torch.cuda.synchronize()
+    ttft = time.perf_counter() - t_pre
+    for _ in range(W - 1):
+        next(gen)
+    torch.cuda.synchronize()
+    step_times = []
+    t0 = time.perf_counter()
+    for _ in range(K):
+        t1 = time.perf_counter()
+        next(gen)
+        step_times.append(time.perf_counter() - t1)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    tok_per_s = BATCH * K / elapsed
+
+    # ---- kernel-level timing, HIP events on the launch stream, same process and state
+    lib.nc_profile_enable(1)
+    for _ in range(P):
+        next(gen)
+    torch.cuda.synchronize()
+    prof = {c: read_profile(lib, c) for c in range(5)}
+    lib.nc_profile_enable(0)
+    gen.close()
+    att_ms, _, att_n = prof[0]
+    ctx_mid = CONTEXT + P // 2                 # profiled steps sit just past the timed region
+    att_bytes_step = attention_bytes_per_step(model, BATCH, ctx_mid)
+    launches_per_step = model.config.n_layer
+    att_avg_s = att_ms * 1e-3 / att_n
+    att_bytes_launch = att_bytes_step / launches_per_step
+    achieved = att_bytes_launch / att_avg_s
+    per_step_ms = {name: round(prof[c][0] / P, 3) for c, name in enumerate(["attention", "fp8_gemm", "quantize", "rows", "sampler"])}
+
+    result = {
+        "metric": "decode tokens/sec @ d26 bs64 ctx2048",
+        "value": round(tok_per_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(elapsed / K * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 x fp8_e4m3 -> fp32 acc (linears), bf16 (KV cache, activations)",
+        "data": "synthetic: random token ids, random-init weights of the d26 architecture (seed 2)",
+        "config": {"workload": "nanochat d26 decode, batch 64, context 1792->2048, greedy, window pattern SSSL, "
+                               "Engine.generate loop (sample + GPT.forward with KV cache per step)",
+                   "batch": BATCH, "context_end": CONTEXT, "prompt_tokens": prompt_len},
+        "tpot_ms_median": round(sorted(step_times)[len(step_times) // 2] * 1e3, 4),
+        "ttft_s": round(ttft, 3),
+        "roofline": {"bound": "hbm", "kernel": "attn_partial_kernel (+combine) per layer launch",
+                     "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4), "traffic": None,
+                     "bytes_per_launch": int(att_bytes_launch), "avg_launch_us": round(att_avg_s * 1e6, 2),
+                     "launches_timed": att_n},
+        "kernel_ms_per_step": per_step_ms,
+    }
+    if not args.no_gemm:
+        result["fp8_gemm_m8192"] = gemm_rates(device)
+    del gen, engine, model
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

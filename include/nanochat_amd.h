@@ -1,0 +1,173 @@
+/* nanochat_amd -- C ABI of the MI355X (gfx950) FP8 + KV-cache decode path.
+ *
+ * Every entry point replaces one piece of the reference's hot path (citations are into the
+ * reference tree).  Conventions:
+ *   - all pointers are DEVICE pointers unless a parameter says "host";
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*); nothing synchronises;
+ *   - nothing allocates or frees device memory: callers own inputs, outputs and workspaces;
+ *   - return 0 on success, negative on error; nc_last_error() gives the message of the last
+ *     failure on the calling thread (the Python host re-raises it as AssertionError/ValueError,
+ *     which is how the reference reports the same conditions);
+ *   - bf16 tensors are raw uint16_t bit patterns, e4m3 tensors raw uint8_t (OCP e4m3fn, the
+ *     encoding of torch.float8_e4m3fn).
+ */
+#ifndef NANOCHAT_AMD_H
+#define NANOCHAT_AMD_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* nc_stream_t;
+
+int nc_abi_version(void);
+const char* nc_last_error(void);
+
+/* (1) Tensorwise dynamic quantization: nanochat/fp8.py:81-107 (_to_fp8).
+ * x_dtype: 0 = bf16, 1 = fp32.  Writes n payload bytes, *inv_scale_out (= 1/scale, what
+ * torch._scaled_mm takes) and, if not NULL, *scale_out.  amax_ws: one uint32 of scratch that
+ * the call clears itself.  encoder: 0 = hardware convert, 1 = integer software encoder. */
+int nc_fp8_quantize_tensorwise(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out,
+                               float* inv_scale_out, uint32_t* amax_ws, int encoder, nc_stream_t stream);
+
+/* Encoder only, with a caller-given scale (no amax pass); x is bf16.  For exhaustive checks of
+ * the cast at nanochat/fp8.py:101-103. */
+int nc_e4m3_encode_with_scale(const uint16_t* x, int64_t n, float scale, uint8_t* out, int encoder,
+                              nc_stream_t stream);
+
+/* (2) FP8 scaled GEMM: torch._scaled_mm as called at nanochat/fp8.py:143-153.
+ * out[M,N] = bf16((a[M,K] . b[N,K]^T, fp32 accumulate) * *inv_a * inv_b[seg(n)]).
+ * b may stack up to 4 weight matrices along N; seg_ends (HOST array of nseg exclusive column ends)
+ * says where each one stops and inv_b holds one inverse scale per segment.
+ * out_kind 0: bf16 out with leading dimension ldc.  out_kind 1: fp32 out of
+ * softcap*tanh(bf16(v)/softcap), i.e. lm_head followed by nanochat/gpt.py:512-515.
+ * kernel: 0 auto, 1 skinny (M<=128), 2/3/4 tile 256x256 / 256x128 / 128x128. */
+int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b,
+                   const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap, int M, int N,
+                   int K, int ldc, int kernel, nc_stream_t stream);
+
+/* (4a) Parameter-free RMSNorm over the last dimension: nanochat/gpt.py:42-43.  If amax_ws is not
+ * NULL the kernel also atomically max-reduces |out| into it (fp32 bits; caller clears it). */
+int nc_rmsnorm(const uint16_t* x, uint16_t* out, int rows, int cols, uint32_t* amax_ws, nc_stream_t stream);
+
+/* (4b) Embedding gather + norm + smear: nanochat/gpt.py:471-492.  idx [B,T] int64; wte bf16
+ * [vocab_rows,E]; smear_w fp32 [24]; smear_lambda fp32 [1]; prev_in bf16 [B,E] or NULL (the
+ * KVCache.prev_embedding of the previous call); prev_out bf16 [B,E]; x_out bf16 [B*T,E]. */
+int nc_embed_norm_smear(const int64_t* idx, const uint16_t* wte, const float* smear_w, const float* smear_lambda,
+                        const uint16_t* prev_in, uint16_t* prev_out, uint16_t* x_out, int B, int T, int E,
+                        int vocab_rows, nc_stream_t stream);
+
+/* (4c) Residual add, per-layer lambda mix or backout, RMSNorm: nanochat/gpt.py:500, 151-152, 503-508.
+ *   x1 = x (+ add);  backout_save <- x1 (if not NULL);
+ *   x2 = rl*x1 + xl*x0 (if resid_lambda)  |  x1 - bl*backout_src (if backout_lambda)  |  x1;
+ *   x <- x2 (in place);  xn_out <- rms_norm(x2);  amax_ws <- max|xn_out| (if not NULL). */
+int nc_mix_norm(uint16_t* x, const uint16_t* add, const uint16_t* x0, const float* resid_lambda,
+                const float* x0_lambda, const float* backout_lambda, const uint16_t* backout_src,
+                uint16_t* backout_save, uint16_t* xn_out, int rows, int cols, uint32_t* amax_ws,
+                nc_stream_t stream);
+
+/* relu(h)^2 elementwise in bf16 (+ amax): nanochat/gpt.py:139. */
+int nc_relu2(const uint16_t* h, uint16_t* out, int64_t n, uint32_t* amax_ws, nc_stream_t stream);
+
+/* (4d) Rotary + QK-norm + 1.2 gain on q and k, value-embedding gate on v, and the in-place KV-cache
+ * append: nanochat/gpt.py:89-104 and nanochat/flash_attention.py:167-170.  head_dim is 128.
+ * qkv bf16 [B*T, ld_qkv] = q heads | k heads | v heads; xn bf16 [B*T, ld_xn] (gate input, first 12
+ * channels); ve_table bf16 [vocab_rows, Hkv*128] or NULL; ve_gate_w fp32 [Hkv,12]; cos/sin bf16
+ * [rope_len,64]; cache_seqlens int32 [B] = tokens in the cache BEFORE this call; k_cache/v_cache
+ * bf16 [B,Tmax,Hkv,128] of this layer; q_out bf16 [B*T,H,128].  Token t of row b goes to slot
+ * cache_seqlens[b]+t; slots outside [0,Tmax) are skipped. */
+int nc_qkv_rope_append(const uint16_t* qkv, int ld_qkv, const uint16_t* xn, int ld_xn, const int64_t* idx,
+                       const uint16_t* ve_table, const float* ve_gate_w, const uint16_t* cos, const uint16_t* sin,
+                       int rope_len, const int32_t* cache_seqlens, uint16_t* k_cache, uint16_t* v_cache,
+                       uint16_t* q_out, int B, int T, int H, int Hkv, int Tmax, int vocab_rows, nc_stream_t stream);
+
+/* (3) Attention of T new tokens per row over the KV cache (decode: T = 1): flash_attn_with_kvcache
+ * as called at nanochat/gpt.py:113-120 (nanochat/flash_attention.py:139-185), after the append.
+ * q bf16 [B*T,H,128]; caches bf16 [B,Tmax,Hkv,128]; out bf16 [B*T,H,128].
+ * Query t of row b sees keys [max(0,p-window_left), p], p = cache_seqlens[b] + t (window_left < 0:
+ * unlimited).  seqlens_include_new: set to 1 if cache_seqlens was already advanced by T.
+ * splits: 0 = choose; workspace must hold nc_attention_workspace_bytes() when more than one split
+ * is used.  amax_ws as above (or NULL). */
+size_t nc_attention_workspace_bytes(int B, int T, int H, int Tmax);
+int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                        const int32_t* cache_seqlens, int window_left, uint16_t* out, int B, int T, int H, int Hkv,
+                        int Tmax, int seqlens_include_new, void* workspace, size_t workspace_bytes,
+                        uint32_t* amax_ws, int splits, nc_stream_t stream);
+
+/* (5) softcap * tanh(bf16 logits / softcap) -> fp32: nanochat/gpt.py:511-515. */
+int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_stream_t stream);
+
+/* (5) Next-token selection: nanochat/engine.py:140-156.  logits fp32 [B,ld]; temperature 0 =>
+ * argmax (first index on ties).  Otherwise noise holds Exp(1) draws, [B,k] with top-k (k =
+ * min(top_k,V) <= 256; rank j of the descending top-k list uses noise[b,j]) or [B,V] without
+ * (top_k <= 0), and the draw is argmax_j softmax_j / noise_j, which is what torch.multinomial
+ * computes.  out_ids int64 [B]. */
+int nc_sample(const float* logits, int B, int V, int ld, float temperature, int top_k, const float* noise,
+              int64_t* out_ids, nc_stream_t stream);
+
+/* ---- the whole GPT.forward(idx, kv_cache=...) : nanochat/gpt.py:459-524 --------------------- */
+typedef struct nc_layer_desc {
+    const uint8_t* w_qkv;        /* e4m3 [(H+2Hkv)*128, E]: c_q | c_k | c_v rows (gpt.py:77-79) */
+    const float* inv_qkv;        /* fp32 [3]: one inverse scale per stacked weight */
+    const uint8_t* w_attn_proj;  /* e4m3 [E, H*128]        (gpt.py:80)  */
+    const float* inv_attn_proj;  /* fp32 [1] */
+    const uint8_t* w_fc;         /* e4m3 [4E, E]           (gpt.py:134) */
+    const float* inv_fc;
+    const uint8_t* w_mlp_proj;   /* e4m3 [E, 4E]           (gpt.py:135) */
+    const float* inv_mlp_proj;
+    const uint16_t* ve_table;    /* bf16 [padded_vocab, Hkv*128] or NULL (gpt.py:192) */
+    const float* ve_gate_w;      /* fp32 [Hkv,12] or NULL  (gpt.py:82)  */
+    int window_left;             /* gpt.py:287-314 */
+    int reserved;
+} nc_layer_desc;
+
+typedef struct nc_model_desc {
+    int n_layer, n_head, n_kv_head, n_embd, vocab_size, padded_vocab, rope_len, reserved;
+    float softcap;
+    float reserved_f;
+    const uint16_t* wte;         /* bf16 [padded_vocab, E] */
+    const uint8_t* w_lm_head;    /* e4m3 [padded_vocab, E] */
+    const float* inv_lm_head;    /* fp32 [1] */
+    const float* resid_lambdas;  /* fp32 [L] */
+    const float* x0_lambdas;     /* fp32 [L] */
+    const float* smear_w;        /* fp32 [24] */
+    const float* smear_lambda;   /* fp32 [1] */
+    const float* backout_lambda; /* fp32 [1] */
+    const uint16_t* cos;         /* bf16 [rope_len, 64] */
+    const uint16_t* sin;
+    const nc_layer_desc* layers; /* HOST array of n_layer entries */
+} nc_model_desc;
+
+typedef struct nc_cache_desc {
+    uint16_t* k_cache;           /* bf16 [L, B, Tmax, Hkv, 128]  (engine.py:98-99) */
+    uint16_t* v_cache;
+    const int32_t* cache_seqlens;/* int32 [B], tokens cached before this call; the caller advances it */
+    const uint16_t* prev_in;     /* bf16 [B,E] or NULL: KVCache.prev_embedding */
+    uint16_t* prev_out;          /* bf16 [B,E]: the value to keep for the next call */
+    int batch, max_seq_len;
+} nc_cache_desc;
+
+size_t nc_gpt_workspace_bytes(const nc_model_desc* model /*host*/, int B, int T);
+
+/* idx int64 [B,T]; logits_out fp32 [B*T, vocab_size] (all positions) or, with last_only = 1,
+ * [B, vocab_size] (the last position of every row, which is all Engine.generate reads).
+ * workspace: nc_gpt_workspace_bytes() bytes, 256-byte aligned.  Appends K/V of the T tokens at
+ * cache_seqlens[b].. in every layer; the caller then advances cache_seqlens by T (gpt.py:122-123). */
+int nc_gpt_forward(const nc_model_desc* model /*host*/, const nc_cache_desc* cache /*host*/, const int64_t* idx,
+                   int B, int T, float* logits_out, int last_only, void* workspace, size_t workspace_bytes,
+                   nc_stream_t stream);
+
+/* ---- measurement aid (no counterpart in the reference) --------------------------------------
+ * While enabled, every launch made by this library is bracketed by a HIP event pair on its stream.
+ * Classes: 0 attention (partial + combine), 1 FP8 GEMM, 2 quantize/convert, 3 row kernels, 4 sampler.
+ * `units` are the algorithmic bytes (classes 0,2,3,4) or flops (class 1) of the launches.  Not thread
+ * safe; at most 16384 launches are recorded per enable. */
+int nc_profile_enable(int on);
+int nc_profile_read(int cls, double* total_ms /*host*/, double* total_units /*host*/, int64_t* count /*host*/);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

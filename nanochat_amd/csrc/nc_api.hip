@@ -1,0 +1,97 @@
+// extern "C" surface of libnanochat_amd.so: argument validation, the thread-local error message and
+// thin forwarding into the launch functions.  Declarations and reference citations: include/nanochat_amd.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include "../../include/nanochat_amd.h"
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+static thread_local char g_error[512] = "";
+
+void nc_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" {
+
+int nc_abi_version(void) { return 1; }
+const char* nc_last_error(void) { return g_error; }
+
+int nc_fp8_quantize_tensorwise(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_scale_out,
+                               uint32_t* amax_ws, int encoder, nc_stream_t stream) {
+    NC_CHECK_ARG(encoder == 0 || encoder == 1, "fp8_quantize: encoder must be 0 (hardware) or 1 (software)");
+    return nc_launch_quantize(x, x_dtype, n, out, scale_out, inv_scale_out, amax_ws, encoder, (hipStream_t)stream);
+}
+
+int nc_e4m3_encode_with_scale(const uint16_t* x, int64_t n, float scale, uint8_t* out, int encoder, nc_stream_t stream) {
+    NC_CHECK_ARG(encoder == 0 || encoder == 1, "e4m3_encode: encoder must be 0 (hardware) or 1 (software)");
+    return nc_launch_encode_with_scale(x, n, scale, out, encoder, (hipStream_t)stream);
+}
+
+int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, const int32_t* seg_ends, int nseg,
+                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int kernel, nc_stream_t stream) {
+    NcGemmSegs segs{1, {N, 0, 0, 0}};
+    if (seg_ends) {
+        NC_CHECK_ARG(nseg >= 1 && nseg <= 4, "fp8_gemm: 1..4 column segments supported, got %d", nseg);
+        segs.nseg = nseg;
+        for (int i = 0; i < nseg; i++) segs.end[i] = seg_ends[i];
+    }
+    return nc_launch_gemm(a, b, inv_a, inv_b, segs, out, out_kind, softcap, M, N, K, ldc, kernel, (hipStream_t)stream);
+}
+
+int nc_rmsnorm(const uint16_t* x, uint16_t* out, int rows, int cols, uint32_t* amax_ws, nc_stream_t stream) {
+    return nc_launch_rmsnorm(x, out, rows, cols, amax_ws, (hipStream_t)stream);
+}
+
+int nc_embed_norm_smear(const int64_t* idx, const uint16_t* wte, const float* smear_w, const float* smear_lambda,
+                        const uint16_t* prev_in, uint16_t* prev_out, uint16_t* x_out, int B, int T, int E, int vocab_rows,
+                        nc_stream_t stream) {
+    return nc_launch_embed_norm_smear(idx, wte, smear_w, smear_lambda, prev_in, prev_out, x_out, B, T, E, vocab_rows,
+                                      (hipStream_t)stream);
+}
+
+int nc_mix_norm(uint16_t* x, const uint16_t* add, const uint16_t* x0, const float* resid_lambda, const float* x0_lambda,
+                const float* backout_lambda, const uint16_t* backout_src, uint16_t* backout_save, uint16_t* xn_out, int rows,
+                int cols, uint32_t* amax_ws, nc_stream_t stream) {
+    return nc_launch_mix_norm(x, add, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, rows, cols,
+                              amax_ws, (hipStream_t)stream);
+}
+
+int nc_relu2(const uint16_t* h, uint16_t* out, int64_t n, uint32_t* amax_ws, nc_stream_t stream) {
+    return nc_launch_relu2(h, out, n, amax_ws, (hipStream_t)stream);
+}
+
+int nc_qkv_rope_append(const uint16_t* qkv, int ld_qkv, const uint16_t* xn, int ld_xn, const int64_t* idx, const uint16_t* ve_table,
+                       const float* ve_gate_w, const uint16_t* cos, const uint16_t* sin, int rope_len, const int32_t* cache_seqlens,
+                       uint16_t* k_cache, uint16_t* v_cache, uint16_t* q_out, int B, int T, int H, int Hkv, int Tmax, int vocab_rows,
+                       nc_stream_t stream) {
+    return nc_launch_qkv_rope_append(qkv, ld_qkv, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin, rope_len, cache_seqlens, k_cache,
+                                     v_cache, q_out, B, T, H, Hkv, Tmax, vocab_rows, (hipStream_t)stream);
+}
+
+size_t nc_attention_workspace_bytes(int B, int T, int H, int Tmax) {
+    (void)Tmax;
+    if (B <= 0 || T <= 0 || H <= 0) return 0;
+    return nc_attn_ws_bytes(B, T, H);
+}
+
+int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int32_t* cache_seqlens,
+                        int window_left, uint16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
+                        void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits, nc_stream_t stream) {
+    return nc_launch_attention(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new,
+                               workspace, workspace_bytes, amax_ws, splits, (hipStream_t)stream);
+}
+
+int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_stream_t stream) {
+    return nc_launch_softcap(raw, out, n, softcap, (hipStream_t)stream);
+}
+
+int nc_sample(const float* logits, int B, int V, int ld, float temperature, int top_k, const float* noise, int64_t* out_ids,
+              nc_stream_t stream) {
+    return nc_launch_sample(logits, B, V, ld, temperature, top_k, noise, out_ids, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,268 @@
+// Split-K attention over the KV cache for newly appended tokens (decode: one token per row).
+// Replaces flash_attn_with_kvcache as called at nanochat/gpt.py:113-120 (FA3 signature,
+// nanochat/flash_attention.py:139-161): causal, left sliding window of w keys (w+1 keys visible,
+// flash_attention.py:91-97), GQA with q head h reading kv head h / (H/Hkv), per-row cache lengths.
+// The cache append itself is done by the rotary kernel that runs just before this one.
+//
+// Layout: q [B*T, H, 128] bf16; k_cache, v_cache [B, Tmax, Hkv, 128] bf16 (one layer).
+// A key is 256 contiguous bytes; consecutive keys of one head are Hkv*256 bytes apart.
+//
+// Mapping: a wave owns a contiguous run of keys of one (row, kv head).  16 lanes share one key, 16 bytes
+// (8 dims) each, so one 64-lane load instruction fetches four whole keys as four 256-byte segments.  The
+// 16-lane dot product is finished with DPP row rotations; each 16-lane group runs its own online softmax
+// over the keys it sees (no cross-lane traffic in the loop), and the four groups, then the four waves of
+// the workgroup, then the splits, are merged with the usual (max, sum, acc) rescale.  All G = H/Hkv
+// query heads that share the kv head are processed by the same wave so K and V are read exactly once.
+//
+// HBM traffic per (row, kv head): 2 * n_keys * 256 bytes, the algorithmic minimum.
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+#define NEG_BIG (-1.0e30f)
+#define PART_STRIDE 132     // floats per partial: m, l, pad, pad, acc[128]
+
+template <int G>
+__global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+                                                           const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
+                                                           int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
+                                                           float* __restrict__ partials, uint32_t* __restrict__ amax_ws, int T, int H,
+                                                           int Hkv, int Tmax, int nsplit) {
+    __shared__ float merge[4][G][PART_STRIDE];
+    const int split = blockIdx.x, hk = blockIdx.y, row = blockIdx.z;
+    const int b = row / T, t = row % T;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int grp = lane >> 4, sub = lane & 15;
+
+    // visible keys [lo, hi]
+    int pos = cache_seqlens[b];
+    if (seqlens_include_new) pos -= T;
+    int hi = pos + t;
+    if (hi > Tmax - 1) hi = Tmax - 1;
+    int lo = (window_left < 0) ? 0 : hi - window_left;
+    if (lo < 0) lo = 0;
+    const int n_keys = hi - lo + 1;
+    // contiguous runs, multiples of 4 keys, over nsplit * 4 waves
+    const int nw = nsplit * 4;
+    int chunk = (n_keys + nw - 1) / nw;
+    chunk = (chunk + 3) & ~3;
+    const int gw = split * 4 + wave;
+    const int k_begin = lo + gw * chunk;
+    int k_end = k_begin + chunk;
+    if (k_end > hi + 1) k_end = hi + 1;
+
+    // q for the G heads of this kv head, pre-scaled by log2(e) / sqrt(128)
+    const float qscale = 1.4426950408889634f * 0.08838834764831845f;
+    float qf[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const uint4 qv = *(const uint4*)(q + ((size_t)row * H + hk * G + g) * 128 + sub * 8);
+        const uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            qf[g][2 * j] = bf16_lo(w[j]) * qscale;
+            qf[g][2 * j + 1] = bf16_hi(w[j]) * qscale;
+        }
+    }
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        m[g] = NEG_BIG, l[g] = 0.f;
+#pragma unroll
+        for (int d = 0; d < 8; d++) acc[g][d] = 0.f;
+    }
+
+    const size_t key_stride = (size_t)Hkv * 128;   // elements between consecutive keys
+    const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
+    const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
+
+    constexpr int UNROLL = 8;     // 8 loads x 4 keys = 32 keys (8 KB of K and 8 KB of V) in flight per wave
+    for (int kb0 = k_begin; kb0 < k_end; kb0 += 4 * UNROLL) {
+        uint4 kr[UNROLL], vr[UNROLL];
+        bool ok[UNROLL];
+#pragma unroll
+        for (int i = 0; i < UNROLL; i++) {
+            const int j = kb0 + 4 * i + grp;
+            ok[i] = j < k_end;
+            kr[i] = ok[i] ? *(const uint4*)(kbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < UNROLL; i++) {
+            const int j = kb0 + 4 * i + grp;
+            vr[i] = ok[i] ? *(const uint4*)(vbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
+        }
+        float sc[G][UNROLL];
+#pragma unroll
+        for (int i = 0; i < UNROLL; i++) {
+            const uint32_t w[4] = {kr[i].x, kr[i].y, kr[i].z, kr[i].w};
+            float kf[8];
+#pragma unroll
+            for (int j = 0; j < 4; j++) kf[2 * j] = bf16_lo(w[j]), kf[2 * j + 1] = bf16_hi(w[j]);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                float d = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) d = fmaf(qf[g][e], kf[e], d);
+                d = row16_sum(d);
+                sc[g][i] = ok[i] ? d : NEG_BIG;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float mn = m[g];
+#pragma unroll
+            for (int i = 0; i < UNROLL; i++) mn = fmaxf(mn, sc[g][i]);
+            const float corr = exp2f(m[g] - mn);
+            m[g] = mn;
+            l[g] *= corr;
+#pragma unroll
+            for (int d = 0; d < 8; d++) acc[g][d] *= corr;
+#pragma unroll
+            for (int i = 0; i < UNROLL; i++) sc[g][i] = ok[i] ? exp2f(sc[g][i] - mn) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < UNROLL; i++) {
+            const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+            float vf[8];
+#pragma unroll
+            for (int j = 0; j < 4; j++) vf[2 * j] = bf16_lo(w[j]), vf[2 * j + 1] = bf16_hi(w[j]);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                l[g] += sc[g][i];
+#pragma unroll
+                for (int d = 0; d < 8; d++) acc[g][d] = fmaf(sc[g][i], vf[d], acc[g][d]);
+            }
+        }
+    }
+
+    // merge the four 16-lane groups of the wave
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        float mm = fmaxf(m[g], __shfl_xor(m[g], 16));
+        mm = fmaxf(mm, __shfl_xor(mm, 32));
+        const float w = exp2f(m[g] - mm);
+        float lw = l[g] * w;
+        lw += __shfl_xor(lw, 16);
+        lw += __shfl_xor(lw, 32);
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            float a = acc[g][d] * w;
+            a += __shfl_xor(a, 16);
+            a += __shfl_xor(a, 32);
+            acc[g][d] = a;
+        }
+        m[g] = mm, l[g] = lw;
+        if (grp == 0) {
+            if (sub == 0) merge[wave][g][0] = mm, merge[wave][g][1] = lw;
+#pragma unroll
+            for (int d = 0; d < 8; d++) merge[wave][g][4 + sub * 8 + d] = acc[g][d];
+        }
+    }
+    __syncthreads();
+
+    // merge the four waves: thread (g, d) for d < 128
+    float am = 0.f;
+    for (int item = threadIdx.x; item < G * 128; item += 256) {
+        const int g = item >> 7, d = item & 127;
+        float mm = NEG_BIG;
+#pragma unroll
+        for (int w = 0; w < 4; w++) mm = fmaxf(mm, merge[w][g][0]);
+        float ls = 0.f, a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float sc = exp2f(merge[w][g][0] - mm);
+            ls += merge[w][g][1] * sc;
+            a += merge[w][g][4 + d] * sc;
+        }
+        const int head = hk * G + g;
+        if (nsplit == 1) {
+            const bf16_t o = f32_to_bf16(a / ls);
+            out[((size_t)row * H + head) * 128 + d] = o;
+            am = fmaxf(am, fabsf(bf16_to_f32(o)));
+        } else {
+            float* p = partials + (((size_t)row * H + head) * nsplit + split) * PART_STRIDE;
+            if (d == 0) p[0] = mm, p[1] = ls;
+            p[4 + d] = a;
+        }
+    }
+    if (nsplit == 1 && amax_ws) {
+        am = wave_max(am);
+        if (lane == 0 && am > 0.f) atomicMax(amax_ws, __float_as_uint(am));
+    }
+}
+
+// one wave per (row, head): merge nsplit partials, write bf16
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ partials, bf16_t* __restrict__ out,
+                                                           uint32_t* __restrict__ amax_ws, int nsplit, int total) {
+    const int lane = threadIdx.x & 63;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= total) return;
+    const float* p = partials + (size_t)item * nsplit * PART_STRIDE;
+    float mm = NEG_BIG;
+    for (int s = 0; s < nsplit; s++) mm = fmaxf(mm, p[s * PART_STRIDE]);
+    float ls = 0.f, a0 = 0.f, a1 = 0.f;
+    for (int s = 0; s < nsplit; s++) {
+        const float sc = exp2f(p[s * PART_STRIDE] - mm);
+        ls += p[s * PART_STRIDE + 1] * sc;
+        const float2 av = *(const float2*)(p + s * PART_STRIDE + 4 + lane * 2);
+        a0 += av.x * sc;
+        a1 += av.y * sc;
+    }
+    const bf16_t o0 = f32_to_bf16(a0 / ls), o1 = f32_to_bf16(a1 / ls);
+    *(uint32_t*)(out + (size_t)item * 128 + lane * 2) = (uint32_t)o0 | ((uint32_t)o1 << 16);
+    if (amax_ws) {
+        float am = wave_max(fmaxf(fabsf(bf16_to_f32(o0)), fabsf(bf16_to_f32(o1))));
+        if (lane == 0 && am > 0.f) atomicMax(amax_ws, __float_as_uint(am));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+static int pick_splits(int B, int T, int Hkv, int max_keys) {
+    // aim for >= 8192 waves (8 per SIMD... 32 per CU) while keeping >= 128 keys per wave
+    const long base_waves = (long)B * T * Hkv * 4;
+    int s = 1;
+    while (s < 16 && base_waves * s < 8192 && max_keys / (4 * s * 2) >= 64) s *= 2;
+    return s;
+}
+
+size_t nc_attn_ws_bytes(int B, int T, int H) {
+    return (size_t)B * T * H * 16 * PART_STRIDE * sizeof(float);
+}
+
+int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
+                        int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
+                        void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int force_splits, hipStream_t s) {
+    NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
+    NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0, "decode_attention: bad shape");
+    NC_CHECK_ARG(H % Hkv == 0, "decode_attention: n_head %d not a multiple of n_kv_head %d", H, Hkv);
+    const int G = H / Hkv;
+    NC_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8, "decode_attention: query group size %d not in {1,2,4,8}", G);
+    NC_CHECK_ARG((long)B * T <= 65535 * 4L && Hkv <= 65535, "decode_attention: grid too large");
+    NC_CHECK_ARG(((uintptr_t)q & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0,
+                 "decode_attention: pointers must be 16-byte aligned");
+    int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
+    int nsplit = force_splits > 0 ? force_splits : pick_splits(B, T, Hkv, max_keys);
+    NC_CHECK_ARG(nsplit >= 1 && nsplit <= 16, "decode_attention: splits must be 1..16");
+    if (nsplit > 1) {
+        const size_t need = (size_t)B * T * H * nsplit * PART_STRIDE * sizeof(float);
+        NC_CHECK_ARG(workspace && workspace_bytes >= need, "decode_attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    }
+    float* parts = (float*)workspace;
+    NcProfScope prof(0, 0.0, s);
+    dim3 grid(nsplit, Hkv, B * T), block(256);
+    NC_CHECK_ARG(B * T <= 65535, "decode_attention: more than 65535 query rows in one launch");
+#define LAUNCH_G(GG)                                                                                                         \
+    hipLaunchKernelGGL(attn_partial_kernel<GG>, grid, block, 0, s, q, k_cache, v_cache, cache_seqlens, window_left,             \
+                       seqlens_include_new, out, parts, amax_ws, T, H, Hkv, Tmax, nsplit)
+    if (G == 1) LAUNCH_G(1);
+    else if (G == 2) LAUNCH_G(2);
+    else if (G == 4) LAUNCH_G(4);
+    else LAUNCH_G(8);
+#undef LAUNCH_G
+    NC_CHECK_LAUNCH("decode_attention");
+    if (nsplit > 1) {
+        const int total = B * T * H;
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((total + 3) / 4), dim3(256), 0, s, parts, out, amax_ws, nsplit, total);
+        NC_CHECK_LAUNCH("decode_attention_combine");
+    }
+    return 0;
+}

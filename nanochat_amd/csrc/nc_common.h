@@ -1,0 +1,131 @@
+// Shared device/host helpers for the gfx950 kernels: bf16 and e4m3 conversion, wave64
+// reductions over DPP, and the error channel of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define NC_WAVE 64
+
+typedef uint16_t bf16_t;   // raw bfloat16 bits
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------- error channel (host)
+void nc_set_error(const char* fmt, ...);
+#define NC_FAIL(code, ...)        \
+    do {                          \
+        nc_set_error(__VA_ARGS__); \
+        return (code);            \
+    } while (0)
+#define NC_CHECK_ARG(cond, ...)            \
+    do {                                   \
+        if (!(cond)) NC_FAIL(-1, __VA_ARGS__); \
+    } while (0)
+#define NC_CHECK_LAUNCH(name)                                                        \
+    do {                                                                             \
+        hipError_t e__ = hipGetLastError();                                          \
+        if (e__ != hipSuccess) NC_FAIL(-2, "%s: launch failed: %s", name, hipGetErrorString(e__)); \
+    } while (0)
+
+// ---------------------------------------------------------------- bf16
+__device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+
+// round-to-nearest-even fp32 -> bf16 (NaN kept quiet)
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+// value of f after rounding to bf16, as fp32 (one rounding site of a bf16 eager op)
+__device__ __forceinline__ float rbf(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// ---------------------------------------------------------------- e4m3fn (OCP) encode
+// |y| must already be clamped to <= 448.  Round to nearest even, subnormals down to 2^-9.
+__device__ __forceinline__ uint32_t e4m3_encode_sw(float y) {
+    uint32_t u = __float_as_uint(y);
+    uint32_t sign = (u >> 24) & 0x80u;
+    u &= 0x7fffffffu;
+    uint32_t out;
+    if (u >= 0x3c800000u) {                      // >= 2^-6: normal in e4m3
+        u += 0x7ffffu + ((u >> 20) & 1u);        // RNE at mantissa bit 20
+        out = (u >> 20) - ((127u - 7u) << 3);
+    } else {                                     // subnormal: multiples of 2^-9
+        float m = __uint_as_float(u) * 512.0f;   // exact
+        out = (uint32_t)__builtin_rintf(m);      // 0..8, ties to even; 8 == 0x08 == 2^-6
+    }
+    return sign | out;
+}
+
+// four fp32 (already scaled and clamped) -> four packed e4m3 bytes, hardware convert
+__device__ __forceinline__ uint32_t e4m3_pack4_hw(float a, float b, float c, float d) {
+    int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+    return (uint32_t)r;
+}
+__device__ __forceinline__ uint32_t e4m3_pack4_sw(float a, float b, float c, float d) {
+    return e4m3_encode_sw(a) | (e4m3_encode_sw(b) << 8) | (e4m3_encode_sw(c) << 16) | (e4m3_encode_sw(d) << 24);
+}
+__device__ __forceinline__ float clamp448(float y) { return fminf(fmaxf(y, -448.0f), 448.0f); }
+
+// scale = fp32(448 / max(fp64(amax), 1e-12)) -- the divide is done in fp64 like the reference
+__device__ __forceinline__ float scale_from_amax(float amax) {
+    double d = (double)amax;
+    if (d < 1e-12) d = 1e-12;
+    return (float)(448.0 / d);
+}
+
+// ---------------------------------------------------------------- wave64 reductions
+// DPP row_ror within rows of 16 lanes: all 16 lanes end with the row total.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f32<0x128>(v);   // row_ror:8
+    v += dpp_f32<0x124>(v);   // row_ror:4
+    v += dpp_f32<0x122>(v);   // row_ror:2
+    v += dpp_f32<0x121>(v);   // row_ror:1
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        uint32_t t = (uint32_t)__shfl_xor((int)v, o);
+        v = v > t ? v : t;
+    }
+    return v;
+}
+
+// block-wide sum for blockDim.x == 64 * NW, result broadcast to every thread
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red /* >= NW floats of LDS */) {
+    v = wave_sum(v);
+    if (NW == 1) return v;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; i++) t += red[i];
+    return t;
+}

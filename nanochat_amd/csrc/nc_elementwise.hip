@@ -1,0 +1,297 @@
+// Row kernels of the decode step: embedding + norm + smear, residual mix + RMSNorm, relu^2, and the
+// fused rotary / QK-norm / value-embedding gate / KV-cache append.
+//
+// The reference runs these as separate eager bf16 ops (nanochat/gpt.py:42-43, 57-65, 94-104, 471-508),
+// each of which rounds its result to bf16.  The kernels keep values in fp32 registers but apply rbf()
+// (round to bf16) at every point where the eager graph materialises a bf16 tensor, so results agree
+// with the eager sequence instead of with an idealised fused formula.
+//
+// All of them are HBM/L2-bandwidth bound with tiny footprints at decode (a few hundred KB); the point
+// of fusing is launch count, and producing the amax of the normalised row for the FP8 quantizer that
+// follows (atomicMax on the fp32 bit pattern, valid because the values are non-negative).
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+#define RMS_EPS 1.1920928955078125e-07f   // fp32 machine epsilon: F.rms_norm's default eps
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ void block_amax_commit(float local_abs_max, uint32_t* amax_ws, float* red) {
+    if (!amax_ws) return;
+    float m = wave_max(local_abs_max);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[w] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < nw; i++) m = fmaxf(m, red[i]);
+        atomicMax(amax_ws, __float_as_uint(m));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// x_out[b,t] = smear(norm(wte[idx[b,t]])), prev_out[b] = norm(wte[idx[b,T-1]])      (gpt.py:471-492)
+// One block of 256 threads per token.  Row buffers live in LDS (fp32), cols <= 8192.
+__global__ __launch_bounds__(256) void embed_norm_smear_kernel(const int64_t* __restrict__ idx, const bf16_t* __restrict__ wte,
+                                                               const float* __restrict__ smear_w, const float* __restrict__ smear_lambda,
+                                                               const bf16_t* __restrict__ prev_in, bf16_t* __restrict__ prev_out,
+                                                               bf16_t* __restrict__ x_out, int T, int E, int vocab_rows) {
+    extern __shared__ float rowbuf[];          // [2][E]: this token, previous token (both normalised, bf16 values)
+    __shared__ float red[8];
+    const int row = blockIdx.x, b = row / T, t = row % T;
+    const bool use_prev_token = (T > 1 && t >= 1);
+    const bool use_prev_cache = (T == 1 && prev_in != nullptr);
+
+    for (int which = 0; which < (use_prev_token ? 2 : 1); which++) {
+        int64_t tok = idx[(size_t)b * T + t - which];
+        if (tok < 0 || tok >= vocab_rows) tok = 0;       // host validates; never read out of bounds
+        const bf16_t* e = wte + (size_t)tok * E;
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < E; c += 256) {
+            float v = bf16_to_f32(e[c]);
+            rowbuf[which * E + c] = v;
+            ss += v * v;
+        }
+        ss = block_sum<4>(ss, red);
+        const float rstd = 1.0f / sqrtf(ss / (float)E + RMS_EPS);
+        for (int c = threadIdx.x; c < E; c += 256) rowbuf[which * E + c] = rbf(rowbuf[which * E + c] * rstd);
+        __syncthreads();
+    }
+    if (t == T - 1)
+        for (int c = threadIdx.x; c < E; c += 256) prev_out[(size_t)b * E + c] = f32_to_bf16(rowbuf[c]);
+
+    float gate = 0.f;
+    if (use_prev_token || use_prev_cache) {
+        // gate = bf16(lambda) * sigmoid(W_s . x[:24]); every product of the chain is a bf16 tensor in eager mode
+        float dot = 0.f;
+        for (int c = 0; c < 24; c++) dot += rowbuf[c] * rbf(smear_w[c]);
+        gate = rbf(rbf(*smear_lambda) * rbf(sigmoidf_(rbf(dot))));
+    }
+    for (int c = threadIdx.x; c < E; c += 256) {
+        float v = rowbuf[c];
+        if (use_prev_token) v = rbf(v + rbf(gate * rowbuf[E + c]));
+        else if (use_prev_cache) v = rbf(v + rbf(gate * bf16_to_f32(prev_in[(size_t)b * E + c])));
+        x_out[(size_t)row * E + c] = f32_to_bf16(v);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// x1 = x (+ add);  [backout_save = x1];  x2 = rl*x1 + xl*x0  |  x1 - bl*backout_src  |  x1;
+// x = x2;  xn = rms_norm(x2);  amax(xn).                                    (gpt.py:500, 151-152, 503-508)
+__global__ __launch_bounds__(256) void mix_norm_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ add, const bf16_t* __restrict__ x0,
+                                                       const float* __restrict__ resid_lambda, const float* __restrict__ x0_lambda,
+                                                       const float* __restrict__ backout_lambda, const bf16_t* __restrict__ backout_src,
+                                                       bf16_t* __restrict__ backout_save, bf16_t* __restrict__ xn_out, int cols,
+                                                       uint32_t* __restrict__ amax_ws) {
+    extern __shared__ float rowbuf[];
+    __shared__ float red[8];
+    const size_t base = (size_t)blockIdx.x * cols;
+    const float rl = resid_lambda ? rbf(*resid_lambda) : 0.f;
+    const float xl = x0_lambda ? rbf(*x0_lambda) : 0.f;
+    const float bl = backout_lambda ? rbf(*backout_lambda) : 0.f;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float v = bf16_to_f32(x[base + c]);
+        if (add) v = rbf(v + bf16_to_f32(add[base + c]));
+        if (backout_save) backout_save[base + c] = f32_to_bf16(v);
+        if (resid_lambda) v = rbf(rbf(rl * v) + rbf(xl * bf16_to_f32(x0[base + c])));
+        else if (backout_lambda) v = rbf(v - rbf(bl * bf16_to_f32(backout_src[base + c])));
+        if (add || resid_lambda || backout_lambda) x[base + c] = f32_to_bf16(v);
+        rowbuf[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum<4>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)cols + RMS_EPS);
+    float am = 0.f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        const bf16_t o = f32_to_bf16(rowbuf[c] * rstd);
+        xn_out[base + c] = o;
+        am = fmaxf(am, fabsf(bf16_to_f32(o)));
+    }
+    block_amax_commit(am, amax_ws, red);
+}
+
+// out = rms_norm(x) over the last dim, rows independent (gpt.py:42-43)
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out, int cols,
+                                                      uint32_t* __restrict__ amax_ws) {
+    extern __shared__ float rowbuf[];
+    __shared__ float red[8];
+    const size_t base = (size_t)blockIdx.x * cols;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float v = bf16_to_f32(x[base + c]);
+        rowbuf[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum<4>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)cols + RMS_EPS);
+    float am = 0.f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        const bf16_t o = f32_to_bf16(rowbuf[c] * rstd);
+        out[base + c] = o;
+        am = fmaxf(am, fabsf(bf16_to_f32(o)));
+    }
+    block_amax_commit(am, amax_ws, red);
+}
+
+// out = relu(h)^2, elementwise bf16, plus amax (gpt.py:139)
+__global__ __launch_bounds__(256) void relu2_kernel(const bf16_t* __restrict__ h, bf16_t* __restrict__ out, int64_t n,
+                                                    uint32_t* __restrict__ amax_ws) {
+    __shared__ float red[8];
+    float am = 0.f;
+    const int64_t nvec = n / 8;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * blockDim.x) {
+        uint4 v = ((const uint4*)h)[i];
+        uint32_t w[4] = {v.x, v.y, v.z, v.w}, o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float a = fmaxf(bf16_lo(w[j]), 0.f), b = fmaxf(bf16_hi(w[j]), 0.f);
+            a = rbf(a * a), b = rbf(b * b);
+            am = fmaxf(am, fmaxf(a, b));
+            o[j] = pack_bf16(a, b);
+        }
+        ((uint4*)out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    if (blockIdx.x == 0)
+        for (int64_t i = nvec * 8 + threadIdx.x; i < n; i += blockDim.x) {
+            float a = fmaxf(bf16_to_f32(h[i]), 0.f);
+            a = rbf(a * a);
+            am = fmaxf(am, a);
+            out[i] = f32_to_bf16(a);
+        }
+    block_amax_commit(am, amax_ws, red);
+}
+
+// ------------------------------------------------------------------------------------------------
+// One wave per (token, head) of the fused q|k|v projection output; lane l owns dims l and l+64, which
+// is exactly one rotary pair.  head_dim is fixed at 128.
+//   q heads: rotary -> rms_norm over D -> *1.2 -> q_out[token, h, :]
+//   k heads: same -> k_cache[b, pos+t, h, :]
+//   v heads: v + 3*sigmoid(W_g . xn[:12])[h] * ve[idx, h, :] (if the layer has a value embedding) -> v_cache
+// (gpt.py:89-104, flash_attention.py:167-170)
+__global__ __launch_bounds__(256) void qkv_rope_append_kernel(const bf16_t* __restrict__ qkv, int ld_qkv, const bf16_t* __restrict__ xn,
+                                                              int ld_xn, const int64_t* __restrict__ idx, const bf16_t* __restrict__ ve_table,
+                                                              const float* __restrict__ ve_gate_w, const bf16_t* __restrict__ cos_t,
+                                                              const bf16_t* __restrict__ sin_t, int rope_len,
+                                                              const int32_t* __restrict__ cache_seqlens, bf16_t* __restrict__ k_cache,
+                                                              bf16_t* __restrict__ v_cache, bf16_t* __restrict__ q_out, int T, int H,
+                                                              int Hkv, int Tmax, int vocab_rows, int total_waves) {
+    const int lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (gw >= total_waves) return;
+    const int heads = H + 2 * Hkv;
+    const int token = gw / heads, hh = gw % heads;
+    const int b = token / T, t = token % T;
+    const int pos = cache_seqlens[b] + t;
+    const bf16_t* src = qkv + (size_t)token * ld_qkv + (size_t)hh * 128;
+    float x1 = bf16_to_f32(src[lane]), x2 = bf16_to_f32(src[lane + 64]);
+    const bool in_cache = pos >= 0 && pos < Tmax;
+
+    if (hh < H + Hkv) {
+        const int rp = pos < rope_len ? (pos < 0 ? 0 : pos) : rope_len - 1;
+        const float c = bf16_to_f32(cos_t[(size_t)rp * 64 + lane]), s = bf16_to_f32(sin_t[(size_t)rp * 64 + lane]);
+        float y1 = rbf(rbf(x1 * c) + rbf(x2 * s));
+        float y2 = rbf(rbf(x1 * (-s)) + rbf(x2 * c));
+        const float ss = wave_sum(y1 * y1 + y2 * y2);
+        const float rstd = 1.0f / sqrtf(ss / 128.0f + RMS_EPS);
+        y1 = rbf(rbf(y1 * rstd) * 1.2f);
+        y2 = rbf(rbf(y2 * rstd) * 1.2f);
+        if (hh < H) {
+            bf16_t* dst = q_out + ((size_t)token * H + hh) * 128;
+            dst[lane] = f32_to_bf16(y1);
+            dst[lane + 64] = f32_to_bf16(y2);
+        } else if (in_cache) {
+            bf16_t* dst = k_cache + (((size_t)b * Tmax + pos) * Hkv + (hh - H)) * 128;
+            dst[lane] = f32_to_bf16(y1);
+            dst[lane + 64] = f32_to_bf16(y2);
+        }
+    } else {
+        const int hv = hh - H - Hkv;
+        if (ve_table) {
+            float dot = 0.f;
+            const bf16_t* xr = xn + (size_t)token * ld_xn;
+#pragma unroll
+            for (int cidx = 0; cidx < 12; cidx++) dot += bf16_to_f32(xr[cidx]) * rbf(ve_gate_w[hv * 12 + cidx]);
+            const float gate = rbf(3.0f * rbf(sigmoidf_(rbf(dot))));
+            int64_t tok = idx[token];
+            if (tok < 0 || tok >= vocab_rows) tok = 0;
+            const bf16_t* ve = ve_table + ((size_t)tok * Hkv + hv) * 128;
+            x1 = rbf(x1 + rbf(gate * bf16_to_f32(ve[lane])));
+            x2 = rbf(x2 + rbf(gate * bf16_to_f32(ve[lane + 64])));
+        }
+        if (in_cache) {
+            bf16_t* dst = v_cache + (((size_t)b * Tmax + pos) * Hkv + hv) * 128;
+            dst[lane] = f32_to_bf16(x1);
+            dst[lane + 64] = f32_to_bf16(x2);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+static bool row_args_ok(int rows, int cols) { return rows >= 0 && cols > 0 && cols <= 16384; }
+
+int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+    NC_CHECK_ARG(x && out, "rmsnorm: null pointer");
+    NC_CHECK_ARG(row_args_ok(rows, cols), "rmsnorm: bad shape rows=%d cols=%d (cols <= 16384)", rows, cols);
+    if (rows == 0) return 0;
+    NcProfScope prof(3, 4.0 * rows * cols, s);
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, out, cols, amax_ws);
+    NC_CHECK_LAUNCH("rmsnorm");
+    return 0;
+}
+
+int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const float* smear_w, const float* smear_lambda,
+                               const bf16_t* prev_in, bf16_t* prev_out, bf16_t* x_out, int B, int T, int E, int vocab_rows,
+                               hipStream_t s) {
+    NC_CHECK_ARG(idx && wte && smear_w && smear_lambda && prev_out && x_out, "embed_norm_smear: null pointer");
+    NC_CHECK_ARG(B > 0 && T > 0 && E >= 24 && E <= 8192, "embed_norm_smear: bad shape B=%d T=%d E=%d", B, T, E);
+    NcProfScope prof(3, 4.0 * B * T * E, s);
+    hipLaunchKernelGGL(embed_norm_smear_kernel, dim3(B * T), dim3(256), 2 * E * sizeof(float), s, idx, wte, smear_w, smear_lambda,
+                       prev_in, prev_out, x_out, T, E, vocab_rows);
+    NC_CHECK_LAUNCH("embed_norm_smear");
+    return 0;
+}
+
+int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
+                       const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
+                       int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+    NC_CHECK_ARG(x && xn_out, "mix_norm: null pointer");
+    NC_CHECK_ARG(row_args_ok(rows, cols), "mix_norm: bad shape rows=%d cols=%d", rows, cols);
+    NC_CHECK_ARG(!resid_lambda || (x0 && x0_lambda), "mix_norm: the residual mix needs x0 and x0_lambda");
+    NC_CHECK_ARG(!backout_lambda || backout_src, "mix_norm: backout needs its source rows");
+    NC_CHECK_ARG(!(resid_lambda && backout_lambda), "mix_norm: residual mix and backout are exclusive");
+    if (rows == 0) return 0;
+    NcProfScope prof(3, 8.0 * rows * cols, s);
+    hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, add, x0, resid_lambda, x0_lambda,
+                       backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws);
+    NC_CHECK_LAUNCH("mix_norm");
+    return 0;
+}
+
+int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, hipStream_t s) {
+    NC_CHECK_ARG(h && out && n >= 0, "relu2: bad arguments");
+    NC_CHECK_ARG(((uintptr_t)h & 15) == 0 && ((uintptr_t)out & 15) == 0, "relu2: pointers must be 16-byte aligned");
+    int64_t g = (n / 8 + 255) / 256;
+    if (g < 1) g = 1;
+    if (g > 2048) g = 2048;
+    NcProfScope prof(3, 4.0 * n, s);
+    hipLaunchKernelGGL(relu2_kernel, dim3((int)g), dim3(256), 0, s, h, out, n, amax_ws);
+    NC_CHECK_LAUNCH("relu2");
+    return 0;
+}
+
+int nc_launch_qkv_rope_append(const bf16_t* qkv, int ld_qkv, const bf16_t* xn, int ld_xn, const int64_t* idx,
+                              const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,
+                              int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,
+                              int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s) {
+    NC_CHECK_ARG(qkv && cos && sin && cache_seqlens && k_cache && v_cache && q_out, "qkv_rope_append: null pointer");
+    NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && Tmax > 0 && rope_len > 0, "qkv_rope_append: bad shape");
+    NC_CHECK_ARG(ld_qkv >= (H + 2 * Hkv) * 128, "qkv_rope_append: ld_qkv too small (head_dim is fixed at 128)");
+    NC_CHECK_ARG(!ve_table || (ve_gate_w && xn && idx && ld_xn >= 12), "qkv_rope_append: value embedding needs gate weights, xn and idx");
+    const int total = B * T * (H + 2 * Hkv);
+    NcProfScope prof(3, 4.0 * total * 128, s);
+    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, qkv, ld_qkv, xn, ld_xn, idx, ve_table, ve_gate_w,
+                       cos, sin, rope_len, cache_seqlens, k_cache, v_cache, q_out, T, H, Hkv, Tmax, vocab_rows, total);
+    NC_CHECK_LAUNCH("qkv_rope_append");
+    return 0;
+}

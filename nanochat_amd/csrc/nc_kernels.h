@@ -1,0 +1,59 @@
+// Internal launch functions shared between the C ABI (nc_api.hip) and the fused forward
+// (nc_forward.hip).  Every function enqueues work on the given stream, never synchronises,
+// never allocates, and returns 0 or a negative code after nc_set_error().
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint16_t bf16_t;
+
+// ---- quantize (nc_quantize.hip)
+void nc_clear_u32(uint32_t* p, int n, hipStream_t s);
+int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_out,
+                       uint32_t* amax_ws, int encoder, hipStream_t s);
+int nc_launch_convert_only(const void* x, int64_t n, uint8_t* out, float* inv_out, const uint32_t* amax_ws, hipStream_t s);
+int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, uint8_t* out, int encoder, hipStream_t s);
+
+// ---- GEMM (nc_gemm.hip)
+struct NcGemmSegs {      // column segments of B, each with its own weight inv-scale
+    int nseg;
+    int end[4];          // exclusive column end of each segment
+};
+// out_kind: 0 = bf16 [M,ldc];  1 = fp32 [M,ldc] of softcap*tanh(bf16(v)/softcap)
+int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
+                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, hipStream_t s);
+
+// ---- elementwise / norm / rope (nc_elementwise.hip)
+int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s);
+int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const float* smear_w, const float* smear_lambda,
+                               const bf16_t* prev_in, bf16_t* prev_out, bf16_t* x_out, int B, int T, int E, int vocab_rows,
+                               hipStream_t s);
+int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
+                       const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
+                       int rows, int cols, uint32_t* amax_ws, hipStream_t s);
+int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, hipStream_t s);
+int nc_launch_qkv_rope_append(const bf16_t* qkv, int ld_qkv, const bf16_t* xn, int ld_xn, const int64_t* idx,
+                              const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,
+                              int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,
+                              int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s);
+
+// ---- attention (nc_attention.hip)
+size_t nc_attn_ws_bytes(int B, int T, int H);
+int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
+                        int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
+                        void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int force_splits, hipStream_t s);
+
+// ---- sampling (nc_sample.hip)
+int nc_launch_softcap(const bf16_t* raw, float* out, int64_t n, float softcap, hipStream_t s);
+int nc_launch_sample(const float* logits, int B, int V, int ld, float temperature, int top_k, const float* noise,
+                     int64_t* out_ids, hipStream_t s);
+
+// ---- optional event timing (nc_profile.hip)
+int nc_prof_begin(int cls, double units, hipStream_t s);
+void nc_prof_end(int slot, hipStream_t s);
+struct NcProfScope {
+    int slot;
+    hipStream_t s;
+    NcProfScope(int cls, double units, hipStream_t st) : slot(nc_prof_begin(cls, units, st)), s(st) {}
+    ~NcProfScope() { nc_prof_end(slot, s); }
+};

@@ -1,0 +1,179 @@
+// Tensorwise dynamic e4m3 quantization: amax reduce, then scale + saturate + convert.
+// Replaces the eight eager ops of nanochat/fp8.py:91-106 (_to_fp8).
+//
+// Bit contract: amax in fp32; scale = fp32(448 / max(fp64(amax), 1e-12)); y = fp32(x) * scale
+// (one fp32 rounding); clamp to +-448; round to nearest even into OCP e4m3fn; inv = 1.0f / scale
+// with an IEEE divide.  HBM traffic: the amax pass reads the tensor once, the convert pass reads
+// it again (normally from L2 / infinity cache) and writes one byte per element.
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+// ---------------------------------------------------------------- pass 1: amax
+// bf16: |x| ordering equals integer ordering of the low 15 bits; fp32 likewise on 31 bits.
+// Each thread takes 16-byte vectors grid-stride; one atomicMax per block on the fp32 bit pattern.
+template <bool IS_BF16>
+__global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, int64_t n, uint32_t* __restrict__ amax_bits) {
+    constexpr int PER_VEC = IS_BF16 ? 8 : 4;
+    const int64_t nvec = n / PER_VEC;
+    const uint4* xv = (const uint4*)x;
+    uint32_t m = 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * blockDim.x) {
+        uint4 v = xv[i];
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (IS_BF16) {
+                uint32_t lo = (w[j] & 0x7fffu) << 16, hi = w[j] & 0x7fff0000u;
+                m = m > lo ? m : lo;
+                m = m > hi ? m : hi;
+            } else {
+                uint32_t a = w[j] & 0x7fffffffu;
+                m = m > a ? m : a;
+            }
+        }
+    }
+    // tail elements (n not a multiple of the vector width)
+    if (blockIdx.x == 0) {
+        for (int64_t i = nvec * PER_VEC + threadIdx.x; i < n; i += blockDim.x) {
+            uint32_t a = IS_BF16 ? (((uint32_t)((const bf16_t*)x)[i] & 0x7fffu) << 16)
+                                 : (((const uint32_t*)x)[i] & 0x7fffffffu);
+            m = m > a ? m : a;
+        }
+    }
+    m = wave_max_u32(m);
+    __shared__ uint32_t red[4];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) red[w] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t t = red[0];
+        for (int i = 1; i < 4; i++) t = t > red[i] ? t : red[i];
+        atomicMax(amax_bits, t);
+    }
+}
+
+// ---------------------------------------------------------------- pass 2: convert
+template <bool IS_BF16, bool HW_CVT>
+__global__ __launch_bounds__(256) void convert_kernel(const void* __restrict__ x, int64_t n, const uint32_t* __restrict__ amax_bits,
+                                                      uint8_t* __restrict__ out, float* __restrict__ scale_out,
+                                                      float* __restrict__ inv_out) {
+    const float amax = __uint_as_float(*amax_bits);
+    const float scale = scale_from_amax(amax);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (scale_out) *scale_out = scale;
+        *inv_out = 1.0f / scale;
+    }
+    // 16 elements per thread-iteration: 32 B of bf16 (or 64 B of fp32) in, 16 B out
+    const int64_t n16 = n / 16;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (int64_t)gridDim.x * blockDim.x) {
+        float f[16];
+        if (IS_BF16) {
+            const uint4* p = (const uint4*)x + i * 2;
+            uint4 a = p[0], b = p[1];
+            uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                f[2 * j] = bf16_lo(w[j]);
+                f[2 * j + 1] = bf16_hi(w[j]);
+            }
+        } else {
+            const float4* p = (const float4*)x + i * 4;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float4 v = p[j];
+                f[4 * j] = v.x, f[4 * j + 1] = v.y, f[4 * j + 2] = v.z, f[4 * j + 3] = v.w;
+            }
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float y0 = clamp448(f[4 * j] * scale), y1 = clamp448(f[4 * j + 1] * scale);
+            float y2 = clamp448(f[4 * j + 2] * scale), y3 = clamp448(f[4 * j + 3] * scale);
+            o[j] = HW_CVT ? e4m3_pack4_hw(y0, y1, y2, y3) : e4m3_pack4_sw(y0, y1, y2, y3);
+        }
+        ((uint4*)out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    if (blockIdx.x == 0) {
+        for (int64_t i = n16 * 16 + threadIdx.x; i < n; i += blockDim.x) {
+            float v = IS_BF16 ? bf16_to_f32(((const bf16_t*)x)[i]) : ((const float*)x)[i];
+            float y = clamp448(v * scale);
+            out[i] = (uint8_t)(HW_CVT ? (e4m3_pack4_hw(y, 0.f, 0.f, 0.f) & 0xffu) : e4m3_encode_sw(y));
+        }
+    }
+}
+
+__global__ void clear_u32_kernel(uint32_t* p, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// Encode with a caller-given scale (no amax pass): used to check the encoder exhaustively.
+template <bool HW_CVT>
+__global__ void encode_with_scale_kernel(const bf16_t* __restrict__ x, int64_t n, float scale, uint8_t* __restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float y = clamp448(bf16_to_f32(x[i]) * scale);
+        out[i] = (uint8_t)(HW_CVT ? (e4m3_pack4_hw(y, 0.f, 0.f, 0.f) & 0xffu) : e4m3_encode_sw(y));
+    }
+}
+
+static int grid_for(int64_t work_items, int per_block, int max_blocks) {
+    int64_t g = (work_items + per_block - 1) / per_block;
+    if (g < 1) g = 1;
+    if (g > max_blocks) g = max_blocks;
+    return (int)g;
+}
+
+void nc_clear_u32(uint32_t* p, int n, hipStream_t s) {
+    hipLaunchKernelGGL(clear_u32_kernel, dim3((n + 63) / 64), dim3(64), 0, s, p, n);
+}
+
+int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_out,
+                       uint32_t* amax_ws, int encoder, hipStream_t s) {
+    NC_CHECK_ARG(x && out && inv_out && amax_ws, "fp8_quantize: null pointer");
+    NC_CHECK_ARG(n >= 0, "fp8_quantize: negative element count");
+    NC_CHECK_ARG(x_dtype == 0 || x_dtype == 1, "fp8_quantize: dtype must be 0 (bf16) or 1 (fp32)");
+    NC_CHECK_ARG(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "fp8_quantize: pointers must be 16-byte aligned");
+    nc_clear_u32(amax_ws, 1, s);
+    NcProfScope prof(2, 3.0 * n, s);
+    const int per_vec = x_dtype == 0 ? 8 : 4;
+    // 2048 blocks x 256 threads = 8 waves on each of 256 CUs; each block strides the tensor
+    int g1 = grid_for(n / per_vec, 256, 2048);
+    int g2 = grid_for(n / 16, 256, 4096);
+    if (x_dtype == 0) {
+        hipLaunchKernelGGL(amax_kernel<true>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
+        if (encoder == 0)
+            hipLaunchKernelGGL((convert_kernel<true, true>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+        else
+            hipLaunchKernelGGL((convert_kernel<true, false>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+    } else {
+        hipLaunchKernelGGL(amax_kernel<false>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
+        if (encoder == 0)
+            hipLaunchKernelGGL((convert_kernel<false, true>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+        else
+            hipLaunchKernelGGL((convert_kernel<false, false>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+    }
+    NC_CHECK_LAUNCH("fp8_quantize");
+    return 0;
+}
+
+// Convert only, with amax already reduced into amax_ws by a producer kernel.
+int nc_launch_convert_only(const void* x, int64_t n, uint8_t* out, float* inv_out, const uint32_t* amax_ws, hipStream_t s) {
+    NcProfScope prof(2, 3.0 * n, s);
+    int g2 = grid_for(n / 16, 256, 4096);
+    hipLaunchKernelGGL((convert_kernel<true, true>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, (float*)nullptr, inv_out);
+    NC_CHECK_LAUNCH("fp8_convert");
+    return 0;
+}
+
+int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, uint8_t* out, int encoder, hipStream_t s) {
+    NC_CHECK_ARG(x && out && n >= 0, "e4m3_encode: bad arguments");
+    int g = (int)((n + 255) / 256);
+    if (g == 0) return 0;
+    if (encoder == 0)
+        hipLaunchKernelGGL(encode_with_scale_kernel<true>, dim3(g), dim3(256), 0, s, x, n, scale, out);
+    else
+        hipLaunchKernelGGL(encode_with_scale_kernel<false>, dim3(g), dim3(256), 0, s, x, n, scale, out);
+    NC_CHECK_LAUNCH("e4m3_encode");
+    return 0;
+}

@@ -1,0 +1,211 @@
+// Logit softcap and next-token selection.
+//   softcap:  logits = softcap * tanh(float(bf16 lm_head output) / softcap)      nanochat/gpt.py:511-515
+//   sample:   temperature == 0 -> argmax (first index on ties);
+//             top-k -> the k largest logits in descending order, / temperature, softmax over k,
+//             then the multinomial draw written as its definition argmax_j(p_j / e_j), e_j ~ Exp(1)
+//             supplied by the caller (drawn from the torch generator)            nanochat/engine.py:140-156
+//             no top-k -> softmax over the whole vocabulary and the same draw.
+// One workgroup per batch row; a row of 32768 fp32 logits is 128 KB and is re-read from L2 by the
+// radix-select passes.  Bandwidth bound: B * V * 4 bytes from HBM once.
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+#define SAMPLE_THREADS 256
+#define MAX_TOP_K 256
+
+__global__ __launch_bounds__(256) void softcap_kernel(const bf16_t* __restrict__ raw, float* __restrict__ out, int64_t n, float softcap) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        out[i] = softcap * tanhf(bf16_to_f32(raw[i]) / softcap);
+}
+
+// order-preserving map float -> uint32 (larger float <=> larger key)
+__device__ __forceinline__ uint32_t fkey(float f) {
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float fkey_inv(uint32_t k) {
+    uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return __uint_as_float(u);
+}
+
+// (value desc, index asc) argmax across the block; returns the winner to every thread
+__device__ __forceinline__ void block_argmax(float& v, int& i, float* sval, int* sidx) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o);
+        const int oi = __shfl_xor(i, o);
+        if (ov > v || (ov == v && oi < i)) v = ov, i = oi;
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) sval[w] = v, sidx[w] = i;
+    __syncthreads();
+    v = sval[0], i = sidx[0];
+    for (int k = 1; k < SAMPLE_THREADS / 64; k++)
+        if (sval[k] > v || (sval[k] == v && sidx[k] < i)) v = sval[k], i = sidx[k];
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, int V, int ld, float temperature,
+                                                                int top_k, const float* __restrict__ noise, int64_t* __restrict__ out_ids) {
+    __shared__ float sval[4];
+    __shared__ int sidx[4];
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t sel_prefix, sel_need;
+    __shared__ unsigned long long cand[MAX_TOP_K];    // (key << 32) | ~index : sorts by value desc, index asc
+    __shared__ uint32_t cand_count;
+    __shared__ uint32_t scan[SAMPLE_THREADS];
+    __shared__ float probs[MAX_TOP_K];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float* lr = logits + (size_t)row * ld;
+
+    if (temperature == 0.0f) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = tid; i < V; i += SAMPLE_THREADS) {
+            const float v = lr[i];
+            if (v > bv || (v == bv && i < bi)) bv = v, bi = i;      // NaN never wins; an all-NaN row yields index 0 below
+        }
+        block_argmax(bv, bi, sval, sidx);
+        if (tid == 0) out_ids[row] = (bi == 0x7fffffff) ? 0 : bi;
+        return;
+    }
+
+    if (top_k <= 0 || top_k >= V) {
+        // full-vocabulary softmax: argmax_i exp((l_i - max)/T) / e_i  ==  argmax_i (l_i/T - max/T - log e_i)
+        float mx = -INFINITY;
+        int dummy = 0;
+        for (int i = tid; i < V; i += SAMPLE_THREADS) mx = fmaxf(mx, lr[i] / temperature);
+        block_argmax(mx, dummy, sval, sidx);
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = tid; i < V; i += SAMPLE_THREADS) {
+            const float p = expf(lr[i] / temperature - mx) / noise[(size_t)row * V + i];
+            if (p > bv || (p == bv && i < bi)) bv = p, bi = i;
+        }
+        block_argmax(bv, bi, sval, sidx);
+        if (tid == 0) out_ids[row] = (bi == 0x7fffffff) ? 0 : bi;
+        return;
+    }
+
+    // ---- radix select of the k-th largest key, 8 bits per pass from the top
+    const uint32_t k = (uint32_t)top_k;
+    if (tid == 0) sel_prefix = 0, sel_need = k, cand_count = 0;
+    for (int pass = 0; pass < 4; pass++) {
+        const int shift = 24 - 8 * pass;
+        hist[tid] = 0;
+        __syncthreads();
+        const uint32_t prefix = sel_prefix;
+        const uint32_t himask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+        for (int i = tid; i < V; i += SAMPLE_THREADS) {
+            const uint32_t key = fkey(lr[i]);
+            if ((key & himask) == prefix) atomicAdd(&hist[(key >> shift) & 0xff], 1u);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t need = sel_need, bin = 255;
+            for (;; bin--) {
+                if (hist[bin] >= need || bin == 0) break;
+                need -= hist[bin];
+            }
+            sel_need = need;                       // how many are still wanted inside the chosen bin
+            sel_prefix = prefix | (bin << shift);
+        }
+        __syncthreads();
+    }
+    const uint32_t kth = sel_prefix;               // key of the k-th largest logit
+    const uint32_t need_eq = sel_need;             // how many entries equal to it belong to the top k
+
+    // ---- collect: everything above the threshold, plus the lowest-index `need_eq` ties.
+    // Each thread owns a contiguous index range so ties are ranked by index with one block scan.
+    const int per = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    const int i0 = tid * per, i1 = min(V, i0 + per);
+    uint32_t eq_local = 0;
+    for (int i = i0; i < i1; i++) {
+        const uint32_t key = fkey(lr[i]);
+        if (key > kth) {
+            const uint32_t slot = atomicAdd(&cand_count, 1u);
+            if (slot < MAX_TOP_K) cand[slot] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
+        } else if (key == kth) eq_local++;
+    }
+    scan[tid] = eq_local;
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t run = 0;
+        for (int j = 0; j < SAMPLE_THREADS; j++) {
+            const uint32_t c = scan[j];
+            scan[j] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    uint32_t rank = scan[tid];
+    const uint32_t gt_count = cand_count;          // all "greater" entries are in by the barrier above
+    __syncthreads();
+    for (int i = i0; i < i1 && rank < need_eq; i++) {
+        if (fkey(lr[i]) == kth) {
+            const uint32_t slot = gt_count + rank;
+            if (slot < MAX_TOP_K) cand[slot] = ((unsigned long long)kth << 32) | (uint32_t)(~(uint32_t)i);
+            rank++;
+        }
+    }
+    for (int j = tid; j < MAX_TOP_K; j += SAMPLE_THREADS)
+        if ((uint32_t)j >= k) cand[j] = 0ull;      // padding sorts last
+    __syncthreads();
+
+    // ---- bitonic sort, descending, MAX_TOP_K entries, one per thread
+    for (int size = 2; size <= MAX_TOP_K; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            const int j = tid, partner = j ^ stride;
+            if (partner > j && j < MAX_TOP_K) {
+                const bool desc = ((j & size) == 0);
+                const unsigned long long a = cand[j], c = cand[partner];
+                if ((a < c) == desc) cand[j] = c, cand[partner] = a;
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- softmax over the k sorted values / T, then the draw
+    const float vmax = fkey_inv((uint32_t)(cand[0] >> 32)) / temperature;
+    float e = 0.f;
+    if ((uint32_t)tid < k) e = expf(fkey_inv((uint32_t)(cand[tid] >> 32)) / temperature - vmax);
+    probs[tid] = e;
+    __syncthreads();
+    float denom = 0.f;
+    for (uint32_t j = 0; j < k; j++) denom += probs[j];     // same order on every thread: deterministic
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    if ((uint32_t)tid < k) {
+        bv = (e / denom) / noise[(size_t)row * k + tid];
+        bi = tid;
+    }
+    block_argmax(bv, bi, sval, sidx);
+    if (tid == 0) {
+        const int choice = (bi == 0x7fffffff) ? 0 : bi;
+        out_ids[row] = (int64_t)(~(uint32_t)(cand[choice] & 0xffffffffull));
+    }
+}
+
+int nc_launch_softcap(const bf16_t* raw, float* out, int64_t n, float softcap, hipStream_t s) {
+    NC_CHECK_ARG(raw && out && n >= 0 && softcap > 0.f, "softcap: bad arguments");
+    int64_t g = (n + 255) / 256;
+    if (g < 1) g = 1;
+    if (g > 4096) g = 4096;
+    hipLaunchKernelGGL(softcap_kernel, dim3((int)g), dim3(256), 0, s, raw, out, n, softcap);
+    NC_CHECK_LAUNCH("softcap");
+    return 0;
+}
+
+int nc_launch_sample(const float* logits, int B, int V, int ld, float temperature, int top_k, const float* noise,
+                     int64_t* out_ids, hipStream_t s) {
+    NC_CHECK_ARG(logits && out_ids, "sample: null pointer");
+    NC_CHECK_ARG(B > 0 && V > 0 && ld >= V, "sample: bad shape B=%d V=%d ld=%d", B, V, ld);
+    NC_CHECK_ARG(temperature >= 0.0f, "sample: temperature must be non-negative");
+    NC_CHECK_ARG(temperature == 0.0f || noise, "sample: temperature > 0 needs the exponential noise buffer");
+    const int k_eff = (top_k > 0 && top_k < V) ? top_k : 0;
+    NC_CHECK_ARG(k_eff <= MAX_TOP_K, "sample: top_k %d exceeds the supported maximum of %d (or pass 0 for none)", top_k, MAX_TOP_K);
+    NcProfScope prof(4, 4.0 * B * V, s);
+    hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(SAMPLE_THREADS), 0, s, logits, V, ld, temperature, k_eff, noise, out_ids);
+    NC_CHECK_LAUNCH("sample");
+    return 0;
+}

@@ -1,0 +1,219 @@
+"""Tensor-level wrappers over the C ABI: validate, hand raw device pointers and the current HIP
+stream to libnanochat_amd.so, return torch tensors.  torch is used for memory and streams only.
+
+Every function requires CUDA (ROCm) tensors and raises otherwise: there is no CPU path here.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+_SCRATCH = {}
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("nanochat_amd ops run on the GPU only (got a CPU tensor); there is no CPU fallback")
+
+
+def _amax_slot(device):
+    """One uint32 of scratch per device and stream for quantize calls that bring no workspace."""
+    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    t = _SCRATCH.get(key)
+    if t is None:
+        t = torch.zeros(64, dtype=torch.int32, device=device)
+        _SCRATCH[key] = t
+    return t
+
+
+# ----------------------------------------------------------------------------- (1) quantize
+def fp8_quantize(x, encoder=0):
+    """Tensorwise e4m3 quantization of a bf16/fp32 tensor (nanochat/fp8.py:81-107).
+
+    Returns (payload float8_e4m3fn with x's shape, inv_scale fp32 0-dim, scale fp32 0-dim)."""
+    _need_cuda(x)
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"fp8_quantize: dtype {x.dtype} not supported (bf16 or fp32)")
+    x = x.contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(2, dtype=torch.float32, device=x.device)
+    ws = _amax_slot(x.device)
+    rc = _lib.lib().nc_fp8_quantize_tensorwise(_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _ptr(out),
+                                               C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4),
+                                               _ptr(ws), encoder, _stream())
+    _lib.check(rc)
+    return out.view(torch.float8_e4m3fn), scales[1], scales[0]
+
+
+def e4m3_encode_with_scale(x_bf16, scale, encoder=0):
+    _need_cuda(x_bf16)
+    assert x_bf16.dtype == torch.bfloat16
+    x = x_bf16.contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.lib().nc_e4m3_encode_with_scale(_ptr(x), x.numel(), float(scale), _ptr(out), encoder, _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------- (2) GEMM
+def fp8_gemm(a8, w8, inv_a, inv_w, seg_ends=None, softcap=None, kernel=0, out=None):
+    """out[M,N] = bf16((a8[M,K] @ w8[N,K]^T, fp32 acc) * inv_a * inv_w[segment]) (nanochat/fp8.py:143-153).
+
+    inv_w may hold several scales when w8 stacks weights along N; seg_ends lists their column ends.
+    With softcap, the result is fp32 softcap*tanh(bf16(v)/softcap) instead."""
+    _need_cuda(a8, w8, inv_a, inv_w)
+    if a8.dim() != 2 or w8.dim() != 2 or a8.shape[1] != w8.shape[1]:
+        raise ValueError(f"fp8_gemm: shapes {tuple(a8.shape)} x {tuple(w8.shape)}^T do not match")
+    if a8.element_size() != 1 or w8.element_size() != 1:
+        raise ValueError("fp8_gemm: operands must be e4m3 (one byte per element)")
+    a8, w8 = a8.contiguous(), w8.contiguous()
+    M, K = a8.shape
+    N = w8.shape[0]
+    inv_a = inv_a.reshape(-1).float()
+    inv_w = inv_w.reshape(-1).float().contiguous()
+    if seg_ends is None:
+        seg_ends = [N]
+    if len(seg_ends) != inv_w.numel():
+        raise ValueError("fp8_gemm: one weight inverse scale per column segment is required")
+    segs = (C.c_int32 * len(seg_ends))(*seg_ends)
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32 if softcap is not None else torch.bfloat16, device=a8.device)
+    rc = _lib.lib().nc_fp8_gemm_tn(_ptr(a8), _ptr(w8), _ptr(inv_a), _ptr(inv_w), segs, len(seg_ends), _ptr(out),
+                                   1 if softcap is not None else 0, float(softcap or 0.0), M, N, K, out.stride(0), kernel,
+                                   _stream())
+    _lib.check(rc)
+    return out
+
+
+# ----------------------------------------------------------------------------- (4) norm / rope / append
+def rms_norm(x):
+    """Parameter-free RMSNorm over the last dim of a bf16 tensor (nanochat/gpt.py:42-43)."""
+    _need_cuda(x)
+    if x.dtype != torch.bfloat16:
+        raise ValueError("rms_norm: bf16 only on the GPU path")
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    cols = x.shape[-1]
+    _lib.check(_lib.lib().nc_rmsnorm(_ptr(x), _ptr(out), x.numel() // cols, cols, C.c_void_p(0), _stream()))
+    return out
+
+
+def relu2(h):
+    _need_cuda(h)
+    h = h.contiguous()
+    out = torch.empty_like(h)
+    _lib.check(_lib.lib().nc_relu2(_ptr(h), _ptr(out), h.numel(), C.c_void_p(0), _stream()))
+    return out
+
+
+def embed_norm_smear(idx, wte, smear_w, smear_lambda, prev):
+    """(x [B,T,E], new prev_embedding [B,1,E]) -- nanochat/gpt.py:471-492."""
+    _need_cuda(idx, wte)
+    B, T = idx.shape
+    E = wte.shape[1]
+    x = torch.empty(B, T, E, dtype=torch.bfloat16, device=idx.device)
+    prev_out = torch.empty(B, 1, E, dtype=torch.bfloat16, device=idx.device)
+    rc = _lib.lib().nc_embed_norm_smear(_ptr(idx.contiguous()), _ptr(wte), _ptr(smear_w.float().contiguous()),
+                                        _ptr(smear_lambda.float().contiguous()), _ptr(prev), _ptr(prev_out), _ptr(x), B, T, E,
+                                        wte.shape[0], _stream())
+    _lib.check(rc)
+    return x, prev_out
+
+
+def mix_norm(x, add=None, x0=None, resid_lambda=None, x0_lambda=None, backout_lambda=None, backout_src=None,
+             want_backout=False):
+    """In-place residual update of x plus RMSNorm; returns (xn, saved_rows or None).  See nc_mix_norm."""
+    _need_cuda(x)
+    assert x.is_contiguous() and x.dtype == torch.bfloat16
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    xn = torch.empty_like(x)
+    saved = torch.empty_like(x) if want_backout else None
+    rc = _lib.lib().nc_mix_norm(_ptr(x), _ptr(add), _ptr(x0), _ptr(resid_lambda), _ptr(x0_lambda), _ptr(backout_lambda),
+                                _ptr(backout_src), _ptr(saved), _ptr(xn), rows, cols, C.c_void_p(0), _stream())
+    _lib.check(rc)
+    return xn, saved
+
+
+def qkv_rope_append(qkv, xn, idx, ve_table, ve_gate_w, cos, sin, cache_seqlens, k_cache, v_cache, n_head, n_kv_head):
+    """Rotary + QK-norm + gain on q,k; value-embedding gate on v; append k,v at cache_seqlens.. (in place).
+    qkv [B,T,(H+2Hkv)*128] bf16.  Returns q [B,T,H,128]."""
+    _need_cuda(qkv, k_cache, v_cache, cache_seqlens)
+    B, T = qkv.shape[0], qkv.shape[1]
+    qkv = qkv.contiguous()
+    q = torch.empty(B, T, n_head, 128, dtype=torch.bfloat16, device=qkv.device)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    Tmax = k_cache.shape[1]
+    vocab_rows = ve_table.shape[0] if ve_table is not None else 0
+    xn_c = xn.contiguous() if xn is not None else None
+    rc = _lib.lib().nc_qkv_rope_append(_ptr(qkv), qkv.shape[-1], _ptr(xn_c), xn_c.shape[-1] if xn_c is not None else 0,
+                                       _ptr(idx.contiguous() if idx is not None else None), _ptr(ve_table),
+                                       _ptr(ve_gate_w.float().contiguous() if ve_gate_w is not None else None),
+                                       _ptr(cos), _ptr(sin), cos.shape[0], _ptr(cache_seqlens), _ptr(k_cache), _ptr(v_cache),
+                                       _ptr(q), B, T, n_head, n_kv_head, Tmax, vocab_rows, _stream())
+    _lib.check(rc)
+    return q
+
+
+# ----------------------------------------------------------------------------- (3) attention
+def decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=-1, seqlens_include_new=False, splits=0):
+    """Attention of q [B,T,H,128] over caches [B,Tmax,Hkv,128] whose new tokens are already appended."""
+    _need_cuda(q, k_cache, v_cache, cache_seqlens)
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise ValueError("decode_attention: bf16 only")
+    if q.shape[-1] != 128 or k_cache.shape[-1] != 128:
+        raise ValueError("decode_attention: head_dim must be 128")
+    if cache_seqlens.dtype != torch.int32:
+        raise ValueError("decode_attention: cache_seqlens must be int32")
+    B, T, H, D = q.shape
+    Tmax, Hkv = k_cache.shape[1], k_cache.shape[2]
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("decode_attention: caches must be contiguous (B,Tmax,Hkv,128)")
+    q = q.contiguous()
+    out = torch.empty_like(q)
+    lib = _lib.lib()
+    ws_bytes = lib.nc_attention_workspace_bytes(B, T, H, Tmax)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    rc = lib.nc_decode_attention(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cache_seqlens), int(window_left), _ptr(out), B, T, H,
+                                 Hkv, Tmax, 1 if seqlens_include_new else 0, _ptr(ws), ws_bytes, C.c_void_p(0), splits,
+                                 _stream())
+    _lib.check(rc)
+    return out
+
+
+# ----------------------------------------------------------------------------- (5) softcap / sample
+def softcap(raw_bf16, cap=15.0):
+    _need_cuda(raw_bf16)
+    raw = raw_bf16.contiguous()
+    out = torch.empty(raw.shape, dtype=torch.float32, device=raw.device)
+    _lib.check(_lib.lib().nc_softcap(_ptr(raw), _ptr(out), raw.numel(), float(cap), _stream()))
+    return out
+
+
+def sample(logits, temperature, top_k, noise=None):
+    """Next-token ids [B,1] from fp32 logits [B,V] (nanochat/engine.py:140-156); noise: Exp(1) draws."""
+    _need_cuda(logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise ValueError("sample: logits must be fp32 [B,V]")
+    if logits.stride(1) != 1 or logits.stride(0) < logits.shape[1]:
+        logits = logits.contiguous()
+    B, V = logits.shape
+    out = torch.empty(B, 1, dtype=torch.int64, device=logits.device)
+    k = 0 if (top_k is None or top_k <= 0) else min(int(top_k), V)
+    if noise is not None:
+        noise = noise.contiguous()
+        want = k if (0 < k < V) else V
+        if tuple(noise.shape) != (B, want):
+            raise ValueError(f"sample: noise must have shape {(B, want)}, got {tuple(noise.shape)}")
+    rc = _lib.lib().nc_sample(_ptr(logits), B, V, logits.stride(0), float(temperature), k, _ptr(noise), _ptr(out), _stream())
+    _lib.check(rc)
+    return out
