@@ -130,8 +130,8 @@ void nc_clear_u32(uint32_t* p, int n, hipStream_t s) {
 
 int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_out,
                        uint32_t* amax_ws, int encoder, hipStream_t s) {
-    NC_CHECK_ARG(x && out && inv_out && amax_ws, "fp8_quantize: null pointer");
     NC_CHECK_ARG(n >= 0, "fp8_quantize: negative element count");
+    NC_CHECK_ARG(inv_out && amax_ws && (n == 0 || (x && out)), "fp8_quantize: null pointer");
     NC_CHECK_ARG(x_dtype == 0 || x_dtype == 1, "fp8_quantize: dtype must be 0 (bf16) or 1 (fp32)");
     NC_CHECK_ARG(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "fp8_quantize: pointers must be 16-byte aligned");
     nc_clear_u32(amax_ws, 1, s);
