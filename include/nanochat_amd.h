@@ -43,10 +43,24 @@ int nc_e4m3_encode_with_scale(const uint16_t* x, int64_t n, float scale, uint8_t
  * says where each one stops and inv_b holds one inverse scale per segment.
  * out_kind 0: bf16 out with leading dimension ldc.  out_kind 1: fp32 out of
  * softcap*tanh(bf16(v)/softcap), i.e. lm_head followed by nanochat/gpt.py:512-515.
- * kernel: 0 auto, 1 skinny (M<=128), 2/3/4 tile 256x256 / 256x128 / 128x128. */
+ * kernel: 0 auto, 1 small-M (M<=128), 2/3/4 tile 256x256 / 256x128 / 128x128.
+ * workspace (may be NULL): lets the small-M kernel split K over workgroups; size from
+ * nc_fp8_small_m_workspace_bytes(); its first 4096 bytes must be zero before the first use and are
+ * left zero by every call. */
 int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b,
                    const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap, int M, int N,
-                   int K, int ldc, int kernel, nc_stream_t stream);
+                   int K, int ldc, int kernel, void* workspace, size_t workspace_bytes, nc_stream_t stream);
+
+/* (1)+(2) fused for decode, M <= 128: Float8Linear.forward (nanochat/fp8.py:202-213) in one launch.
+ * a_bf16 [M,K] is quantized inside the kernel with the tensorwise scale derived from *a_amax (fp32
+ * bits of max|a|, e.g. produced by nc_rmsnorm / nc_mix_norm / nc_decode_attention), bit-identical to
+ * nc_fp8_quantize_tensorwise followed by nc_fp8_gemm_tn.  out_kind 0/1 as above; out_kind 2 writes
+ * bf16 relu(bf16(v))^2 (nanochat/gpt.py:139) and max-reduces it into *out_amax.  ksplits 0 = choose. */
+size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K);
+int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const uint8_t* b, const float* inv_b,
+                          const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap,
+                          uint32_t* out_amax, int M, int N, int K, int ldc, void* workspace, size_t workspace_bytes,
+                          int ksplits, nc_stream_t stream);
 
 /* (4a) Parameter-free RMSNorm over the last dimension: nanochat/gpt.py:42-43.  If amax_ws is not
  * NULL the kernel also atomically max-reduces |out| into it (fp32 bits; caller clears it). */

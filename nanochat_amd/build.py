@@ -15,7 +15,7 @@ OBJ_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(HERE, "libnanochat_amd.so")
 
 SOURCES = ["nc_api.hip", "nc_quantize.hip", "nc_gemm.hip", "nc_elementwise.hip", "nc_attention.hip",
-           "nc_sample.hip", "nc_forward.hip", "nc_profile.hip"]
+           "nc_sample.hip", "nc_forward.hip", "nc_profile.hip", "nc_gemm_decode.hip"]
 
 # -packed-fp32-ops off: packed fp32 VALU forms are not to be generated on this hardware pool
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",

@@ -31,15 +31,39 @@ int nc_e4m3_encode_with_scale(const uint16_t* x, int64_t n, float scale, uint8_t
     return nc_launch_encode_with_scale(x, n, scale, out, encoder, (hipStream_t)stream);
 }
 
-int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, const int32_t* seg_ends, int nseg,
-                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int kernel, nc_stream_t stream) {
-    NcGemmSegs segs{1, {N, 0, 0, 0}};
+static int segs_from(const int32_t* seg_ends, int nseg, int N, NcGemmSegs* segs) {
+    *segs = NcGemmSegs{1, {N, 0, 0, 0}};
     if (seg_ends) {
         NC_CHECK_ARG(nseg >= 1 && nseg <= 4, "fp8_gemm: 1..4 column segments supported, got %d", nseg);
-        segs.nseg = nseg;
-        for (int i = 0; i < nseg; i++) segs.end[i] = seg_ends[i];
+        segs->nseg = nseg;
+        for (int i = 0; i < nseg; i++) segs->end[i] = seg_ends[i];
     }
-    return nc_launch_gemm(a, b, inv_a, inv_b, segs, out, out_kind, softcap, M, N, K, ldc, kernel, (hipStream_t)stream);
+    return 0;
+}
+
+int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, const int32_t* seg_ends, int nseg,
+                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int kernel, void* workspace,
+                   size_t workspace_bytes, nc_stream_t stream) {
+    NcGemmSegs segs;
+    if (int rc = segs_from(seg_ends, nseg, N, &segs)) return rc;
+    return nc_launch_gemm(a, b, inv_a, inv_b, segs, out, out_kind, softcap, M, N, K, ldc, kernel, workspace, workspace_bytes,
+                          (hipStream_t)stream);
+}
+
+size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K) {
+    if (M < 1 || M > 128 || N < 1 || K < 1) return 0;
+    return NC_GEMM_COUNTER_BYTES + nc_gemm_decode_partial_bytes(M, N, K);
+}
+
+int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const uint8_t* b, const float* inv_b,
+                          const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap, uint32_t* out_amax, int M, int N,
+                          int K, int ldc, void* workspace, size_t workspace_bytes, int ksplits, nc_stream_t stream) {
+    NcGemmSegs segs;
+    if (int rc = segs_from(seg_ends, nseg, N, &segs)) return rc;
+    uint32_t* counters = workspace_bytes > NC_GEMM_COUNTER_BYTES ? (uint32_t*)workspace : nullptr;
+    void* parts = counters ? (uint8_t*)workspace + NC_GEMM_COUNTER_BYTES : nullptr;
+    return nc_launch_gemm_decode(a_bf16, 1, a_amax, nullptr, b, inv_b, segs, out, out_kind, softcap, out_amax, M, N, K, ldc, counters,
+                                 parts, counters ? workspace_bytes - NC_GEMM_COUNTER_BYTES : 0, ksplits, (hipStream_t)stream);
 }
 
 int nc_rmsnorm(const uint16_t* x, uint16_t* out, int rows, int cols, uint32_t* amax_ws, nc_stream_t stream) {
@@ -75,14 +99,17 @@ int nc_qkv_rope_append(const uint16_t* qkv, int ld_qkv, const uint16_t* xn, int 
 size_t nc_attention_workspace_bytes(int B, int T, int H, int Tmax) {
     (void)Tmax;
     if (B <= 0 || T <= 0 || H <= 0) return 0;
-    return nc_attn_ws_bytes(B, T, H);
+    return nc_attn_counter_bytes(B, T, H) + nc_attn_partial_bytes(B, T, H);
 }
 
 int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int32_t* cache_seqlens,
                         int window_left, uint16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                         void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits, nc_stream_t stream) {
+    const size_t cb = nc_attn_counter_bytes(B > 0 ? B : 1, T > 0 ? T : 1, H > 0 ? H : 1);
+    uint32_t* counters = (workspace && workspace_bytes > cb) ? (uint32_t*)workspace : nullptr;
+    void* parts = counters ? (uint8_t*)workspace + cb : nullptr;
     return nc_launch_attention(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new,
-                               workspace, workspace_bytes, amax_ws, splits, (hipStream_t)stream);
+                               counters, parts, counters ? workspace_bytes - cb : 0, amax_ws, splits, 0, (hipStream_t)stream);
 }
 
 int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_stream_t stream) {

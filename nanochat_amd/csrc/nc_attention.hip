@@ -11,7 +11,8 @@
 // (8 dims) each, so one 64-lane load instruction fetches four whole keys as four 256-byte segments.  The
 // 16-lane dot product is finished with DPP row rotations; each 16-lane group runs its own online softmax
 // over the keys it sees (no cross-lane traffic in the loop), and the four groups, then the four waves of
-// the workgroup, then the splits, are merged with the usual (max, sum, acc) rescale.  All G = H/Hkv
+// the workgroup, then the splits (by whichever split-workgroup finishes last, through a counter), are
+// merged with the usual (max, sum, acc) rescale.  All G = H/Hkv
 // query heads that share the kv head are processed by the same wave so K and V are read exactly once.
 //
 // HBM traffic per (row, kv head): 2 * n_keys * 256 bytes, the algorithmic minimum.
@@ -25,9 +26,10 @@ template <int G>
 __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                                                            const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
-                                                           float* __restrict__ partials, uint32_t* __restrict__ amax_ws, int T, int H,
-                                                           int Hkv, int Tmax, int nsplit) {
+                                                           float* __restrict__ partials, uint32_t* __restrict__ counters,
+                                                           uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, int nsplit) {
     __shared__ float merge[4][G][PART_STRIDE];
+    __shared__ int last_flag;
     const int split = blockIdx.x, hk = blockIdx.y, row = blockIdx.z;
     const int b = row / T, t = row % T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -184,33 +186,37 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             p[4 + d] = a;
         }
     }
-    if (nsplit == 1 && amax_ws) {
-        am = wave_max(am);
-        if (lane == 0 && am > 0.f) atomicMax(amax_ws, __float_as_uint(am));
+    if (nsplit > 1) {
+        // the split that arrives last at this (row, kv head) merges all of them, in split order
+        __threadfence();
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(&counters[row * Hkv + hk], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = (old == (uint32_t)(nsplit - 1));
+        }
+        __syncthreads();
+        if (!last_flag) return;
+        __threadfence();
+        for (int item = threadIdx.x; item < G * 128; item += 256) {
+            const int g = item >> 7, d = item & 127;
+            const int head = hk * G + g;
+            const float* p = partials + ((size_t)row * H + head) * nsplit * PART_STRIDE;
+            float mm = NEG_BIG;
+            for (int sidx = 0; sidx < nsplit; sidx++) mm = fmaxf(mm, p[sidx * PART_STRIDE]);
+            float ls = 0.f, a = 0.f;
+            for (int sidx = 0; sidx < nsplit; sidx++) {
+                const float sc = exp2f(p[sidx * PART_STRIDE] - mm);
+                ls += p[sidx * PART_STRIDE + 1] * sc;
+                a += p[sidx * PART_STRIDE + 4 + d] * sc;
+            }
+            const bf16_t o = f32_to_bf16(a / ls);
+            out[((size_t)row * H + head) * 128 + d] = o;
+            am = fmaxf(am, fabsf(bf16_to_f32(o)));
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(&counters[row * Hkv + hk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-}
-
-// one wave per (row, head): merge nsplit partials, write bf16
-__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ partials, bf16_t* __restrict__ out,
-                                                           uint32_t* __restrict__ amax_ws, int nsplit, int total) {
-    const int lane = threadIdx.x & 63;
-    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= total) return;
-    const float* p = partials + (size_t)item * nsplit * PART_STRIDE;
-    float mm = NEG_BIG;
-    for (int s = 0; s < nsplit; s++) mm = fmaxf(mm, p[s * PART_STRIDE]);
-    float ls = 0.f, a0 = 0.f, a1 = 0.f;
-    for (int s = 0; s < nsplit; s++) {
-        const float sc = exp2f(p[s * PART_STRIDE] - mm);
-        ls += p[s * PART_STRIDE + 1] * sc;
-        const float2 av = *(const float2*)(p + s * PART_STRIDE + 4 + lane * 2);
-        a0 += av.x * sc;
-        a1 += av.y * sc;
-    }
-    const bf16_t o0 = f32_to_bf16(a0 / ls), o1 = f32_to_bf16(a1 / ls);
-    *(uint32_t*)(out + (size_t)item * 128 + lane * 2) = (uint32_t)o0 | ((uint32_t)o1 << 16);
     if (amax_ws) {
-        float am = wave_max(fmaxf(fabsf(bf16_to_f32(o0)), fabsf(bf16_to_f32(o1))));
+        am = wave_max(am);
         if (lane == 0 && am > 0.f) atomicMax(amax_ws, __float_as_uint(am));
     }
 }
@@ -224,19 +230,20 @@ static int pick_splits(int B, int T, int Hkv, int max_keys) {
     return s;
 }
 
-size_t nc_attn_ws_bytes(int B, int T, int H) {
-    return (size_t)B * T * H * 16 * PART_STRIDE * sizeof(float);
-}
+// arrival counters, one per (row, kv head), zero between launches; split partials for up to 16 splits
+size_t nc_attn_counter_bytes(int B, int T, int H) { return (((size_t)B * T * H * sizeof(uint32_t)) + 255) & ~(size_t)255; }
+size_t nc_attn_partial_bytes(int B, int T, int H) { return (size_t)B * T * H * 16 * PART_STRIDE * sizeof(float); }
 
 int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
                         int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
-                        void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int force_splits, hipStream_t s) {
+                        uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
+                        int counters_are_zero, hipStream_t s) {
     NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
     NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0, "decode_attention: bad shape");
     NC_CHECK_ARG(H % Hkv == 0, "decode_attention: n_head %d not a multiple of n_kv_head %d", H, Hkv);
     const int G = H / Hkv;
     NC_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8, "decode_attention: query group size %d not in {1,2,4,8}", G);
-    NC_CHECK_ARG((long)B * T <= 65535 * 4L && Hkv <= 65535, "decode_attention: grid too large");
+    NC_CHECK_ARG((long)B * T <= 65535 && Hkv <= 65535, "decode_attention: more than 65535 query rows in one launch");
     NC_CHECK_ARG(((uintptr_t)q & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0,
                  "decode_attention: pointers must be 16-byte aligned");
     int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
@@ -244,25 +251,22 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
     NC_CHECK_ARG(nsplit >= 1 && nsplit <= 16, "decode_attention: splits must be 1..16");
     if (nsplit > 1) {
         const size_t need = (size_t)B * T * H * nsplit * PART_STRIDE * sizeof(float);
-        NC_CHECK_ARG(workspace && workspace_bytes >= need, "decode_attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        NC_CHECK_ARG(counters && partials && partial_bytes >= need, "decode_attention: %zu bytes of split workspace needed, %zu given",
+                     need, partial_bytes);
+        NC_CHECK_ARG(((uintptr_t)partials & 15) == 0, "decode_attention: workspace must be 16-byte aligned");
+        if (!counters_are_zero) nc_clear_u32(counters, B * T * Hkv, s);
     }
-    float* parts = (float*)workspace;
     NcProfScope prof(0, 0.0, s);
+    float* parts = (float*)partials;
     dim3 grid(nsplit, Hkv, B * T), block(256);
-    NC_CHECK_ARG(B * T <= 65535, "decode_attention: more than 65535 query rows in one launch");
 #define LAUNCH_G(GG)                                                                                                         \
     hipLaunchKernelGGL(attn_partial_kernel<GG>, grid, block, 0, s, q, k_cache, v_cache, cache_seqlens, window_left,             \
-                       seqlens_include_new, out, parts, amax_ws, T, H, Hkv, Tmax, nsplit)
+                       seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit)
     if (G == 1) LAUNCH_G(1);
     else if (G == 2) LAUNCH_G(2);
     else if (G == 4) LAUNCH_G(4);
     else LAUNCH_G(8);
 #undef LAUNCH_G
     NC_CHECK_LAUNCH("decode_attention");
-    if (nsplit > 1) {
-        const int total = B * T * H;
-        hipLaunchKernelGGL(attn_combine_kernel, dim3((total + 3) / 4), dim3(256), 0, s, parts, out, amax_ws, nsplit, total);
-        NC_CHECK_LAUNCH("decode_attention_combine");
-    }
     return 0;
 }

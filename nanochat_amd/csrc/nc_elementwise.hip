@@ -111,25 +111,81 @@ __global__ __launch_bounds__(256) void mix_norm_kernel(bf16_t* __restrict__ x, c
     block_amax_commit(am, amax_ws, red);
 }
 
-// out = rms_norm(x) over the last dim, rows independent (gpt.py:42-43)
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out, int cols,
-                                                      uint32_t* __restrict__ amax_ws) {
-    extern __shared__ float rowbuf[];
+// Same contract as mix_norm_kernel for cols % 8 == 0 and cols <= 2048 * NV: the row stays in registers,
+// eight bf16 per 16-byte access, one reduction, one pass over memory.
+template <int NV>
+__global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ add,
+                                                           const bf16_t* __restrict__ x0, const float* __restrict__ resid_lambda,
+                                                           const float* __restrict__ x0_lambda, const float* __restrict__ backout_lambda,
+                                                           const bf16_t* __restrict__ backout_src, bf16_t* __restrict__ backout_save,
+                                                           bf16_t* __restrict__ xn_out, int cols, uint32_t* __restrict__ amax_ws) {
     __shared__ float red[8];
     const size_t base = (size_t)blockIdx.x * cols;
+    const float rl = resid_lambda ? rbf(*resid_lambda) : 0.f;
+    const float xl = x0_lambda ? rbf(*x0_lambda) : 0.f;
+    const float bl = backout_lambda ? rbf(*backout_lambda) : 0.f;
+    const bool writes_x = add || resid_lambda || backout_lambda;
+    float v[NV][8];
     float ss = 0.f;
-    for (int c = threadIdx.x; c < cols; c += 256) {
-        float v = bf16_to_f32(x[base + c]);
-        rowbuf[c] = v;
-        ss += v * v;
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int c = (threadIdx.x + it * 256) * 8;
+        if (c < cols) {
+            const uint4 xv = *(const uint4*)(x + base + c);
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[it][2 * j] = bf16_lo(xw[j]), v[it][2 * j + 1] = bf16_hi(xw[j]);
+            if (add) {
+                const uint4 av = *(const uint4*)(add + base + c);
+                const uint32_t aw[4] = {av.x, av.y, av.z, av.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    v[it][2 * j] = rbf(v[it][2 * j] + bf16_lo(aw[j]));
+                    v[it][2 * j + 1] = rbf(v[it][2 * j + 1] + bf16_hi(aw[j]));
+                }
+            }
+            if (backout_save)
+                *(uint4*)(backout_save + base + c) = make_uint4(pack_bf16(v[it][0], v[it][1]), pack_bf16(v[it][2], v[it][3]),
+                                                                pack_bf16(v[it][4], v[it][5]), pack_bf16(v[it][6], v[it][7]));
+            if (resid_lambda) {
+                const uint4 zv = *(const uint4*)(x0 + base + c);
+                const uint32_t zw[4] = {zv.x, zv.y, zv.z, zv.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    v[it][2 * j] = rbf(rbf(rl * v[it][2 * j]) + rbf(xl * bf16_lo(zw[j])));
+                    v[it][2 * j + 1] = rbf(rbf(rl * v[it][2 * j + 1]) + rbf(xl * bf16_hi(zw[j])));
+                }
+            } else if (backout_lambda) {
+                const uint4 zv = *(const uint4*)(backout_src + base + c);
+                const uint32_t zw[4] = {zv.x, zv.y, zv.z, zv.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    v[it][2 * j] = rbf(v[it][2 * j] - rbf(bl * bf16_lo(zw[j])));
+                    v[it][2 * j + 1] = rbf(v[it][2 * j + 1] - rbf(bl * bf16_hi(zw[j])));
+                }
+            }
+            if (writes_x)
+                *(uint4*)(x + base + c) = make_uint4(pack_bf16(v[it][0], v[it][1]), pack_bf16(v[it][2], v[it][3]),
+                                                     pack_bf16(v[it][4], v[it][5]), pack_bf16(v[it][6], v[it][7]));
+#pragma unroll
+            for (int j = 0; j < 8; j++) ss += v[it][j] * v[it][j];
+        }
     }
     ss = block_sum<4>(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)cols + RMS_EPS);
     float am = 0.f;
-    for (int c = threadIdx.x; c < cols; c += 256) {
-        const bf16_t o = f32_to_bf16(rowbuf[c] * rstd);
-        out[base + c] = o;
-        am = fmaxf(am, fabsf(bf16_to_f32(o)));
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int c = (threadIdx.x + it * 256) * 8;
+        if (c < cols) {
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                o[j] = pack_bf16(v[it][2 * j] * rstd, v[it][2 * j + 1] * rstd);
+                am = fmaxf(am, fmaxf(fabsf(bf16_lo(o[j])), fabsf(bf16_hi(o[j]))));
+            }
+            *(uint4*)(xn_out + base + c) = make_uint4(o[0], o[1], o[2], o[3]);
+        }
     }
     block_amax_commit(am, amax_ws, red);
 }
@@ -233,11 +289,9 @@ static bool row_args_ok(int rows, int cols) { return rows >= 0 && cols > 0 && co
 int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
     NC_CHECK_ARG(x && out, "rmsnorm: null pointer");
     NC_CHECK_ARG(row_args_ok(rows, cols), "rmsnorm: bad shape rows=%d cols=%d (cols <= 16384)", rows, cols);
-    if (rows == 0) return 0;
-    NcProfScope prof(3, 4.0 * rows * cols, s);
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, out, cols, amax_ws);
-    NC_CHECK_LAUNCH("rmsnorm");
-    return 0;
+    // the mix kernel with no residual work never writes x
+    return nc_launch_mix_norm(const_cast<bf16_t*>(x), nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, out, rows, cols,
+                              amax_ws, s);
 }
 
 int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const float* smear_w, const float* smear_lambda,
@@ -262,8 +316,14 @@ int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const flo
     NC_CHECK_ARG(!(resid_lambda && backout_lambda), "mix_norm: residual mix and backout are exclusive");
     if (rows == 0) return 0;
     NcProfScope prof(3, 8.0 * rows * cols, s);
-    hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, add, x0, resid_lambda, x0_lambda,
-                       backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws);
+    const bool aligned = cols % 8 == 0 && (((uintptr_t)x | (uintptr_t)xn_out | (uintptr_t)add | (uintptr_t)x0 | (uintptr_t)backout_src |
+                                            (uintptr_t)backout_save) & 15) == 0;
+#define MIX_ARGS x, add, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws
+    if (aligned && cols <= 2048) hipLaunchKernelGGL(mix_norm_vec_kernel<1>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
+    else if (aligned && cols <= 4096) hipLaunchKernelGGL(mix_norm_vec_kernel<2>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
+    else if (aligned && cols <= 8192) hipLaunchKernelGGL(mix_norm_vec_kernel<4>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
+    else hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, MIX_ARGS);
+#undef MIX_ARGS
     NC_CHECK_LAUNCH("mix_norm");
     return 0;
 }

@@ -2,20 +2,38 @@
 // Python loop at nanochat/gpt.py:459-524 (and of the module calls it makes into gpt.py:84-153 and
 // fp8.py:202-213).  One call enqueues every kernel of the step; no host synchronisation, no allocation.
 //
-// Workspace layout (carved from the caller's buffer, 256-byte aligned pieces), M = B*T rows:
+// Per layer, decode (M = B*T <= 128 rows), 8 launches:
+//   mix_norm            x += mlp_out(prev); x = rl*x + xl*x0; xn = norm(x); amax(xn)
+//   linear q|k|v        quantize xn (inside the GEMM), three weight scales            -> qkv
+//   qkv_rope_append     rotary, QK-norm, gain, value-embedding gate, KV append        -> q, caches
+//   attention           split-K over the cache, merged by the last split; amax(y)     -> y
+//   linear c_proj       quantize y inside                                             -> o
+//   mix_norm            x += o; xn = norm(x); amax(xn)
+//   linear c_fc         quantize xn inside; epilogue relu^2 + amax                    -> h2
+//   linear mlp c_proj   quantize h2 inside                                            -> o (added by the next mix_norm)
+// Prefill (M > 128) uses the explicit convert kernel and the tiled GEMM instead of the fused small-M linear.
+//
+// Workspace (carved from the caller's buffer, 256-byte aligned pieces), M = B*T rows:
 //   x, x0, xn, xb, o      bf16 [M,E]        residual stream, its initial value, normed rows, backout, GEMM out
 //   qkv                   bf16 [M,(H+2Hkv)*128]
 //   qh, y                 bf16 [M,H*128]    rotated queries, attention output
-//   h, h2                 bf16 [M,4E]       c_fc output, relu^2
-//   a8                    u8   [M,4E]       quantized activations (input of the next GEMM)
-//   xl                    bf16 [B,E]        last-position rows (last_only lm_head)
-//   inv                   fp32 [4L+1]       activation inverse scales, one per FP8 linear input
-//   amax                  u32  [4L+1]       amax slots, cleared once at the start of the call
-//   attn                  fp32              split-K partials
+//   h, h2                 bf16 [M,4E]       c_fc output (prefill only), relu^2
+//   a8                    u8   [M,4E]       quantized activations (prefill only)
+//   xl                    bf16 [B,E]        last-position rows (last_only lm_head at T > 1)
+//   inv                   fp32 [4L+1]       activation inverse scales (prefill only)
+//   zeroed                u32               amax slots [4L+1] | GEMM split counters | attention split counters,
+//                                           cleared by one kernel at the start of the call
+//   gemm_parts, attn_parts                  split-K partials
 #include <stdio.h>
 #include "../../include/nanochat_amd.h"
 #include "nc_common.h"
 #include "nc_kernels.h"
+
+#define TRY(call)              \
+    do {                       \
+        int rc__ = (call);     \
+        if (rc__) return rc__; \
+    } while (0)
 
 namespace {
 struct Carver {
@@ -35,15 +53,17 @@ struct Workspace {
     bf16_t *x, *x0, *xn, *xb, *o, *qkv, *qh, *y, *h, *h2, *xl;
     uint8_t* a8;
     float* inv;
-    uint32_t* amax;
-    void* attn;
-    size_t attn_bytes;
+    uint32_t *amax, *gemm_counters, *attn_counters;
+    int zero_words;
+    uint8_t *gemm_parts, *attn_parts;
+    size_t gemm_part_bytes, attn_part_bytes;
     size_t total;
 };
 
 Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     const size_t M = (size_t)B * T, E = m->n_embd;
     const size_t qkv_w = (size_t)(m->n_head + 2 * m->n_kv_head) * 128;
+    const bool small = M <= 128;
     Carver c(base);
     Workspace w;
     w.x = c.take<bf16_t>(M * E);
@@ -54,14 +74,32 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     w.qkv = c.take<bf16_t>(M * qkv_w);
     w.qh = c.take<bf16_t>(M * m->n_head * 128);
     w.y = c.take<bf16_t>(M * m->n_head * 128);
-    w.h = c.take<bf16_t>(M * 4 * E);
+    w.h = c.take<bf16_t>(small ? 0 : M * 4 * E);
     w.h2 = c.take<bf16_t>(M * 4 * E);
-    w.a8 = c.take<uint8_t>(M * 4 * E);
+    w.a8 = c.take<uint8_t>(small ? 0 : M * 4 * E);
     w.xl = c.take<bf16_t>((size_t)B * E);
     w.inv = c.take<float>(4 * (size_t)m->n_layer + 1);
-    w.amax = c.take<uint32_t>(4 * (size_t)m->n_layer + 1);
-    w.attn_bytes = nc_attn_ws_bytes(B, T, m->n_head);
-    w.attn = c.take<uint8_t>(w.attn_bytes);
+    const size_t amax_words = (4 * (size_t)m->n_layer + 1 + 63) & ~(size_t)63;
+    const size_t gemm_words = NC_GEMM_COUNTER_BYTES / 4;
+    const size_t attn_words = nc_attn_counter_bytes(B, T, m->n_head) / 4;
+    uint32_t* zero = c.take<uint32_t>(amax_words + gemm_words + attn_words);
+    w.amax = zero;
+    w.gemm_counters = zero ? zero + amax_words : nullptr;
+    w.attn_counters = zero ? zero + amax_words + gemm_words : nullptr;
+    w.zero_words = (int)(amax_words + gemm_words + attn_words);
+    size_t gneed = 0;
+    if (small) {
+        const int shapes[5][2] = {{(int)qkv_w, (int)E}, {(int)E, m->n_head * 128}, {(int)(4 * E), (int)E}, {(int)E, (int)(4 * E)},
+                                  {m->vocab_size, (int)E}};
+        for (auto& sh : shapes) {
+            const size_t n = nc_gemm_decode_partial_bytes((int)M, sh[0], sh[1]);
+            gneed = n > gneed ? n : gneed;
+        }
+    }
+    w.gemm_part_bytes = gneed;
+    w.gemm_parts = c.take<uint8_t>(gneed);
+    w.attn_part_bytes = nc_attn_partial_bytes(B, T, m->n_head);
+    w.attn_parts = c.take<uint8_t>(w.attn_part_bytes);
     w.total = (c.off + 255) & ~(size_t)255;
     return w;
 }
@@ -73,18 +111,31 @@ __global__ void gather_last_rows_kernel(const bf16_t* __restrict__ x, bf16_t* __
     const bf16_t* src = x + ((size_t)b * T + (T - 1)) * E;
     for (int c = threadIdx.x; c < E; c += blockDim.x) out[(size_t)b * E + c] = src[c];
 }
+
+// One FP8 linear on `rows` rows of bf16 input whose amax sits in slot `site`.
+struct LinearRunner {
+    const Workspace& w;
+    hipStream_t s;
+    int run(const bf16_t* in, int rows, int site, const uint8_t* w8, const float* inv_w, NcGemmSegs segs, void* out, int out_kind,
+            float softcap, uint32_t* out_amax, int N, int K, int ldc) const {
+        if (rows <= 128)
+            return nc_launch_gemm_decode(in, 1, w.amax + site, nullptr, w8, inv_w, segs, out, out_kind, softcap, out_amax, rows, N, K, ldc,
+                                         w.gemm_counters, w.gemm_parts, w.gemm_part_bytes, 0, s);
+        // large M: explicit convert pass, tiled GEMM; relu^2 (out_kind 2) is a separate kernel there
+        TRY(nc_launch_convert_only(in, (int64_t)rows * K, w.a8, w.inv + site, w.amax + site, s));
+        if (out_kind == 2) {
+            TRY(nc_launch_gemm(w.a8, w8, w.inv + site, inv_w, segs, w.h, 0, 0.f, rows, N, K, N, 0, nullptr, 0, s));
+            return nc_launch_relu2(w.h, (bf16_t*)out, (int64_t)rows * N, out_amax, s);
+        }
+        return nc_launch_gemm(w.a8, w8, w.inv + site, inv_w, segs, out, out_kind, softcap, rows, N, K, ldc, 0, nullptr, 0, s);
+    }
+};
 }  // namespace
 
 extern "C" size_t nc_gpt_workspace_bytes(const nc_model_desc* model, int B, int T) {
     if (!model || B <= 0 || T <= 0) return 0;
     return carve(model, B, T, nullptr).total;
 }
-
-#define TRY(call)              \
-    do {                       \
-        int rc__ = (call);     \
-        if (rc__) return rc__; \
-    } while (0)
 
 extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, const int64_t* idx, int B, int T,
                               float* logits_out, int last_only, void* workspace, size_t workspace_bytes, nc_stream_t stream) {
@@ -102,9 +153,10 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
     const int L = m->n_layer, E = m->n_embd, H = m->n_head, Hkv = m->n_kv_head, M = B * T;
     const int qkv_w = (H + 2 * Hkv) * 128;
     const size_t layer_elems = (size_t)B * kv->max_seq_len * Hkv * 128;
-    int site = 0;   // index into inv / amax
+    const LinearRunner lin{w, s};
+    int site = 0;   // amax / inv slot of the next FP8 linear input
 
-    nc_clear_u32(w.amax, 4 * L + 1, s);
+    nc_clear_u32(w.amax, w.zero_words, s);
     TRY(nc_launch_embed_norm_smear(idx, m->wte, m->smear_w, m->smear_lambda, kv->prev_in, kv->prev_out, w.x, B, T, E,
                                    m->padded_vocab, s));
     // x0 is the post-smear embedding; layer 0 reads it through both x and x0 (gpt.py:495,500)
@@ -120,38 +172,32 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         TRY(nc_launch_mix_norm(w.x, pending_add, w.x0, m->resid_lambdas + i, m->x0_lambdas + i, nullptr, nullptr, save, w.xn, M, E,
                                w.amax + site, s));
         // q|k|v = FP8 linear(xn): one activation quantization, three weight scales
-        TRY(nc_launch_convert_only(w.xn, (int64_t)M * E, w.a8, w.inv + site, w.amax + site, s));
         NcGemmSegs qkv_segs{3, {H * 128, (H + Hkv) * 128, qkv_w, 0}};
-        TRY(nc_launch_gemm(w.a8, ly.w_qkv, w.inv + site, ly.inv_qkv, qkv_segs, w.qkv, 0, 0.f, M, qkv_w, E, qkv_w, 0, s));
+        TRY(lin.run(w.xn, M, site, ly.w_qkv, ly.inv_qkv, qkv_segs, w.qkv, 0, 0.f, nullptr, qkv_w, E, qkv_w));
         site++;
         bf16_t* kc = kv->k_cache + (size_t)i * layer_elems;
         bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
         TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
                                       kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
-        TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0, w.attn,
-                                w.attn_bytes, w.amax + site, 0, s));
-        // attention projection
-        TRY(nc_launch_convert_only(w.y, (int64_t)M * H * 128, w.a8, w.inv + site, w.amax + site, s));
-        TRY(nc_launch_gemm(w.a8, ly.w_attn_proj, w.inv + site, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, M, E, H * 128, E, 0, s));
+        TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
+                                w.attn_counters, w.attn_parts, w.attn_part_bytes, w.amax + site, 0, 1, s));
+        TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E));
         site++;
         // x += attn_out; xn = norm(x)
         TRY(nc_launch_mix_norm(w.x, w.o, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, w.xn, M, E, w.amax + site, s));
-        TRY(nc_launch_convert_only(w.xn, (int64_t)M * E, w.a8, w.inv + site, w.amax + site, s));
-        TRY(nc_launch_gemm(w.a8, ly.w_fc, w.inv + site, ly.inv_fc, one_seg(4 * E), w.h, 0, 0.f, M, 4 * E, E, 4 * E, 0, s));
+        // h2 = relu(c_fc(xn))^2 with its amax in the next slot
+        TRY(lin.run(w.xn, M, site, ly.w_fc, ly.inv_fc, one_seg(4 * E), w.h2, 2, 0.f, w.amax + site + 1, 4 * E, E, 4 * E));
         site++;
-        TRY(nc_launch_relu2(w.h, w.h2, (int64_t)M * 4 * E, w.amax + site, s));
-        TRY(nc_launch_convert_only(w.h2, (int64_t)M * 4 * E, w.a8, w.inv + site, w.amax + site, s));
-        TRY(nc_launch_gemm(w.a8, ly.w_mlp_proj, w.inv + site, ly.inv_mlp_proj, one_seg(E), w.o, 0, 0.f, M, E, 4 * E, E, 0, s));
+        TRY(lin.run(w.h2, M, site, ly.w_mlp_proj, ly.inv_mlp_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, 4 * E, E));
         site++;
         pending_add = w.o;
     }
     // x += mlp_out(last layer); x -= backout_lambda * x_backout; xn = norm(x)      (gpt.py:506-508)
     {
-        const bool last_is_backout = (L - 1) == L / 2;     // only when L == 1
-        bf16_t* save = last_is_backout ? w.xb : nullptr;
+        const bool last_is_backout = (L - 1) == L / 2;     // L == 1 or 2
         if (last_is_backout) {
             // the saved rows and the subtraction need the same x1: do the add first, then the backout pass
-            TRY(nc_launch_mix_norm(w.x, pending_add, nullptr, nullptr, nullptr, nullptr, nullptr, save, w.xn, M, E, nullptr, s));
+            TRY(nc_launch_mix_norm(w.x, pending_add, nullptr, nullptr, nullptr, nullptr, nullptr, w.xb, w.xn, M, E, nullptr, s));
             pending_add = nullptr;
         }
         TRY(nc_launch_mix_norm(w.x, pending_add, nullptr, nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.xn, M, E,
@@ -167,9 +213,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         head_in = w.xl;
         head_rows = B;
     }
-    TRY(nc_launch_convert_only(head_in, (int64_t)head_rows * E, w.a8, w.inv + site, w.amax + site, s));
-    NcGemmSegs head_seg{1, {m->vocab_size, 0, 0, 0}};
-    TRY(nc_launch_gemm(w.a8, m->w_lm_head, w.inv + site, m->inv_lm_head, head_seg, logits_out, 1, m->softcap, head_rows,
-                       m->vocab_size, E, m->vocab_size, 0, s));
+    TRY(lin.run(head_in, head_rows, site, m->w_lm_head, m->inv_lm_head, one_seg(m->vocab_size), logits_out, 1, m->softcap, nullptr,
+                m->vocab_size, E, m->vocab_size));
     return 0;
 }

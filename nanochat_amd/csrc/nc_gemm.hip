@@ -3,16 +3,14 @@
 // accumulation, bf16 output).  B may be several weight matrices stacked along N, each with its own
 // tensorwise inv-scale (the reference's c_q/c_k/c_v are three Float8Linear modules).
 //
-// Both kernels use v_mfma_f32_16x16x128_f8f6f4 (the full-rate fp8 MFMA of CDNA4): a lane supplies 32
+// The kernels use v_mfma_f32_16x16x128_f8f6f4 (the full-rate fp8 MFMA of CDNA4): a lane supplies 32
 // consecutive K bytes of row (lane & 15) from K-block (lane >> 4).  Operands are issued as (B, A) so a
 // lane ends up holding four consecutive output columns of one output row, which packs into one 8-byte
 // bf16 store.
 //
 //   gemm_tile_kernel    M large (prefill, isolated Float8Linear): BMxBNx128 tiles, 4 waves in 2x2,
 //                       double-buffered swizzled LDS, global loads of step k+1 overlap the MFMAs of step k.
-//   gemm_skinny_kernel  M <= 128 (decode): weight-bandwidth bound.  A workgroup owns 64 output columns,
-//                       each wave 16 of them over the whole K; weight rows stream global -> registers,
-//                       the small activation panel is shared through LDS.
+//   M <= 128 (decode) is weight-bandwidth bound and handled by gemm_decode_kernel in nc_gemm_decode.hip.
 #include "nc_common.h"
 #include "nc_kernels.h"
 
@@ -158,100 +156,6 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const uint8_t* __restric
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel: M <= 16*MB rows.  K is walked in super-steps of 512 bytes (four MFMA K-steps).
-// LDS holds the activation panel of one super-step, 512-byte rows, chunk c (0..31) of row r at slot
-// c ^ (r & 15).
-template <int MB>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
-                                                          EpilogueArgs ep, int M, int N, int K) {
-    constexpr int ROWS = MB * 16;
-    constexpr int A_CH = ROWS * 32 / 256;   // 16-byte chunks per thread per super-step
-    __shared__ __align__(16) uint8_t lds[2][ROWS * 512];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int frow = lane & 15, kb = lane >> 4;
-    const int n0 = blockIdx.x * 64 + wave * 16;
-    const int brow = n0 + frow;
-    const bool brow_ok = brow < N;
-    const uint8_t* bptr = B + (size_t)(brow_ok ? brow : 0) * K + kb * 32;
-
-    v4f acc[MB];
-#pragma unroll
-    for (int i = 0; i < MB; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    uint4 ra[A_CH];
-    uint4 rb[2][4][2];
-    auto load_a = [&](int ks) {
-#pragma unroll
-        for (int c = 0; c < A_CH; c++) {
-            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
-            const int gk = ks * 512 + ch * 16;
-            ra[c] = (row < M && gk < K) ? *(const uint4*)(A + (size_t)row * K + gk) : make_uint4(0, 0, 0, 0);
-        }
-    };
-    auto store_a = [&](int buf) {
-#pragma unroll
-        for (int c = 0; c < A_CH; c++) {
-            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
-            *(uint4*)(&lds[buf][row * 512 + ((ch ^ (row & 15)) << 4)]) = ra[c];
-        }
-    };
-    auto load_b = [&](int ks, int slot) {
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            const int gk = ks * 512 + kk * 128 + kb * 32;
-#pragma unroll
-            for (int h = 0; h < 2; h++)
-                rb[slot][kk][h] = (brow_ok && gk + h * 16 < K) ? *(const uint4*)(bptr + ks * 512 + kk * 128 + h * 16)
-                                                              : make_uint4(0, 0, 0, 0);
-        }
-    };
-
-    const int nsteps = (K + 511) / 512;
-    load_a(0);
-    load_b(0, 0);
-    store_a(0);
-    __syncthreads();
-#pragma unroll 1
-    for (int ks = 0; ks < nsteps; ks += 2) {
-        // two super-steps per trip so the register slots of rb are compile-time constants
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int s = ks + half;
-            if (s < nsteps) {
-                const bool more = s + 1 < nsteps;
-                if (more) {
-                    load_a(s + 1);
-                    load_b(s + 1, half ^ 1);
-                }
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) {
-                    v8i bf;
-                    const uint4 lo = rb[half][kk][0], hi = rb[half][kk][1];
-                    bf[0] = lo.x, bf[1] = lo.y, bf[2] = lo.z, bf[3] = lo.w, bf[4] = hi.x, bf[5] = hi.y, bf[6] = hi.z, bf[7] = hi.w;
-#pragma unroll
-                    for (int i = 0; i < MB; i++) {
-                        const int row = i * 16 + frow;
-                        const int c0 = kk * 8 + 2 * kb;
-                        const uint4 alo = *(const uint4*)(&lds[half][row * 512 + ((c0 ^ (row & 15)) << 4)]);
-                        const uint4 ahi = *(const uint4*)(&lds[half][row * 512 + (((c0 + 1) ^ (row & 15)) << 4)]);
-                        v8i af;
-                        af[0] = alo.x, af[1] = alo.y, af[2] = alo.z, af[3] = alo.w, af[4] = ahi.x, af[5] = ahi.y, af[6] = ahi.z, af[7] = ahi.w;
-                        acc[i] = MFMA_F8(acc[i], bf, af);
-                    }
-                }
-                if (more) store_a(half ^ 1);
-                __syncthreads();
-            }
-        }
-    }
-
-    const float inv_a = *ep.inv_a;
-#pragma unroll
-    for (int i = 0; i < MB; i++) store4(ep, inv_a, acc[i], i * 16 + frow, n0 + 4 * kb, M, N);
-}
-
-// ------------------------------------------------------------------------------------------------
 template <int BM, int BN>
 static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -265,7 +169,8 @@ static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& e
 }
 
 int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
-                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, hipStream_t s) {
+                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, void* workspace,
+                   size_t workspace_bytes, hipStream_t s) {
     NC_CHECK_ARG(a && b && inv_a && inv_b && out, "fp8_gemm: null pointer");
     NC_CHECK_ARG(M >= 0 && N > 0 && K > 0, "fp8_gemm: bad shape M=%d N=%d K=%d", M, N, K);
     NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
@@ -282,7 +187,6 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "fp8_gemm: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
     if (M == 0) return 0;
     EpilogueArgs ep{inv_a, inv_b, segs, out, out_kind, softcap, ldc};
-    NcProfScope prof(1, 2.0 * M * N * K, s);
 
     // force_kernel: 0 auto, 1 skinny, 2 tile 256x256, 3 tile 256x128, 4 tile 128x128
     int which = force_kernel;
@@ -294,13 +198,14 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         }
     }
     int rc = 0;
+    if (which != 1) NC_CHECK_ARG(which >= 2 && which <= 4, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s);
     if (which == 1) {
-        NC_CHECK_ARG(M <= 128, "fp8_gemm: skinny kernel needs M <= 128, got %d", M);
-        const int grid = (N + 63) / 64;
-        if (M <= 16) hipLaunchKernelGGL(gemm_skinny_kernel<1>, dim3(grid), dim3(256), 0, s, a, b, ep, M, N, K);
-        else if (M <= 32) hipLaunchKernelGGL(gemm_skinny_kernel<2>, dim3(grid), dim3(256), 0, s, a, b, ep, M, N, K);
-        else if (M <= 64) hipLaunchKernelGGL(gemm_skinny_kernel<4>, dim3(grid), dim3(256), 0, s, a, b, ep, M, N, K);
-        else hipLaunchKernelGGL(gemm_skinny_kernel<8>, dim3(grid), dim3(256), 0, s, a, b, ep, M, N, K);
+        NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
+        uint32_t* counters = workspace_bytes > NC_GEMM_COUNTER_BYTES ? (uint32_t*)workspace : nullptr;
+        void* parts = counters ? (uint8_t*)workspace + NC_GEMM_COUNTER_BYTES : nullptr;
+        return nc_launch_gemm_decode(a, 0, nullptr, inv_a, b, inv_b, segs, out, out_kind, softcap, nullptr, M, N, K, ldc, counters,
+                                     parts, counters ? workspace_bytes - NC_GEMM_COUNTER_BYTES : 0, 0, s);
     } else if (which == 2) rc = launch_tile<256, 256>(a, b, ep, M, N, K, s);
     else if (which == 3) rc = launch_tile<256, 128>(a, b, ep, M, N, K, s);
     else if (which == 4) rc = launch_tile<128, 128>(a, b, ep, M, N, K, s);

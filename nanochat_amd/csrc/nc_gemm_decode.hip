@@ -1,0 +1,312 @@
+// Small-M (decode) FP8 linear:  out[M,N] = epilogue((A[M,K] . W[N,K]^T, fp32 acc) * inv_a * inv_w),  M <= 128.
+// This is Float8Linear.forward (nanochat/fp8.py:202-213) at decode time, where the weight stream from HBM is
+// the whole cost: N*K bytes of e4m3 per call against M*K of activations.
+//
+// Work split: a workgroup (4 waves) owns 64 output columns (16 per wave) and a range of K-steps (128
+// wide); grid = (N/64) x ksplits so that even a 1664x1664 weight (2.8 MB) is spread over a few hundred
+// workgroups and every CU pulls a few KB.  Weight rows go global -> registers (one 16x128-byte MFMA
+// fragment per wave per K-step, two 16-byte loads per lane, rows contiguous).  The activation panel of
+// the K range is shared by the 4 waves through LDS; when A arrives as bf16 plus its tensorwise amax, it is
+// quantized to e4m3 on the way into LDS (scale = fp32(448/max(fp64(amax),1e-12)), saturate, RNE), so the
+// separate convert pass of the quantizer disappears.
+//
+// Split-K partial sums are written to a workspace; the workgroup that arrives last at a per-column-block
+// counter adds them in split order (so the result does not depend on arrival order), applies the scales
+// and the epilogue, and resets the counter.
+//
+// Epilogues: 0 bf16;  1 fp32 softcap*tanh(bf16(v)/softcap) (lm_head, nanochat/gpt.py:512-515);
+//            2 bf16 relu(bf16(v))^2 plus atomic amax of the result (MLP activation, gpt.py:139).
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+#define MFMA_F8(acc, b, a) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4((b), (a), (acc), 0, 0, 0, 0, 0, 0)
+
+struct DecodeGemmArgs {
+    const void* A;            // e4m3 [M,K] or bf16 [M,K]
+    const uint32_t* a_amax;   // bf16 mode: fp32 bits of max|A|
+    const float* inv_a;       // e4m3 mode: inverse scale of A
+    const uint8_t* B;
+    const float* inv_b;
+    NcGemmSegs segs;
+    void* out;
+    int out_kind;
+    float softcap;
+    int ldc;
+    uint32_t* out_amax;       // out_kind 2
+    float4* partials;
+    uint32_t* counters;
+    int ksplits, ksteps_per_split;
+    int M, N, K;
+};
+
+__device__ __forceinline__ float dg_seg_scale(const DecodeGemmArgs& g, int col) {
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+        if (i + 1 < g.segs.nseg && col >= g.segs.end[i]) s = i + 1;
+    return g.inv_b[s];
+}
+
+template <int MB, bool A_BF16>
+__global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
+    constexpr int ROWS = MB * 16;
+    constexpr int A_CH = ROWS * 32 / 256;          // 16-byte LDS chunks per thread per 512-wide sub-chunk
+    __shared__ __align__(16) uint8_t lds[2][ROWS * 512];
+    __shared__ float red[4];
+    __shared__ int last_flag;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int frow = lane & 15, kb = lane >> 4;
+    const int nblk = blockIdx.x, split = blockIdx.y;
+    const int M = g.M, N = g.N, K = g.K;
+    const int n0 = nblk * 64 + wave * 16;
+    const int brow = n0 + frow;
+    const bool brow_ok = brow < N;
+    const uint8_t* bptr = g.B + (size_t)(brow_ok ? brow : 0) * K + kb * 32;
+
+    const int nksteps = (K + 127) >> 7;
+    const int ks_begin = split * g.ksteps_per_split;
+    int ks_end = ks_begin + g.ksteps_per_split;
+    if (ks_end > nksteps) ks_end = nksteps;
+    const int k_hi = (ks_end << 7) < K ? (ks_end << 7) : K;       // exclusive K bound of this split
+
+    float scale = 1.f, inv_a;
+    if (A_BF16) {
+        scale = scale_from_amax(__uint_as_float(*g.a_amax));
+        inv_a = 1.0f / scale;
+    } else {
+        inv_a = *g.inv_a;
+    }
+
+    v4f acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    uint4 ra[A_CH][A_BF16 ? 2 : 1];
+    uint4 rb[2][4][2];
+    // sub-chunk c covers K-steps [ks_begin + 4c, ks_begin + 4c + 4)
+    auto load_a = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < A_CH; c++) {
+            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+            const int gk = k0 + ch * 16;
+            const bool ok = row < M && gk < k_hi;
+            if (A_BF16) {
+                const uint4* p = (const uint4*)((const bf16_t*)g.A + (size_t)row * K + gk);
+                ra[c][0] = ok ? p[0] : make_uint4(0, 0, 0, 0);
+                ra[c][A_BF16 ? 1 : 0] = ok ? p[1] : make_uint4(0, 0, 0, 0);
+            } else {
+                ra[c][0] = ok ? *(const uint4*)((const uint8_t*)g.A + (size_t)row * K + gk) : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < A_CH; c++) {
+            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+            uint4 v;
+            if (A_BF16) {
+                const uint32_t w[8] = {ra[c][0].x, ra[c][0].y, ra[c][0].z, ra[c][0].w,
+                                       ra[c][A_BF16 ? 1 : 0].x, ra[c][A_BF16 ? 1 : 0].y, ra[c][A_BF16 ? 1 : 0].z, ra[c][A_BF16 ? 1 : 0].w};
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    o[j] = e4m3_pack4_hw(clamp448(bf16_lo(w[2 * j]) * scale), clamp448(bf16_hi(w[2 * j]) * scale),
+                                         clamp448(bf16_lo(w[2 * j + 1]) * scale), clamp448(bf16_hi(w[2 * j + 1]) * scale));
+                v = make_uint4(o[0], o[1], o[2], o[3]);
+            } else {
+                v = ra[c][0];
+            }
+            *(uint4*)(&lds[buf][row * 512 + ((ch ^ (row & 15)) << 4)]) = v;
+        }
+    };
+    auto load_b = [&](int k0, int slot) {
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const int gk = k0 + kk * 128 + kb * 32;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                rb[slot][kk][h] = (brow_ok && gk + h * 16 < k_hi) ? *(const uint4*)(bptr + k0 + kk * 128 + h * 16)
+                                                                 : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    const int nsub = (ks_end - ks_begin + 3) >> 2;
+    const int kbase = ks_begin << 7;
+    if (nsub > 0) {
+        load_b(kbase, 0);
+        load_a(kbase);
+        store_a(0);
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int sc = 0; sc < nsub; sc += 2) {
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int s = sc + half;
+            if (s < nsub) {
+                const bool more = s + 1 < nsub;
+                if (more) {
+                    load_b(kbase + (s + 1) * 512, half ^ 1);
+                    load_a(kbase + (s + 1) * 512);
+                }
+                const int nk = min(4, ks_end - ks_begin - 4 * s);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    if (kk < nk) {
+                        v8i bf;
+                        const uint4 lo = rb[half][kk][0], hi = rb[half][kk][1];
+                        bf[0] = lo.x, bf[1] = lo.y, bf[2] = lo.z, bf[3] = lo.w, bf[4] = hi.x, bf[5] = hi.y, bf[6] = hi.z, bf[7] = hi.w;
+#pragma unroll
+                        for (int i = 0; i < MB; i++) {
+                            const int row = i * 16 + frow;
+                            const int c0 = kk * 8 + 2 * kb;
+                            const uint4 alo = *(const uint4*)(&lds[half][row * 512 + ((c0 ^ (row & 15)) << 4)]);
+                            const uint4 ahi = *(const uint4*)(&lds[half][row * 512 + (((c0 + 1) ^ (row & 15)) << 4)]);
+                            v8i af;
+                            af[0] = alo.x, af[1] = alo.y, af[2] = alo.z, af[3] = alo.w, af[4] = ahi.x, af[5] = ahi.y, af[6] = ahi.z, af[7] = ahi.w;
+                            acc[i] = MFMA_F8(acc[i], bf, af);
+                        }
+                    }
+                }
+                if (more) store_a(half ^ 1);
+                __syncthreads();
+            }
+        }
+    }
+
+    // ---- split-K: publish the partial tile; the last workgroup to arrive adds them up in split order
+    if (g.ksplits > 1) {
+        float4* mine = g.partials + ((size_t)(nblk * g.ksplits + split) * MB) * 256 + tid;
+#pragma unroll
+        for (int i = 0; i < MB; i++) mine[i * 256] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(&g.counters[nblk], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = (old == (uint32_t)(g.ksplits - 1));
+        }
+        __syncthreads();
+        if (!last_flag) return;
+        __threadfence();
+#pragma unroll
+        for (int i = 0; i < MB; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < g.ksplits; s++) {
+            const float4* theirs = g.partials + ((size_t)(nblk * g.ksplits + s) * MB) * 256 + tid;
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const float4 p = theirs[i * 256];
+                acc[i][0] += p.x, acc[i][1] += p.y, acc[i][2] += p.z, acc[i][3] += p.w;
+            }
+        }
+        if (tid == 0) __hip_atomic_store(&g.counters[nblk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- epilogue: lane holds rows i*16 + frow, columns n0 + 4*kb .. +3
+    float am = 0.f;
+    const int n = n0 + 4 * kb;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        const int m = i * 16 + frow;
+        if (m < M && n < N) {
+            const float inv_b = dg_seg_scale(g, n);
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] = (acc[i][r] * inv_a) * inv_b;
+            if (g.out_kind == 1) {
+                float* o = (float*)g.out + (size_t)m * g.ldc + n;
+                for (int r = 0; r < 4 && n + r < N; r++) o[r] = g.softcap * tanhf(rbf(v[r]) / g.softcap);
+            } else {
+                if (g.out_kind == 2) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const float t = fmaxf(rbf(v[r]), 0.f);
+                        v[r] = rbf(t * t);
+                        if (n + r < N) am = fmaxf(am, v[r]);
+                    }
+                }
+                bf16_t* o = (bf16_t*)g.out + (size_t)m * g.ldc + n;
+                if (n + 3 < N) *(uint2*)o = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                else
+                    for (int r = 0; r < 4 && n + r < N; r++) o[r] = f32_to_bf16(v[r]);
+            }
+        }
+    }
+    if (g.out_kind == 2 && g.out_amax) {
+        am = wave_max(am);
+        if (lane == 0) red[wave] = am;
+        __syncthreads();
+        if (tid == 0) {
+            am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            if (am > 0.f) atomicMax(g.out_amax, __float_as_uint(am));
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+static void plan_decode(int N, int K, int force_ksplits, int& ksplits, int& kps) {
+    const int nblk = (N + 63) / 64;
+    const int nksteps = (K + 127) / 128;
+    // enough workgroups to give every CU a slice; at most 8 splits keeps the partial traffic near the weight bytes
+    ksplits = force_ksplits > 0 ? force_ksplits : (384 + nblk - 1) / nblk;
+    if (ksplits > 8 && force_ksplits <= 0) ksplits = 8;
+    if (ksplits > nksteps) ksplits = nksteps;
+    kps = (nksteps + ksplits - 1) / ksplits;
+    ksplits = (nksteps + kps - 1) / kps;
+}
+
+// Split-K scratch: NC_GEMM_COUNTER_BYTES of arrival counters (one per 64-column block; zero before the first
+// use, left zero by every launch) and the partial tiles.
+size_t nc_gemm_decode_partial_bytes(int M, int N, int K) {
+    const int MB = M <= 64 ? 4 : 8;
+    const size_t nblk = (N + 63) / 64;
+    int ksplits, kps;
+    plan_decode(N, K, 0, ksplits, kps);
+    return ksplits > 1 ? nblk * ksplits * MB * 256 * sizeof(float4) : 0;
+}
+
+int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
+                          const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
+                          int N, int K, int ldc, uint32_t* counters, void* partials, size_t partial_bytes, int force_ksplits,
+                          hipStream_t s) {
+    NC_CHECK_ARG(a && b && inv_b && out, "fp8_gemm(decode): null pointer");
+    NC_CHECK_ARG(a_is_bf16 ? (a_amax != nullptr) : (inv_a != nullptr), "fp8_gemm(decode): activation scale missing");
+    NC_CHECK_ARG(M >= 1 && M <= 128 && N > 0 && K > 0, "fp8_gemm(decode): bad shape M=%d N=%d K=%d (M <= 128)", M, N, K);
+    NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
+    NC_CHECK_ARG(ldc >= N, "fp8_gemm: ldc=%d < N=%d", ldc, N);
+    NC_CHECK_ARG(((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0, "fp8_gemm: operands must be 16-byte aligned");
+    NC_CHECK_ARG(out_kind >= 0 && out_kind <= 2, "fp8_gemm: out_kind must be 0, 1 or 2");
+    NC_CHECK_ARG(segs.nseg >= 1 && segs.nseg <= 4 && segs.end[segs.nseg - 1] == N, "fp8_gemm: bad column segments");
+    for (int i = 0; i + 1 < segs.nseg; i++)
+        NC_CHECK_ARG(segs.end[i] % 4 == 0 && segs.end[i] < segs.end[i + 1], "fp8_gemm: segment ends must be increasing multiples of 4");
+    if (out_kind != 1) NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "fp8_gemm: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
+
+    const int MB = M <= 64 ? 4 : 8;
+    const int nblk = (N + 63) / 64;
+    const int nksteps = (K + 127) / 128;
+    int ksplits, kps;
+    plan_decode(N, K, force_ksplits, ksplits, kps);
+    const size_t need = (size_t)nblk * ksplits * MB * 256 * sizeof(float4);
+    if (ksplits > 1 && (!counters || !partials || partial_bytes < need || nblk > NC_GEMM_COUNTER_BYTES / 4)) {
+        if (force_ksplits > 1) NC_FAIL(-1, "fp8_gemm(decode): %d splits need %zu bytes of partial-sum workspace", ksplits, need);
+        ksplits = 1;
+        kps = nksteps;
+    }
+    DecodeGemmArgs g;
+    g.A = a, g.a_amax = a_amax, g.inv_a = inv_a, g.B = b, g.inv_b = inv_b, g.segs = segs, g.out = out, g.out_kind = out_kind;
+    g.softcap = softcap, g.ldc = ldc, g.out_amax = out_amax;
+    g.counters = counters;
+    g.partials = (float4*)partials;
+    g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
+    NcProfScope prof(1, 2.0 * M * N * K, s);
+    dim3 grid(nblk, ksplits), block(256);
+    if (MB == 4) {
+        if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<4, true>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((gemm_decode_kernel<4, false>), grid, block, 0, s, g);
+    } else {
+        if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<8, true>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((gemm_decode_kernel<8, false>), grid, block, 0, s, g);
+    }
+    NC_CHECK_LAUNCH("fp8_gemm(decode)");
+    return 0;
+}

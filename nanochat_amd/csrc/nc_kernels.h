@@ -21,7 +21,17 @@ struct NcGemmSegs {      // column segments of B, each with its own weight inv-s
 };
 // out_kind: 0 = bf16 [M,ldc];  1 = fp32 [M,ldc] of softcap*tanh(bf16(v)/softcap)
 int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
-                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, hipStream_t s);
+                   void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, void* workspace,
+                   size_t workspace_bytes, hipStream_t s);
+
+// small-M path (nc_gemm_decode.hip): A is e4m3 (+inv_a) or bf16 (+amax, quantized inside the kernel)
+// out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax
+#define NC_GEMM_COUNTER_BYTES 4096
+size_t nc_gemm_decode_partial_bytes(int M, int N, int K);
+int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
+                          const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
+                          int N, int K, int ldc, uint32_t* counters, void* partials, size_t partial_bytes, int force_ksplits,
+                          hipStream_t s);
 
 // ---- elementwise / norm / rope (nc_elementwise.hip)
 int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s);
@@ -38,10 +48,12 @@ int nc_launch_qkv_rope_append(const bf16_t* qkv, int ld_qkv, const bf16_t* xn, i
                               int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s);
 
 // ---- attention (nc_attention.hip)
-size_t nc_attn_ws_bytes(int B, int T, int H);
+size_t nc_attn_counter_bytes(int B, int T, int H);
+size_t nc_attn_partial_bytes(int B, int T, int H);
 int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
                         int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
-                        void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int force_splits, hipStream_t s);
+                        uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
+                        int counters_are_zero, hipStream_t s);
 
 // ---- sampling (nc_sample.hip)
 int nc_launch_softcap(const bf16_t* raw, float* out, int64_t n, float softcap, hipStream_t s);

@@ -18,7 +18,7 @@ bool g_on = false;
 }  // namespace
 
 int nc_prof_begin(int cls, double units, hipStream_t s) {
-    if (!g_on || g_used >= POOL) return -1;
+    if (!g_on || cls < 0 || g_used >= POOL) return -1;
     if (g_used >= g_created) {
         if (hipEventCreate(&g_recs[g_created].start) != hipSuccess) return -1;
         if (hipEventCreate(&g_recs[g_created].stop) != hipSuccess) return -1;
@@ -27,12 +27,12 @@ int nc_prof_begin(int cls, double units, hipStream_t s) {
     Rec& r = g_recs[g_used];
     r.cls = cls;
     r.units = units;
-    hipEventRecord(r.start, s);
+    (void)hipEventRecord(r.start, s);
     return g_used++;
 }
 
 void nc_prof_end(int slot, hipStream_t s) {
-    if (slot >= 0) hipEventRecord(g_recs[slot].stop, s);
+    if (slot >= 0) (void)hipEventRecord(g_recs[slot].stop, s);
 }
 
 extern "C" {

@@ -65,6 +65,20 @@ def e4m3_encode_with_scale(x_bf16, scale, encoder=0):
 
 
 # ----------------------------------------------------------------------------- (2) GEMM
+_GEMM_WS = {}
+
+
+def _small_m_workspace(device, M, N, K):
+    """Zero-initialised split-K scratch, kept per device and stream (its counter block stays zero between calls)."""
+    need = _lib.lib().nc_fp8_small_m_workspace_bytes(M, N, K)
+    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    ws = _GEMM_WS.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        _GEMM_WS[key] = ws
+    return ws
+
+
 def fp8_gemm(a8, w8, inv_a, inv_w, seg_ends=None, softcap=None, kernel=0, out=None):
     """out[M,N] = bf16((a8[M,K] @ w8[N,K]^T, fp32 acc) * inv_a * inv_w[segment]) (nanochat/fp8.py:143-153).
 
@@ -87,11 +101,42 @@ def fp8_gemm(a8, w8, inv_a, inv_w, seg_ends=None, softcap=None, kernel=0, out=No
     segs = (C.c_int32 * len(seg_ends))(*seg_ends)
     if out is None:
         out = torch.empty(M, N, dtype=torch.float32 if softcap is not None else torch.bfloat16, device=a8.device)
+    ws = _small_m_workspace(a8.device, M, N, K) if 1 <= M <= 128 else None
     rc = _lib.lib().nc_fp8_gemm_tn(_ptr(a8), _ptr(w8), _ptr(inv_a), _ptr(inv_w), segs, len(seg_ends), _ptr(out),
                                    1 if softcap is not None else 0, float(softcap or 0.0), M, N, K, out.stride(0), kernel,
-                                   _stream())
+                                   _ptr(ws), ws.numel() if ws is not None else 0, _stream())
     _lib.check(rc)
     return out
+
+
+def fp8_linear_small_m(a_bf16, amax_bits, w8, inv_w, seg_ends=None, softcap=None, relu2=False, ksplits=0):
+    """Float8Linear.forward for M <= 128 rows in one launch: a_bf16 [M,K] is quantized inside the GEMM with the
+    tensorwise scale of amax_bits (int32 tensor holding the fp32 bits of max|a|).  Returns the output, and with
+    relu2=True also an int32 tensor with the fp32 bits of max(relu(out)^2)."""
+    _need_cuda(a_bf16, amax_bits, w8, inv_w)
+    assert a_bf16.dtype == torch.bfloat16 and a_bf16.dim() == 2
+    a = a_bf16.contiguous()
+    w8 = w8.contiguous()
+    M, K = a.shape
+    N = w8.shape[0]
+    inv_w = inv_w.reshape(-1).float().contiguous()
+    if seg_ends is None:
+        seg_ends = [N]
+    segs = (C.c_int32 * len(seg_ends))(*seg_ends)
+    kind = 1 if softcap is not None else (2 if relu2 else 0)
+    out = torch.empty(M, N, dtype=torch.float32 if kind == 1 else torch.bfloat16, device=a.device)
+    out_amax = torch.zeros(1, dtype=torch.int32, device=a.device) if relu2 else None
+    ws = _small_m_workspace(a.device, M, N, K)
+    rc = _lib.lib().nc_fp8_linear_small_m(_ptr(a), _ptr(amax_bits), _ptr(w8), _ptr(inv_w), segs, len(seg_ends), _ptr(out), kind,
+                                          float(softcap or 0.0), _ptr(out_amax), M, N, K, out.stride(0), _ptr(ws), ws.numel(),
+                                          ksplits, _stream())
+    _lib.check(rc)
+    return (out, out_amax) if relu2 else out
+
+
+def amax_bits(x):
+    """fp32 bit pattern of max|x| as a one-element int32 tensor (what the producer kernels leave in an amax slot)."""
+    return x.detach().abs().max().float().reshape(1).view(torch.int32)
 
 
 # ----------------------------------------------------------------------------- (4) norm / rope / append
@@ -182,7 +227,7 @@ def decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=-1, seqlens
     out = torch.empty_like(q)
     lib = _lib.lib()
     ws_bytes = lib.nc_attention_workspace_bytes(B, T, H, Tmax)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)      # the call clears its own counters
     rc = lib.nc_decode_attention(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cache_seqlens), int(window_left), _ptr(out), B, T, H,
                                  Hkv, Tmax, 1 if seqlens_include_new else 0, _ptr(ws), ws_bytes, C.c_void_p(0), splits,
                                  _stream())

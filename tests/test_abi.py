@@ -29,7 +29,7 @@ def test_binding_and_error_channel():
     # argument validation happens before any GPU call, so it can be exercised without a device
     rc = lib.nc_fp8_quantize_tensorwise(None, 0, 16, None, None, None, None, 0, None)
     assert rc == -1 and b"null pointer" in lib.nc_last_error()
-    rc = lib.nc_fp8_gemm_tn(None, None, None, None, None, 1, None, 0, 0.0, 4, 4, 16, 4, 0, None)
+    rc = lib.nc_fp8_gemm_tn(None, None, None, None, None, 1, None, 0, 0.0, 4, 4, 16, 4, 0, None, 0, None)
     assert rc == -1
     rc = lib.nc_sample(None, 1, 8, 8, 1.0, 0, None, None, None)
     assert rc == -1

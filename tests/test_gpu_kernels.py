@@ -198,6 +198,34 @@ def test_gemm_softcap_epilogue(ops):
     assert (got_sc - want).abs().max().item() < 1e-5
 
 
+@pytest.mark.parametrize("M,N,K,ksplits", [(64, 1664, 1664, 0), (64, 4992, 1664, 0), (64, 6656, 1664, 0), (64, 1664, 6656, 0),
+                                           (64, 32768, 1664, 0), (64, 1664, 1664, 1), (64, 1664, 1664, 13), (64, 1664, 6656, 5),
+                                           (8, 256, 1024, 0), (1, 1024, 256, 2), (100, 2048, 2048, 0), (128, 512, 8192, 7),
+                                           (37, 208, 400, 3)])
+def test_fused_small_m_linear(ops, M, N, K, ksplits):
+    """Quantize-inside-the-GEMM decode linear: same bytes as quantize + GEMM, whatever the K split."""
+    say(f"fused small-M linear M={M} N={N} K={K} ksplits={ksplits}")
+    a, w = make_operands(M, N, K, seed=M + N + K)
+    a8, ia, _ = fp8_ref.to_fp8(a)
+    w8, iw, _ = fp8_ref.to_fp8(w)
+    want = fp8_ref.scaled_mm_emulated(a8, w8, ia, iw)
+    ad, w8d, iwd = a.to(DEV), w8.to(DEV), iw.reshape(1).to(DEV)
+    bits = ops.amax_bits(ad)
+    got = ops.fp8_linear_small_m(ad, bits, w8d, iwd, ksplits=ksplits)
+    err = rel_l2(got.cpu(), want)
+    assert err <= 2e-3, err
+    again = ops.fp8_linear_small_m(ad, bits, w8d, iwd, ksplits=ksplits)
+    assert torch.equal(got, again)                       # split-K is summed in a fixed order: run-to-run identical
+    two_step = ops.fp8_gemm(a8.to(DEV), w8d, ia.to(DEV), iwd, kernel=1)
+    if ksplits == 0:
+        assert torch.equal(got, two_step)                # the in-kernel quantizer produces the same payload
+    # relu^2 epilogue and its amax
+    h2, am = ops.fp8_linear_small_m(ad, bits, w8d, iwd, relu2=True, ksplits=ksplits)
+    want_h2 = torch.relu(got).square()
+    assert torch.equal(h2, want_h2)
+    assert am.view(torch.float32).item() == want_h2.float().max().item()
+
+
 @pytest.mark.parametrize("K,N", [(1664, 4992), (1664, 1664), (1664, 6656), (6656, 1664)])
 def test_gemm_full_float8linear_shapes(ops, K, N):
     """The isolated Float8Linear forward at M=8192: quantize + GEMM on the GPU; the oracle checks
