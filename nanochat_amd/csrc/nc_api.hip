@@ -52,7 +52,7 @@ int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const
 
 size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K) {
     if (M < 1 || M > 128 || N < 1 || K < 1) return 0;
-    return NC_GEMM_COUNTER_BYTES + nc_gemm_decode_partial_bytes(M, N, K);
+    return nc_gemm_decode_partial_bytes(M, N, K);
 }
 
 int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const uint8_t* b, const float* inv_b,
@@ -60,10 +60,18 @@ int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const 
                           int K, int ldc, void* workspace, size_t workspace_bytes, int ksplits, nc_stream_t stream) {
     NcGemmSegs segs;
     if (int rc = segs_from(seg_ends, nseg, N, &segs)) return rc;
-    uint32_t* counters = workspace_bytes > NC_GEMM_COUNTER_BYTES ? (uint32_t*)workspace : nullptr;
-    void* parts = counters ? (uint8_t*)workspace + NC_GEMM_COUNTER_BYTES : nullptr;
-    return nc_launch_gemm_decode(a_bf16, 1, a_amax, nullptr, b, inv_b, segs, out, out_kind, softcap, out_amax, M, N, K, ldc, counters,
-                                 parts, counters ? workspace_bytes - NC_GEMM_COUNTER_BYTES : 0, ksplits, (hipStream_t)stream);
+    NC_CHECK_ARG(out && inv_b, "fp8_linear_small_m: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int ks = ksplits > 0 ? ksplits : nc_gemm_decode_splits(N, K);
+    if (ksplits <= 0 && ks > 1 && (!workspace || workspace_bytes < (size_t)ks * M * N * sizeof(float))) ks = 1;
+    int used = 1;
+    if (int rc = nc_launch_gemm_decode(a_bf16, 1, a_amax, nullptr, b, inv_b, segs, out, out_kind, softcap, out_amax, M, N, K, ldc,
+                                       (float*)workspace, workspace_bytes, ks, &used, s))
+        return rc;
+    if (used > 1)
+        return nc_launch_finish_partials((const float*)workspace, used, a_amax, nullptr, inv_b, segs, out, out_kind, softcap, out_amax, M,
+                                         N, ldc, s);
+    return 0;
 }
 
 int nc_rmsnorm(const uint16_t* x, uint16_t* out, int rows, int cols, uint32_t* amax_ws, nc_stream_t stream) {

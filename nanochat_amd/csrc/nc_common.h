@@ -115,6 +115,45 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     return v;
 }
 
+// ---------------------------------------------------------------- cross-workgroup hand-off without cache flushes
+// Split results travel between workgroups through device-scope relaxed atomic accesses: such stores are
+// written through to the device coherence point and such loads are served from it, so no L2 write-back /
+// invalidate (what a device-scope fence costs on a multi-XCD part) is needed.  Ordering against the
+// arrival counter comes from waiting for the stores to complete before the counter is bumped.
+__device__ __forceinline__ void coherent_store_f4(float* p, float a, float b, float c, float d) {
+    unsigned long long lo = ((unsigned long long)__float_as_uint(b) << 32) | __float_as_uint(a);
+    unsigned long long hi = ((unsigned long long)__float_as_uint(d) << 32) | __float_as_uint(c);
+    __hip_atomic_store((unsigned long long*)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store((unsigned long long*)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coherent_load_f4(const float* p, float& a, float& b, float& c, float& d) {
+    unsigned long long lo = __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned long long hi = __hip_atomic_load((const unsigned long long*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    a = __uint_as_float((uint32_t)lo), b = __uint_as_float((uint32_t)(lo >> 32));
+    c = __uint_as_float((uint32_t)hi), d = __uint_as_float((uint32_t)(hi >> 32));
+}
+__device__ __forceinline__ void coherent_store_f1(float* p, float a) {
+    __hip_atomic_store((uint32_t*)p, __float_as_uint(a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load_f1(const float* p) {
+    return __uint_as_float(__hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+// All of this workgroup's coherent stores are complete when this returns on every thread (call from all threads);
+// returns true in every thread of the workgroup that arrived last at `counter` (of `expected` arrivals).
+__device__ __forceinline__ bool arrive_and_check_last(uint32_t* counter, uint32_t expected, int* flag_lds) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);       // vmcnt(0) expcnt(0) lgkmcnt(0): every store issued above has been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag_lds = (old == expected - 1u);
+    }
+    __syncthreads();
+    const bool last = *flag_lds != 0;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    return last;
+}
+
 // block-wide sum for blockDim.x == 64 * NW, result broadcast to every thread
 template <int NW>
 __device__ __forceinline__ float block_sum(float v, float* red /* >= NW floats of LDS */) {

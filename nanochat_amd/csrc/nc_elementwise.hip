@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void mix_norm_kernel(bf16_t* __restrict__ x, c
 // Same contract as mix_norm_kernel for cols % 8 == 0 and cols <= 2048 * NV: the row stays in registers,
 // eight bf16 per 16-byte access, one reduction, one pass over memory.
 template <int NV>
-__global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ add,
+__global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ add, NcPartialSrc padd,
                                                            const bf16_t* __restrict__ x0, const float* __restrict__ resid_lambda,
                                                            const float* __restrict__ x0_lambda, const float* __restrict__ backout_lambda,
                                                            const bf16_t* __restrict__ backout_src, bf16_t* __restrict__ backout_save,
@@ -124,7 +124,12 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
     const float rl = resid_lambda ? rbf(*resid_lambda) : 0.f;
     const float xl = x0_lambda ? rbf(*x0_lambda) : 0.f;
     const float bl = backout_lambda ? rbf(*backout_lambda) : 0.f;
-    const bool writes_x = add || resid_lambda || backout_lambda;
+    const bool writes_x = add || padd.parts || resid_lambda || backout_lambda;
+    float p_inv_a = 0.f, p_inv_b = 0.f;
+    if (padd.parts) {
+        p_inv_a = 1.0f / scale_from_amax(__uint_as_float(*padd.a_amax));
+        p_inv_b = padd.inv_b[0];
+    }
     float v[NV][8];
     float ss = 0.f;
 #pragma unroll
@@ -143,6 +148,18 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
                     v[it][2 * j] = rbf(v[it][2 * j] + bf16_lo(aw[j]));
                     v[it][2 * j + 1] = rbf(v[it][2 * j + 1] + bf16_hi(aw[j]));
                 }
+            }
+            if (padd.parts) {
+                float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                const float* pp = padd.parts + (size_t)blockIdx.x * padd.ld + c;
+                for (int sp = 0; sp < padd.nsplit; sp++) {
+                    const float4 a0 = *(const float4*)(pp + (size_t)sp * padd.split_stride);
+                    const float4 a1 = *(const float4*)(pp + (size_t)sp * padd.split_stride + 4);
+                    acc8[0] += a0.x, acc8[1] += a0.y, acc8[2] += a0.z, acc8[3] += a0.w;
+                    acc8[4] += a1.x, acc8[5] += a1.y, acc8[6] += a1.z, acc8[7] += a1.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[it][j] = rbf(v[it][j] + rbf((acc8[j] * p_inv_a) * p_inv_b));
             }
             if (backout_save)
                 *(uint4*)(backout_save + base + c) = make_uint4(pack_bf16(v[it][0], v[it][1]), pack_bf16(v[it][2], v[it][3]),
@@ -225,7 +242,8 @@ __global__ __launch_bounds__(256) void relu2_kernel(const bf16_t* __restrict__ h
 //   k heads: same -> k_cache[b, pos+t, h, :]
 //   v heads: v + 3*sigmoid(W_g . xn[:12])[h] * ve[idx, h, :] (if the layer has a value embedding) -> v_cache
 // (gpt.py:89-104, flash_attention.py:167-170)
-__global__ __launch_bounds__(256) void qkv_rope_append_kernel(const bf16_t* __restrict__ qkv, int ld_qkv, const bf16_t* __restrict__ xn,
+__global__ __launch_bounds__(256) void qkv_rope_append_kernel(const bf16_t* __restrict__ qkv, int ld_qkv, NcPartialSrc pq,
+                                                              const bf16_t* __restrict__ xn,
                                                               int ld_xn, const int64_t* __restrict__ idx, const bf16_t* __restrict__ ve_table,
                                                               const float* __restrict__ ve_gate_w, const bf16_t* __restrict__ cos_t,
                                                               const bf16_t* __restrict__ sin_t, int rope_len,
@@ -239,8 +257,24 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(const bf16_t* __re
     const int token = gw / heads, hh = gw % heads;
     const int b = token / T, t = token % T;
     const int pos = cache_seqlens[b] + t;
-    const bf16_t* src = qkv + (size_t)token * ld_qkv + (size_t)hh * 128;
-    float x1 = bf16_to_f32(src[lane]), x2 = bf16_to_f32(src[lane + 64]);
+    float x1, x2;
+    if (pq.parts) {
+        // the q|k|v linear's output still sits in split partials: add them up, scale, round to bf16
+        const int col = hh * 128 + lane;
+        const float* pp = pq.parts + (size_t)token * pq.ld + col;
+        float a1 = 0.f, a2 = 0.f;
+        for (int sp = 0; sp < pq.nsplit; sp++) {
+            a1 += pp[(size_t)sp * pq.split_stride];
+            a2 += pp[(size_t)sp * pq.split_stride + 64];
+        }
+        const float inv_a = 1.0f / scale_from_amax(__uint_as_float(*pq.a_amax));
+        const float inv_b = pq.inv_b[col >= pq.seg_end1 ? 2 : (col >= pq.seg_end0 ? 1 : 0)];
+        x1 = rbf((a1 * inv_a) * inv_b);
+        x2 = rbf((a2 * inv_a) * inv_b);
+    } else {
+        const bf16_t* src = qkv + (size_t)token * ld_qkv + (size_t)hh * 128;
+        x1 = bf16_to_f32(src[lane]), x2 = bf16_to_f32(src[lane + 64]);
+    }
     const bool in_cache = pos >= 0 && pos < Tmax;
 
     if (hh < H + Hkv) {
@@ -306,26 +340,48 @@ int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const floa
     return 0;
 }
 
-int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
-                       const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
-                       int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+static int launch_mix_norm_impl(bf16_t* x, const bf16_t* add, NcPartialSrc padd, const bf16_t* x0, const float* resid_lambda,
+                                const float* x0_lambda, const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save,
+                                bf16_t* xn_out, int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
     NC_CHECK_ARG(x && xn_out, "mix_norm: null pointer");
     NC_CHECK_ARG(row_args_ok(rows, cols), "mix_norm: bad shape rows=%d cols=%d", rows, cols);
     NC_CHECK_ARG(!resid_lambda || (x0 && x0_lambda), "mix_norm: the residual mix needs x0 and x0_lambda");
     NC_CHECK_ARG(!backout_lambda || backout_src, "mix_norm: backout needs its source rows");
     NC_CHECK_ARG(!(resid_lambda && backout_lambda), "mix_norm: residual mix and backout are exclusive");
+    NC_CHECK_ARG(!(add && padd.parts), "mix_norm: give the added tensor either as bf16 or as partials");
     if (rows == 0) return 0;
     NcProfScope prof(3, 8.0 * rows * cols, s);
     const bool aligned = cols % 8 == 0 && (((uintptr_t)x | (uintptr_t)xn_out | (uintptr_t)add | (uintptr_t)x0 | (uintptr_t)backout_src |
-                                            (uintptr_t)backout_save) & 15) == 0;
-#define MIX_ARGS x, add, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws
+                                            (uintptr_t)backout_save | (uintptr_t)padd.parts) & 15) == 0 && padd.ld % 4 == 0 &&
+                         padd.split_stride % 4 == 0;
+#define MIX_ARGS x, add, padd, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws
     if (aligned && cols <= 2048) hipLaunchKernelGGL(mix_norm_vec_kernel<1>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
     else if (aligned && cols <= 4096) hipLaunchKernelGGL(mix_norm_vec_kernel<2>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
     else if (aligned && cols <= 8192) hipLaunchKernelGGL(mix_norm_vec_kernel<4>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
-    else hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, MIX_ARGS);
+    else {
+        NC_CHECK_ARG(!padd.parts, "mix_norm: partial-sum input needs cols %% 8 == 0, cols <= 8192 and 16-byte alignment");
+        hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, add, x0, resid_lambda, x0_lambda,
+                           backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws);
+    }
 #undef MIX_ARGS
     NC_CHECK_LAUNCH("mix_norm");
     return 0;
+}
+
+int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
+                       const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
+                       int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+    NcPartialSrc none{nullptr, 0, 0, 0, nullptr, nullptr, 0, 0};
+    return launch_mix_norm_impl(x, add, none, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, rows,
+                                cols, amax_ws, s);
+}
+
+int nc_launch_mix_norm_p(bf16_t* x, NcPartialSrc add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
+                         const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
+                         int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+    NC_CHECK_ARG(!add.parts || (add.nsplit >= 1 && add.a_amax && add.inv_b && add.ld >= cols), "mix_norm: bad partial-sum source");
+    return launch_mix_norm_impl(x, nullptr, add, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, rows,
+                                cols, amax_ws, s);
 }
 
 int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, hipStream_t s) {
@@ -340,18 +396,36 @@ int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, 
     return 0;
 }
 
+static int launch_rope_impl(const bf16_t* qkv, int ld_qkv, NcPartialSrc pq, const bf16_t* xn, int ld_xn, const int64_t* idx,
+                            const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin, int rope_len,
+                            const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out, int B, int T, int H, int Hkv,
+                            int Tmax, int vocab_rows, hipStream_t s) {
+    NC_CHECK_ARG((qkv || pq.parts) && cos && sin && cache_seqlens && k_cache && v_cache && q_out, "qkv_rope_append: null pointer");
+    NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && Tmax > 0 && rope_len > 0, "qkv_rope_append: bad shape");
+    NC_CHECK_ARG((pq.parts ? pq.ld : ld_qkv) >= (H + 2 * Hkv) * 128, "qkv_rope_append: row stride too small (head_dim is fixed at 128)");
+    NC_CHECK_ARG(!ve_table || (ve_gate_w && xn && idx && ld_xn >= 12), "qkv_rope_append: value embedding needs gate weights, xn and idx");
+    const int total = B * T * (H + 2 * Hkv);
+    NcProfScope prof(3, 4.0 * total * 128, s);
+    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, qkv, ld_qkv, pq, xn, ld_xn, idx, ve_table,
+                       ve_gate_w, cos, sin, rope_len, cache_seqlens, k_cache, v_cache, q_out, T, H, Hkv, Tmax, vocab_rows, total);
+    NC_CHECK_LAUNCH("qkv_rope_append");
+    return 0;
+}
+
 int nc_launch_qkv_rope_append(const bf16_t* qkv, int ld_qkv, const bf16_t* xn, int ld_xn, const int64_t* idx,
                               const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,
                               int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,
                               int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s) {
-    NC_CHECK_ARG(qkv && cos && sin && cache_seqlens && k_cache && v_cache && q_out, "qkv_rope_append: null pointer");
-    NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && Tmax > 0 && rope_len > 0, "qkv_rope_append: bad shape");
-    NC_CHECK_ARG(ld_qkv >= (H + 2 * Hkv) * 128, "qkv_rope_append: ld_qkv too small (head_dim is fixed at 128)");
-    NC_CHECK_ARG(!ve_table || (ve_gate_w && xn && idx && ld_xn >= 12), "qkv_rope_append: value embedding needs gate weights, xn and idx");
-    const int total = B * T * (H + 2 * Hkv);
-    NcProfScope prof(3, 4.0 * total * 128, s);
-    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, qkv, ld_qkv, xn, ld_xn, idx, ve_table, ve_gate_w,
-                       cos, sin, rope_len, cache_seqlens, k_cache, v_cache, q_out, T, H, Hkv, Tmax, vocab_rows, total);
-    NC_CHECK_LAUNCH("qkv_rope_append");
-    return 0;
+    NcPartialSrc none{nullptr, 0, 0, 0, nullptr, nullptr, 0, 0};
+    return launch_rope_impl(qkv, ld_qkv, none, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin, rope_len, cache_seqlens, k_cache, v_cache,
+                            q_out, B, T, H, Hkv, Tmax, vocab_rows, s);
+}
+
+int nc_launch_qkv_rope_append_p(NcPartialSrc qkv_parts, const bf16_t* xn, int ld_xn, const int64_t* idx,
+                                const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,
+                                int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,
+                                int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s) {
+    NC_CHECK_ARG(qkv_parts.parts && qkv_parts.nsplit >= 1 && qkv_parts.a_amax && qkv_parts.inv_b, "qkv_rope_append: bad partial-sum source");
+    return launch_rope_impl(nullptr, 0, qkv_parts, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin, rope_len, cache_seqlens, k_cache,
+                            v_cache, q_out, B, T, H, Hkv, Tmax, vocab_rows, s);
 }

@@ -2,15 +2,16 @@
 // Python loop at nanochat/gpt.py:459-524 (and of the module calls it makes into gpt.py:84-153 and
 // fp8.py:202-213).  One call enqueues every kernel of the step; no host synchronisation, no allocation.
 //
-// Per layer, decode (M = B*T <= 128 rows), 8 launches:
-//   mix_norm            x += mlp_out(prev); x = rl*x + xl*x0; xn = norm(x); amax(xn)
-//   linear q|k|v        quantize xn (inside the GEMM), three weight scales            -> qkv
-//   qkv_rope_append     rotary, QK-norm, gain, value-embedding gate, KV append        -> q, caches
-//   attention           split-K over the cache, merged by the last split; amax(y)     -> y
-//   linear c_proj       quantize y inside                                             -> o
-//   mix_norm            x += o; xn = norm(x); amax(xn)
-//   linear c_fc         quantize xn inside; epilogue relu^2 + amax                    -> h2
-//   linear mlp c_proj   quantize h2 inside                                            -> o (added by the next mix_norm)
+// Per layer, decode (M = B*T <= 128 rows), 9 launches, each making a single dependent trip to memory:
+//   mix_norm            x += mlp_out(prev) [read from split partials]; x = rl*x + xl*x0; xn = norm(x); amax(xn)
+//   linear q|k|v        quantize xn inside the GEMM; K split over workgroups           -> fp32 partials
+//   qkv_rope_append     sums the partials (three weight scales), rotary, QK-norm, gain, VE gate, KV append -> q, caches
+//   attention           over the cache; amax(y)                                        -> y
+//   linear c_proj       quantize y inside                                              -> partials
+//   mix_norm            x += o [from partials]; xn = norm(x); amax(xn)
+//   linear c_fc         quantize xn inside                                             -> partials
+//   finish_partials     sum, scale, relu^2, amax                                       -> h2
+//   linear mlp c_proj   quantize h2 inside                                             -> partials (added by the next mix_norm)
 // Prefill (M > 128) uses the explicit convert kernel and the tiled GEMM instead of the fused small-M linear.
 //
 // Workspace (carved from the caller's buffer, 256-byte aligned pieces), M = B*T rows:
@@ -21,9 +22,9 @@
 //   a8                    u8   [M,4E]       quantized activations (prefill only)
 //   xl                    bf16 [B,E]        last-position rows (last_only lm_head at T > 1)
 //   inv                   fp32 [4L+1]       activation inverse scales (prefill only)
-//   zeroed                u32               amax slots [4L+1] | GEMM split counters | attention split counters,
-//                                           cleared by one kernel at the start of the call
-//   gemm_parts, attn_parts                  split-K partials
+//   zeroed                u32               amax slots [4L+1] | attention split counters, cleared by one kernel at
+//                                           the start of the call
+//   gemm_parts, attn_parts                  split partials of the small-M linears and of attention
 #include <stdio.h>
 #include "../../include/nanochat_amd.h"
 #include "nc_common.h"
@@ -53,7 +54,7 @@ struct Workspace {
     bf16_t *x, *x0, *xn, *xb, *o, *qkv, *qh, *y, *h, *h2, *xl;
     uint8_t* a8;
     float* inv;
-    uint32_t *amax, *gemm_counters, *attn_counters;
+    uint32_t *amax, *attn_counters;
     int zero_words;
     uint8_t *gemm_parts, *attn_parts;
     size_t gemm_part_bytes, attn_part_bytes;
@@ -80,13 +81,11 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     w.xl = c.take<bf16_t>((size_t)B * E);
     w.inv = c.take<float>(4 * (size_t)m->n_layer + 1);
     const size_t amax_words = (4 * (size_t)m->n_layer + 1 + 63) & ~(size_t)63;
-    const size_t gemm_words = NC_GEMM_COUNTER_BYTES / 4;
     const size_t attn_words = nc_attn_counter_bytes(B, T, m->n_head) / 4;
-    uint32_t* zero = c.take<uint32_t>(amax_words + gemm_words + attn_words);
+    uint32_t* zero = c.take<uint32_t>(amax_words + attn_words);
     w.amax = zero;
-    w.gemm_counters = zero ? zero + amax_words : nullptr;
-    w.attn_counters = zero ? zero + amax_words + gemm_words : nullptr;
-    w.zero_words = (int)(amax_words + gemm_words + attn_words);
+    w.attn_counters = zero ? zero + amax_words : nullptr;
+    w.zero_words = (int)(amax_words + attn_words);
     size_t gneed = 0;
     if (small) {
         const int shapes[5][2] = {{(int)qkv_w, (int)E}, {(int)E, m->n_head * 128}, {(int)(4 * E), (int)E}, {(int)E, (int)(4 * E)},
@@ -112,15 +111,29 @@ __global__ void gather_last_rows_kernel(const bf16_t* __restrict__ x, bf16_t* __
     for (int c = threadIdx.x; c < E; c += blockDim.x) out[(size_t)b * E + c] = src[c];
 }
 
-// One FP8 linear on `rows` rows of bf16 input whose amax sits in slot `site`.
+const NcPartialSrc NO_PARTIALS{nullptr, 0, 0, 0, nullptr, nullptr, 0, 0};
+
+// One FP8 linear on `rows` rows of bf16 input whose amax sits in slot `site`.  Small M: the result is either
+// in `out` (single split: epilogue done in the GEMM) or described by *src (split partials for the consumer).
 struct LinearRunner {
     const Workspace& w;
     hipStream_t s;
     int run(const bf16_t* in, int rows, int site, const uint8_t* w8, const float* inv_w, NcGemmSegs segs, void* out, int out_kind,
-            float softcap, uint32_t* out_amax, int N, int K, int ldc) const {
-        if (rows <= 128)
-            return nc_launch_gemm_decode(in, 1, w.amax + site, nullptr, w8, inv_w, segs, out, out_kind, softcap, out_amax, rows, N, K, ldc,
-                                         w.gemm_counters, w.gemm_parts, w.gemm_part_bytes, 0, s);
+            float softcap, uint32_t* out_amax, int N, int K, int ldc, NcPartialSrc* src) const {
+        if (src) *src = NO_PARTIALS;
+        if (rows <= 128) {
+            int used = 1;
+            TRY(nc_launch_gemm_decode(in, 1, w.amax + site, nullptr, w8, inv_w, segs, out, out_kind, softcap, out_amax, rows, N, K, ldc,
+                                      (float*)w.gemm_parts, w.gemm_part_bytes, src || out_kind == 2 ? 0 : 1, &used, s));
+            if (used == 1) return 0;
+            if (src) {
+                *src = NcPartialSrc{(const float*)w.gemm_parts, used, N, (size_t)rows * N, w.amax + site, inv_w,
+                                    segs.nseg > 1 ? segs.end[0] : 0x7fffffff, segs.nseg > 2 ? segs.end[1] : 0x7fffffff};
+                return 0;
+            }
+            return nc_launch_finish_partials((const float*)w.gemm_parts, used, w.amax + site, nullptr, inv_w, segs, out, out_kind, softcap,
+                                             out_amax, rows, N, ldc, s);
+        }
         // large M: explicit convert pass, tiled GEMM; relu^2 (out_kind 2) is a separate kernel there
         TRY(nc_launch_convert_only(in, (int64_t)rows * K, w.a8, w.inv + site, w.amax + site, s));
         if (out_kind == 2) {
@@ -163,45 +176,56 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
     if (hipMemcpyAsync(w.x0, w.x, (size_t)M * E * sizeof(bf16_t), hipMemcpyDeviceToDevice, s) != hipSuccess)
         NC_FAIL(-2, "gpt_forward: x0 copy failed");
 
-    const bf16_t* pending_add = nullptr;   // GEMM output still to be added into the residual stream
+    // output of the previous MLP projection, still to be added into the residual stream: bf16 rows or split partials
+    const bf16_t* pending_add = nullptr;
+    NcPartialSrc pending_parts = NO_PARTIALS;
+    auto mix = [&](const float* rl, const float* xl, const float* bl, const bf16_t* bsrc, bf16_t* save, uint32_t* amax) -> int {
+        if (pending_parts.parts) return nc_launch_mix_norm_p(w.x, pending_parts, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
+        return nc_launch_mix_norm(w.x, pending_add, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
+    };
     for (int i = 0; i < L; i++) {
         const nc_layer_desc& ly = m->layers[i];
         NC_CHECK_ARG(ly.w_qkv && ly.inv_qkv && ly.w_attn_proj && ly.w_fc && ly.w_mlp_proj, "gpt_forward: layer %d has no FP8 weights", i);
         // x += mlp_out(prev layer); [save backout]; x = rl*x + xl*x0; xn = norm(x)
         bf16_t* save = (i > 0 && (i - 1) == L / 2) ? w.xb : nullptr;
-        TRY(nc_launch_mix_norm(w.x, pending_add, w.x0, m->resid_lambdas + i, m->x0_lambdas + i, nullptr, nullptr, save, w.xn, M, E,
-                               w.amax + site, s));
+        TRY(mix(m->resid_lambdas + i, m->x0_lambdas + i, nullptr, nullptr, save, w.amax + site));
         // q|k|v = FP8 linear(xn): one activation quantization, three weight scales
         NcGemmSegs qkv_segs{3, {H * 128, (H + Hkv) * 128, qkv_w, 0}};
-        TRY(lin.run(w.xn, M, site, ly.w_qkv, ly.inv_qkv, qkv_segs, w.qkv, 0, 0.f, nullptr, qkv_w, E, qkv_w));
+        NcPartialSrc qsrc;
+        TRY(lin.run(w.xn, M, site, ly.w_qkv, ly.inv_qkv, qkv_segs, w.qkv, 0, 0.f, nullptr, qkv_w, E, qkv_w, &qsrc));
         site++;
         bf16_t* kc = kv->k_cache + (size_t)i * layer_elems;
         bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
-        TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
-                                      kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
+        if (qsrc.parts)
+            TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len, kv->cache_seqlens,
+                                            kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
+        else
+            TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
+                                          kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
         TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
                                 w.attn_counters, w.attn_parts, w.attn_part_bytes, w.amax + site, 0, 1, s));
-        TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E));
+        TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E, &pending_parts));
+        pending_add = pending_parts.parts ? nullptr : w.o;
         site++;
         // x += attn_out; xn = norm(x)
-        TRY(nc_launch_mix_norm(w.x, w.o, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, w.xn, M, E, w.amax + site, s));
+        TRY(mix(nullptr, nullptr, nullptr, nullptr, nullptr, w.amax + site));
         // h2 = relu(c_fc(xn))^2 with its amax in the next slot
-        TRY(lin.run(w.xn, M, site, ly.w_fc, ly.inv_fc, one_seg(4 * E), w.h2, 2, 0.f, w.amax + site + 1, 4 * E, E, 4 * E));
+        TRY(lin.run(w.xn, M, site, ly.w_fc, ly.inv_fc, one_seg(4 * E), w.h2, 2, 0.f, w.amax + site + 1, 4 * E, E, 4 * E, nullptr));
         site++;
-        TRY(lin.run(w.h2, M, site, ly.w_mlp_proj, ly.inv_mlp_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, 4 * E, E));
+        TRY(lin.run(w.h2, M, site, ly.w_mlp_proj, ly.inv_mlp_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, 4 * E, E, &pending_parts));
+        pending_add = pending_parts.parts ? nullptr : w.o;
         site++;
-        pending_add = w.o;
     }
     // x += mlp_out(last layer); x -= backout_lambda * x_backout; xn = norm(x)      (gpt.py:506-508)
     {
         const bool last_is_backout = (L - 1) == L / 2;     // L == 1 or 2
         if (last_is_backout) {
             // the saved rows and the subtraction need the same x1: do the add first, then the backout pass
-            TRY(nc_launch_mix_norm(w.x, pending_add, nullptr, nullptr, nullptr, nullptr, nullptr, w.xb, w.xn, M, E, nullptr, s));
+            TRY(mix(nullptr, nullptr, nullptr, nullptr, w.xb, nullptr));
             pending_add = nullptr;
+            pending_parts = NO_PARTIALS;
         }
-        TRY(nc_launch_mix_norm(w.x, pending_add, nullptr, nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.xn, M, E,
-                               w.amax + site, s));
+        TRY(mix(nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.amax + site));
     }
     // lm_head.  Its activation scale is tensorwise over all M rows (that is what the reference quantizes),
     // even when only the last position of every row is projected.
@@ -214,6 +238,6 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         head_rows = B;
     }
     TRY(lin.run(head_in, head_rows, site, m->w_lm_head, m->inv_lm_head, one_seg(m->vocab_size), logits_out, 1, m->softcap, nullptr,
-                m->vocab_size, E, m->vocab_size));
+                m->vocab_size, E, m->vocab_size, nullptr));
     return 0;
 }

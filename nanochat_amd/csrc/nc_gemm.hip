@@ -202,10 +202,17 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
-        uint32_t* counters = workspace_bytes > NC_GEMM_COUNTER_BYTES ? (uint32_t*)workspace : nullptr;
-        void* parts = counters ? (uint8_t*)workspace + NC_GEMM_COUNTER_BYTES : nullptr;
-        return nc_launch_gemm_decode(a, 0, nullptr, inv_a, b, inv_b, segs, out, out_kind, softcap, nullptr, M, N, K, ldc, counters,
-                                     parts, counters ? workspace_bytes - NC_GEMM_COUNTER_BYTES : 0, 0, s);
+        // split-K when the caller brought room for the partial sums, finished by a second small kernel
+        int ks = nc_gemm_decode_splits(N, K);
+        if (ks > 1 && (!workspace || workspace_bytes < (size_t)ks * M * N * sizeof(float))) ks = 1;
+        int used = 1;
+        rc = nc_launch_gemm_decode(a, 0, nullptr, inv_a, b, inv_b, segs, out, out_kind, softcap, nullptr, M, N, K, ldc, (float*)workspace,
+                                   workspace_bytes, ks, &used, s);
+        if (rc) return rc;
+        if (used > 1)
+            return nc_launch_finish_partials((const float*)workspace, used, nullptr, inv_a, inv_b, segs, out, out_kind, softcap, nullptr, M,
+                                             N, ldc, s);
+        return 0;
     } else if (which == 2) rc = launch_tile<256, 256>(a, b, ep, M, N, K, s);
     else if (which == 3) rc = launch_tile<256, 128>(a, b, ep, M, N, K, s);
     else if (which == 4) rc = launch_tile<128, 128>(a, b, ep, M, N, K, s);

@@ -10,9 +10,11 @@
 // quantized to e4m3 on the way into LDS (scale = fp32(448/max(fp64(amax),1e-12)), saturate, RNE), so the
 // separate convert pass of the quantizer disappears.
 //
-// Split-K partial sums are written to a workspace; the workgroup that arrives last at a per-column-block
-// counter adds them in split order (so the result does not depend on arrival order), applies the scales
-// and the epilogue, and resets the counter.
+// A dependent trip to memory costs a couple of microseconds here, which is more than the arithmetic of one of
+// these GEMMs, so the kernel is built to make exactly one: all loads of a workgroup's K range are issued
+// at once, and with split-K the raw fp32 partial tiles are simply stored ([split][M][N]) -- the kernel that
+// consumes the linear's output (residual/norm, rotary/append, or nc_finish_partials) adds the splits in a
+// fixed order, applies inv_a * inv_w and rounds to bf16 while it reads them, which it had to read anyway.
 //
 // Epilogues: 0 bf16;  1 fp32 softcap*tanh(bf16(v)/softcap) (lm_head, nanochat/gpt.py:512-515);
 //            2 bf16 relu(bf16(v))^2 plus atomic amax of the result (MLP activation, gpt.py:139).
@@ -33,8 +35,7 @@ struct DecodeGemmArgs {
     float softcap;
     int ldc;
     uint32_t* out_amax;       // out_kind 2
-    float4* partials;
-    uint32_t* counters;
+    float* partial_out;       // ksplits > 1: [ksplits][M][N] raw fp32 sums
     int ksplits, ksteps_per_split;
     int M, N, K;
 };
@@ -53,7 +54,6 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
     constexpr int A_CH = ROWS * 32 / 256;          // 16-byte LDS chunks per thread per 512-wide sub-chunk
     __shared__ __align__(16) uint8_t lds[2][ROWS * 512];
     __shared__ float red[4];
-    __shared__ int last_flag;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int frow = lane & 15, kb = lane >> 4;
@@ -111,8 +111,9 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
                 uint32_t o[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    o[j] = e4m3_pack4_hw(clamp448(bf16_lo(w[2 * j]) * scale), clamp448(bf16_hi(w[2 * j]) * scale),
-                                         clamp448(bf16_lo(w[2 * j + 1]) * scale), clamp448(bf16_hi(w[2 * j + 1]) * scale));
+                    // no clamp needed: |x| <= amax gives |x*scale| <= 448*(1+2^-23), which rounds to 448 like the clamped value
+                    o[j] = e4m3_pack4_hw(bf16_lo(w[2 * j]) * scale, bf16_hi(w[2 * j]) * scale, bf16_lo(w[2 * j + 1]) * scale,
+                                         bf16_hi(w[2 * j + 1]) * scale);
                 v = make_uint4(o[0], o[1], o[2], o[3]);
             } else {
                 v = ra[c][0];
@@ -133,73 +134,63 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
 
     const int nsub = (ks_end - ks_begin + 3) >> 2;
     const int kbase = ks_begin << 7;
-    if (nsub > 0) {
-        load_b(kbase, 0);
-        load_a(kbase);
-        store_a(0);
-    }
-    __syncthreads();
+    auto compute = [&](int s, int buf, int slot) {
+        const int nk = min(4, ks_end - ks_begin - 4 * s);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            if (kk < nk) {
+                v8i bf;
+                const uint4 lo = rb[slot][kk][0], hi = rb[slot][kk][1];
+                bf[0] = lo.x, bf[1] = lo.y, bf[2] = lo.z, bf[3] = lo.w, bf[4] = hi.x, bf[5] = hi.y, bf[6] = hi.z, bf[7] = hi.w;
+#pragma unroll
+                for (int i = 0; i < MB; i++) {
+                    const int row = i * 16 + frow;
+                    const int c0 = kk * 8 + 2 * kb;
+                    const uint4 alo = *(const uint4*)(&lds[buf][row * 512 + ((c0 ^ (row & 15)) << 4)]);
+                    const uint4 ahi = *(const uint4*)(&lds[buf][row * 512 + (((c0 + 1) ^ (row & 15)) << 4)]);
+                    v8i af;
+                    af[0] = alo.x, af[1] = alo.y, af[2] = alo.z, af[3] = alo.w, af[4] = ahi.x, af[5] = ahi.y, af[6] = ahi.z, af[7] = ahi.w;
+                    acc[i] = MFMA_F8(acc[i], bf, af);
+                }
+            }
+        }
+    };
+    {
+        if (nsub > 0) {
+            load_b(kbase, 0);
+            load_a(kbase);
+            store_a(0);
+        }
+        __syncthreads();
 #pragma unroll 1
-    for (int sc = 0; sc < nsub; sc += 2) {
+        for (int sc = 0; sc < nsub; sc += 2) {
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int s = sc + half;
-            if (s < nsub) {
-                const bool more = s + 1 < nsub;
-                if (more) {
-                    load_b(kbase + (s + 1) * 512, half ^ 1);
-                    load_a(kbase + (s + 1) * 512);
-                }
-                const int nk = min(4, ks_end - ks_begin - 4 * s);
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) {
-                    if (kk < nk) {
-                        v8i bf;
-                        const uint4 lo = rb[half][kk][0], hi = rb[half][kk][1];
-                        bf[0] = lo.x, bf[1] = lo.y, bf[2] = lo.z, bf[3] = lo.w, bf[4] = hi.x, bf[5] = hi.y, bf[6] = hi.z, bf[7] = hi.w;
-#pragma unroll
-                        for (int i = 0; i < MB; i++) {
-                            const int row = i * 16 + frow;
-                            const int c0 = kk * 8 + 2 * kb;
-                            const uint4 alo = *(const uint4*)(&lds[half][row * 512 + ((c0 ^ (row & 15)) << 4)]);
-                            const uint4 ahi = *(const uint4*)(&lds[half][row * 512 + (((c0 + 1) ^ (row & 15)) << 4)]);
-                            v8i af;
-                            af[0] = alo.x, af[1] = alo.y, af[2] = alo.z, af[3] = alo.w, af[4] = ahi.x, af[5] = ahi.y, af[6] = ahi.z, af[7] = ahi.w;
-                            acc[i] = MFMA_F8(acc[i], bf, af);
-                        }
+            for (int half = 0; half < 2; half++) {
+                const int s = sc + half;
+                if (s < nsub) {
+                    const bool more = s + 1 < nsub;
+                    if (more) {
+                        load_b(kbase + (s + 1) * 512, half ^ 1);
+                        load_a(kbase + (s + 1) * 512);
                     }
+                    compute(s, half, half);
+                    if (more) store_a(half ^ 1);
+                    __syncthreads();
                 }
-                if (more) store_a(half ^ 1);
-                __syncthreads();
             }
         }
     }
 
-    // ---- split-K: publish the partial tile; the last workgroup to arrive adds them up in split order
+    // ---- split-K: store the raw partial tile; the consumer adds the splits
     if (g.ksplits > 1) {
-        float4* mine = g.partials + ((size_t)(nblk * g.ksplits + split) * MB) * 256 + tid;
+        const int n = n0 + 4 * kb;
 #pragma unroll
-        for (int i = 0; i < MB; i++) mine[i * 256] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
-        __threadfence();
-        __syncthreads();
-        if (tid == 0) {
-            const uint32_t old = __hip_atomic_fetch_add(&g.counters[nblk], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            last_flag = (old == (uint32_t)(g.ksplits - 1));
+        for (int i = 0; i < MB; i++) {
+            const int m = i * 16 + frow;
+            if (m < M && n < N)
+                *(float4*)(g.partial_out + ((size_t)split * M + m) * N + n) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
         }
-        __syncthreads();
-        if (!last_flag) return;
-        __threadfence();
-#pragma unroll
-        for (int i = 0; i < MB; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < g.ksplits; s++) {
-            const float4* theirs = g.partials + ((size_t)(nblk * g.ksplits + s) * MB) * 256 + tid;
-#pragma unroll
-            for (int i = 0; i < MB; i++) {
-                const float4 p = theirs[i * 256];
-                acc[i][0] += p.x, acc[i][1] += p.y, acc[i][2] += p.z, acc[i][3] += p.w;
-            }
-        }
-        if (tid == 0) __hip_atomic_store(&g.counters[nblk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
     }
 
     // ---- epilogue: lane holds rows i*16 + frow, columns n0 + 4*kb .. +3
@@ -244,59 +235,130 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------------
-static void plan_decode(int N, int K, int force_ksplits, int& ksplits, int& kps) {
+// out = epilogue((sum over splits of partials) * inv_a * inv_w[segment]) -- the finishing pass for callers that
+// need the linear's output materialised (the MLP activation, and the stand-alone API).
+__global__ __launch_bounds__(256) void finish_partials_kernel(const float* __restrict__ parts, int nsplit, size_t split_stride,
+                                                              const uint32_t* __restrict__ a_amax, const float* __restrict__ inv_a_ptr,
+                                                              const float* __restrict__ inv_b,
+                                                              NcGemmSegs segs, void* __restrict__ out, int out_kind, float softcap,
+                                                              uint32_t* __restrict__ out_amax, int M, int N, int ldc) {
+    __shared__ float red[4];
+    const float inv_a = a_amax ? 1.0f / scale_from_amax(__uint_as_float(*a_amax)) : *inv_a_ptr;
+    const int n4 = N / 4;
+    float am = 0.f;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)M * n4; i += (size_t)gridDim.x * 256) {
+        const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < nsplit; s++) {
+            const float4 p = *(const float4*)(parts + (size_t)s * split_stride + (size_t)m * N + n);
+            a.x += p.x, a.y += p.y, a.z += p.z, a.w += p.w;
+        }
+        int sg = 0;
+#pragma unroll
+        for (int k = 0; k < 3; k++)
+            if (k + 1 < segs.nseg && n >= segs.end[k]) sg = k + 1;
+        const float ib = inv_b[sg];
+        float v[4] = {(a.x * inv_a) * ib, (a.y * inv_a) * ib, (a.z * inv_a) * ib, (a.w * inv_a) * ib};
+        if (out_kind == 1) {
+            float* o = (float*)out + (size_t)m * ldc + n;
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[r] = softcap * tanhf(rbf(v[r]) / softcap);
+        } else {
+            if (out_kind == 2) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float t = fmaxf(rbf(v[r]), 0.f);
+                    v[r] = rbf(t * t);
+                    am = fmaxf(am, v[r]);
+                }
+            }
+            *(uint2*)((bf16_t*)out + (size_t)m * ldc + n) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+        }
+    }
+    if (out_kind == 2 && out_amax) {
+        am = wave_max(am);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = am;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            if (am > 0.f) atomicMax(out_amax, __float_as_uint(am));
+        }
+    }
+}
+
+int nc_launch_finish_partials(const float* parts, int nsplit, const uint32_t* a_amax, const float* inv_a, const float* inv_b,
+                              NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M, int N, int ldc,
+                              hipStream_t s) {
+    NC_CHECK_ARG(parts && (a_amax || inv_a) && inv_b && out && nsplit >= 1 && N % 4 == 0, "finish_partials: bad arguments");
+    NC_CHECK_ARG(ldc >= N && out_kind >= 0 && out_kind <= 2, "finish_partials: bad output description");
+    if (out_kind != 1) NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "finish_partials: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
+    NcProfScope prof(3, 4.0 * nsplit * M * N, s);
+    int grid = (int)(((size_t)M * (N / 4) + 255) / 256);
+    if (grid > 2048) grid = 2048;
+    hipLaunchKernelGGL(finish_partials_kernel, dim3(grid), dim3(256), 0, s, parts, nsplit, (size_t)M * N, a_amax, inv_a, inv_b, segs,
+                       out, out_kind, softcap, out_amax, M, N, ldc);
+    NC_CHECK_LAUNCH("finish_partials");
+    return 0;
+}
+
+// How many K splits a [M<=128] x [N,K] linear is cut into: one 512-wide K chunk per workgroup (a single round
+// of loads) as long as that keeps the partial traffic moderate; big-N layers need fewer to fill the machine.
+// How many K splits a [M<=128] x [N,K] linear is cut into.  Measured on d26 shapes at M=64: a workgroup that
+// covers one 512-wide K chunk (a single round of loads) finishes in ~6 us, every further chunk it walks adds
+// ~3 us of exposed latency, so K is split down to one chunk per workgroup (at most 16 splits).  Only a layer
+// with hundreds of column blocks of its own (lm_head) runs unsplit with the epilogue in the GEMM.
+int nc_gemm_decode_splits(int N, int K) {
     const int nblk = (N + 63) / 64;
     const int nksteps = (K + 127) / 128;
-    // enough workgroups to give every CU a slice; at most 8 splits keeps the partial traffic near the weight bytes
-    ksplits = force_ksplits > 0 ? force_ksplits : (384 + nblk - 1) / nblk;
-    if (ksplits > 8 && force_ksplits <= 0) ksplits = 8;
-    if (ksplits > nksteps) ksplits = nksteps;
-    kps = (nksteps + ksplits - 1) / ksplits;
-    ksplits = (nksteps + kps - 1) / kps;
+    if (N % 4 != 0 || nblk >= 256) return 1;
+    int ks = (nksteps + 3) / 4;
+    if (ks > 16) ks = 16;
+    if (ks < 1) ks = 1;
+    const int kps = (nksteps + ks - 1) / ks;
+    return (nksteps + kps - 1) / kps;
 }
 
-// Split-K scratch: NC_GEMM_COUNTER_BYTES of arrival counters (one per 64-column block; zero before the first
-// use, left zero by every launch) and the partial tiles.
 size_t nc_gemm_decode_partial_bytes(int M, int N, int K) {
-    const int MB = M <= 64 ? 4 : 8;
-    const size_t nblk = (N + 63) / 64;
-    int ksplits, kps;
-    plan_decode(N, K, 0, ksplits, kps);
-    return ksplits > 1 ? nblk * ksplits * MB * 256 * sizeof(float4) : 0;
+    const int ks = nc_gemm_decode_splits(N, K);
+    return ks > 1 ? (size_t)ks * M * N * sizeof(float) : 0;
 }
 
+// ksplits: 0 = nc_gemm_decode_splits().  With more than one split the result is left in `partials`
+// ([ksplits][M][N] fp32, raw sums) and *ksplits_out says how many; out/out_kind are then unused.
 int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
                           const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
-                          int N, int K, int ldc, uint32_t* counters, void* partials, size_t partial_bytes, int force_ksplits,
-                          hipStream_t s) {
-    NC_CHECK_ARG(a && b && inv_b && out, "fp8_gemm(decode): null pointer");
+                          int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s) {
+    NC_CHECK_ARG(a && b, "fp8_gemm(decode): null pointer");
     NC_CHECK_ARG(a_is_bf16 ? (a_amax != nullptr) : (inv_a != nullptr), "fp8_gemm(decode): activation scale missing");
     NC_CHECK_ARG(M >= 1 && M <= 128 && N > 0 && K > 0, "fp8_gemm(decode): bad shape M=%d N=%d K=%d (M <= 128)", M, N, K);
     NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
-    NC_CHECK_ARG(ldc >= N, "fp8_gemm: ldc=%d < N=%d", ldc, N);
     NC_CHECK_ARG(((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0, "fp8_gemm: operands must be 16-byte aligned");
-    NC_CHECK_ARG(out_kind >= 0 && out_kind <= 2, "fp8_gemm: out_kind must be 0, 1 or 2");
-    NC_CHECK_ARG(segs.nseg >= 1 && segs.nseg <= 4 && segs.end[segs.nseg - 1] == N, "fp8_gemm: bad column segments");
-    for (int i = 0; i + 1 < segs.nseg; i++)
-        NC_CHECK_ARG(segs.end[i] % 4 == 0 && segs.end[i] < segs.end[i + 1], "fp8_gemm: segment ends must be increasing multiples of 4");
-    if (out_kind != 1) NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "fp8_gemm: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
+    const int nksteps = (K + 127) / 128;
+    if (ksplits <= 0) ksplits = nc_gemm_decode_splits(N, K);
+    if (ksplits > nksteps) ksplits = nksteps;
+    int kps = (nksteps + ksplits - 1) / ksplits;
+    ksplits = (nksteps + kps - 1) / kps;
+    if (ksplits > 1) {
+        NC_CHECK_ARG(N % 4 == 0, "fp8_gemm(decode): split-K needs N %% 4 == 0");
+        NC_CHECK_ARG(partials && partial_bytes >= (size_t)ksplits * M * N * sizeof(float) && ((uintptr_t)partials & 15) == 0,
+                     "fp8_gemm(decode): %d splits need %zu bytes of 16-byte aligned partial-sum workspace", ksplits,
+                     (size_t)ksplits * M * N * sizeof(float));
+    } else {
+        NC_CHECK_ARG(out && inv_b, "fp8_gemm(decode): null output");
+        NC_CHECK_ARG(ldc >= N, "fp8_gemm: ldc=%d < N=%d", ldc, N);
+        NC_CHECK_ARG(out_kind >= 0 && out_kind <= 2, "fp8_gemm: out_kind must be 0, 1 or 2");
+        NC_CHECK_ARG(segs.nseg >= 1 && segs.nseg <= 4 && segs.end[segs.nseg - 1] == N, "fp8_gemm: bad column segments");
+        for (int i = 0; i + 1 < segs.nseg; i++)
+            NC_CHECK_ARG(segs.end[i] % 4 == 0 && segs.end[i] < segs.end[i + 1], "fp8_gemm: segment ends must be increasing multiples of 4");
+        if (out_kind != 1) NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "fp8_gemm: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
+    }
+    if (ksplits_out) *ksplits_out = ksplits;
 
     const int MB = M <= 64 ? 4 : 8;
     const int nblk = (N + 63) / 64;
-    const int nksteps = (K + 127) / 128;
-    int ksplits, kps;
-    plan_decode(N, K, force_ksplits, ksplits, kps);
-    const size_t need = (size_t)nblk * ksplits * MB * 256 * sizeof(float4);
-    if (ksplits > 1 && (!counters || !partials || partial_bytes < need || nblk > NC_GEMM_COUNTER_BYTES / 4)) {
-        if (force_ksplits > 1) NC_FAIL(-1, "fp8_gemm(decode): %d splits need %zu bytes of partial-sum workspace", ksplits, need);
-        ksplits = 1;
-        kps = nksteps;
-    }
     DecodeGemmArgs g;
     g.A = a, g.a_amax = a_amax, g.inv_a = inv_a, g.B = b, g.inv_b = inv_b, g.segs = segs, g.out = out, g.out_kind = out_kind;
-    g.softcap = softcap, g.ldc = ldc, g.out_amax = out_amax;
-    g.counters = counters;
-    g.partials = (float4*)partials;
+    g.softcap = softcap, g.ldc = ldc, g.out_amax = out_amax, g.partial_out = partials;
     g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
     NcProfScope prof(1, 2.0 * M * N * K, s);
     dim3 grid(nblk, ksplits), block(256);

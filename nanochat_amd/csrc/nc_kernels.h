@@ -25,13 +25,28 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
                    size_t workspace_bytes, hipStream_t s);
 
 // small-M path (nc_gemm_decode.hip): A is e4m3 (+inv_a) or bf16 (+amax, quantized inside the kernel)
-// out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax
-#define NC_GEMM_COUNTER_BYTES 4096
+// out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax.
+// With K split over workgroups the raw fp32 sums land in `partials` [ksplits][M][N] and a consumer finishes them.
+int nc_gemm_decode_splits(int N, int K);
 size_t nc_gemm_decode_partial_bytes(int M, int N, int K);
 int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
                           const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
-                          int N, int K, int ldc, uint32_t* counters, void* partials, size_t partial_bytes, int force_ksplits,
-                          hipStream_t s);
+                          int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s);
+int nc_launch_finish_partials(const float* parts, int nsplit, const uint32_t* a_amax, const float* inv_a, const float* inv_b,
+                              NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M, int N, int ldc,
+                              hipStream_t s);
+
+// An FP8 linear's output that still sits in split partials: value(row, col) =
+// bf16((sum_s parts[s*split_stride + row*ld + col]) * inv_a * inv_b[segment(col)]), inv_a = 1/scale(amax).
+struct NcPartialSrc {
+    const float* parts;       // nullptr: not used
+    int nsplit;
+    int ld;
+    size_t split_stride;
+    const uint32_t* a_amax;
+    const float* inv_b;       // one per segment
+    int seg_end0, seg_end1;   // column ends of segments 0 and 1 (INT_MAX when there is a single segment)
+};
 
 // ---- elementwise / norm / rope (nc_elementwise.hip)
 int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s);
@@ -41,7 +56,15 @@ int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const floa
 int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
                        const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
                        int rows, int cols, uint32_t* amax_ws, hipStream_t s);
+// same, with the added tensor given as split partials of the linear that produced it (decode path)
+int nc_launch_mix_norm_p(bf16_t* x, NcPartialSrc add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
+                         const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
+                         int rows, int cols, uint32_t* amax_ws, hipStream_t s);
 int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, hipStream_t s);
+int nc_launch_qkv_rope_append_p(NcPartialSrc qkv_parts, const bf16_t* xn, int ld_xn, const int64_t* idx,
+                                const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,
+                                int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,
+                                int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s);
 int nc_launch_qkv_rope_append(const bf16_t* qkv, int ld_qkv, const bf16_t* xn, int ld_xn, const int64_t* idx,
                               const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,
                               int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,

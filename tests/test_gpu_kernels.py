@@ -226,6 +226,51 @@ def test_fused_small_m_linear(ops, M, N, K, ksplits):
     assert am.view(torch.float32).item() == want_h2.float().max().item()
 
 
+def test_split_hand_off_never_reads_stale_partials(ops):
+    """The split-K GEMM and the split attention pass partial results between workgroups through a scratch
+    buffer that is reused by every call.  Alternate two different inputs many times: a stale partial from
+    the previous call would show up as a gross error."""
+    say("split hand-off stress: GEMM")
+    M, N, K = 64, 1664, 6656
+    cases = []
+    for seed in (1, 2):
+        a, w = make_operands(M, N, K, seed=seed)
+        a = a * (1.0 if seed == 1 else -3.0)
+        a8, ia, _ = fp8_ref.to_fp8(a)
+        w8, iw, _ = fp8_ref.to_fp8(w)
+        cases.append((a.to(DEV), ops.amax_bits(a.to(DEV)), w8.to(DEV), iw.reshape(1).to(DEV),
+                      fp8_ref.scaled_mm_emulated(a8, w8, ia, iw).to(DEV)))
+    first = [None, None]
+    for it in range(300):
+        ad, bits, w8d, iwd, want = cases[it % 2]
+        got = ops.fp8_linear_small_m(ad, bits, w8d, iwd)
+        if first[it % 2] is None:
+            first[it % 2] = got.clone()
+            assert rel_l2(got.cpu(), want.cpu()) < 2e-3
+        else:
+            assert torch.equal(got, first[it % 2]), f"iteration {it}"
+    say("split hand-off stress: attention")
+    g = torch.Generator().manual_seed(3)
+    B, H, Tmax = 16, 13, 1024
+    acases = []
+    for seed in (0, 1):
+        kc = torch.randn(B, Tmax, H, 128, generator=g).bfloat16().to(DEV)
+        vc = torch.randn(B, Tmax, H, 128, generator=g).bfloat16().to(DEV)
+        q = torch.randn(B, 1, H, 128, generator=g).bfloat16().to(DEV)
+        seq = torch.randint(200, Tmax - 1, (B,), generator=g).int().to(DEV)
+        ref1 = ops.decode_attention(q, kc, vc, seq, splits=1)
+        acases.append((q, kc, vc, seq, ref1))
+    afirst = [None, None]
+    for it in range(300):
+        q, kc, vc, seq, ref1 = acases[it % 2]
+        got = ops.decode_attention(q, kc, vc, seq, splits=8)
+        if afirst[it % 2] is None:
+            afirst[it % 2] = got.clone()
+            assert torch.allclose(got.float(), ref1.float(), atol=1e-2, rtol=1e-2)
+        else:
+            assert torch.equal(got, afirst[it % 2]), f"iteration {it}"
+
+
 @pytest.mark.parametrize("K,N", [(1664, 4992), (1664, 1664), (1664, 6656), (6656, 1664)])
 def test_gemm_full_float8linear_shapes(ops, K, N):
     """The isolated Float8Linear forward at M=8192: quantize + GEMM on the GPU; the oracle checks
