@@ -14,6 +14,8 @@
 #include "nc_common.h"
 #include "nc_kernels.h"
 
+// 16-byte chunk c of LDS row r is kept at chunk slot c ^ NC_SWZ(r) by the buffer-load kernels
+#define NC_SWZ(row) (((row) >> 1) & 7)
 #define MFMA_F8(acc, b, a) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4((b), (a), (acc), 0, 0, 0, 0, 0, 0)
 
 struct EpilogueArgs {
@@ -55,9 +57,27 @@ __device__ __forceinline__ void store4(const EpilogueArgs& e, float inv_a, v4f a
     }
 }
 
+// Tile order.  Workgroups are dealt to the 8 XCDs round robin (workgroup id % 8) and each XCD has its own 4 MB L2,
+// so (1) every XCD gets a contiguous run of the tile sequence, and (2) the sequence walks the tile grid in bands of
+// GROUP_M tile rows, column by column inside a band: the ~64 tiles an XCD works on at one time then cover about
+// GROUP_M rows x 8 columns and share GROUP_M A panels and 8 B panels (a few MB) instead of streaming all of B
+// past one A panel.
+#define NC_GROUP_M 8
+__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int ntiles = tiles_m * tiles_n;
+    const int per = ntiles / 8, rem = ntiles % 8;
+    const int xcd = wg % 8, local = wg / 8;
+    const int seq = xcd * per + (xcd < rem ? xcd : rem) + local;
+    const int band_tiles = NC_GROUP_M * tiles_n;
+    const int band = seq / band_tiles, in_band = seq % band_tiles;
+    const int rows_here = min(NC_GROUP_M, tiles_m - band * NC_GROUP_M);
+    tm = band * NC_GROUP_M + in_band % rows_here;
+    tn = in_band / rows_here;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Tile kernel.  LDS rows are 128 bytes (one K step); 16-byte chunk c of row r lives at chunk slot
-// c ^ ((r >> 1) & 7), which makes both the row-major fills and the per-lane fragment reads conflict free.
+// c ^ (r & 7), which makes both the row-major fills and the per-lane fragment reads conflict free.
 template <int BM, int BN>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         EpilogueArgs ep, int M, int N, int K, int tiles_m, int tiles_n) {
@@ -67,16 +87,9 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const uint8_t* __restric
     auto tile_a = [&](int buf) -> uint8_t* { return lds + buf * (BM + BN) * 128; };
     auto tile_b = [&](int buf) -> uint8_t* { return lds + buf * (BM + BN) * 128 + BM * 128; };
 
-    // Workgroups are handed to the 8 XCDs round robin; give each XCD a contiguous run of tiles (N fastest)
-    // so the A row panels and the B panel it touches stay in that XCD's L2.
-    const int ntiles = tiles_m * tiles_n;
-    int pid = blockIdx.x;
-    {
-        const int per = ntiles / 8, rem = ntiles % 8;
-        const int xcd = pid % 8, local = pid / 8;
-        pid = xcd * per + (xcd < rem ? xcd : rem) + local;
-    }
-    const int m0 = (pid / tiles_n) * BM, n0 = (pid % tiles_n) * BN;
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -107,16 +120,16 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const uint8_t* __restric
 #pragma unroll
         for (int c = 0; c < A_CH; c++) {
             const int id = tid + c * 256, row = id >> 3, ch = id & 7;
-            *(uint4*)(tile_a(buf) + row * 128 + ((ch ^ ((row >> 1) & 7)) << 4)) = ra[c];
+            *(uint4*)(tile_a(buf) + row * 128 + ((ch ^ (row & 7)) << 4)) = ra[c];
         }
 #pragma unroll
         for (int c = 0; c < B_CH; c++) {
             const int id = tid + c * 256, row = id >> 3, ch = id & 7;
-            *(uint4*)(tile_b(buf) + row * 128 + ((ch ^ ((row >> 1) & 7)) << 4)) = rb[c];
+            *(uint4*)(tile_b(buf) + row * 128 + ((ch ^ (row & 7)) << 4)) = rb[c];
         }
     };
     auto read_frag = [&](const uint8_t* base, int row) -> v8i {
-        const int sw = (row >> 1) & 7;
+        const int sw = row & 7;
         const uint4 lo = *(const uint4*)(base + row * 128 + (((2 * kb) ^ sw) << 4));
         const uint4 hi = *(const uint4*)(base + row * 128 + (((2 * kb + 1) ^ sw) << 4));
         v8i f;
@@ -154,6 +167,181 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const uint8_t* __restric
             store4(ep, inv_a, acc[i][j], m, n, M, N);
         }
 }
+
+// ------------------------------------------------------------------------------------------------
+// Buffer-load tile kernel: the same tiling, LDS layout and MFMA mapping as gemm_tile_kernel, with a main
+// loop free of branches.  Global reads go through buffer descriptors, whose hardware range check returns
+// zeros for rows past M / N and for the K tail, so no load sits under a lane mask and the loads of K-steps
+// k+2 and k+3 stay in flight (two register stages) while step k is computed; the waits the compiler places
+// then count outstanding loads instead of draining them.  Waves form a WGM x WGN grid over the BM x BN tile.
+#define NC_BUF_OOB 0x80000000u
+// Accumulate in place: tying the result to the accumulator operand keeps every 16x16 tile in the same four
+// accumulation registers for the whole K loop (the builtin lets the register allocator pick a different result
+// tuple, which it repairs with dozens of register copies per K-step once the loop is unrolled).
+__device__ __forceinline__ void mfma_f8_acc(v4f& acc, const v8i& b, const v8i& a) {
+    asm("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+template <int BM, int BN, int WGM, int WGN, int OUT_KIND>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                                 EpilogueArgs ep, int M, int N, int K, int tiles_m, int tiles_n) {
+    constexpr int NT = 64 * WGM * WGN;
+    constexpr int WTM = BM / WGM / 16, WTN = BN / WGN / 16;     // 16x16 tiles per wave along M and N
+    constexpr int A_CH = BM * 8 / NT, B_CH = BN * 8 / NT;       // 16-byte pieces per thread and K-step
+    constexpr int PASS_ROWS = NT / 8;                           // tile rows covered by one piece of every thread
+    constexpr int STAGE = (BM + BN) * 128;
+    static_assert(PASS_ROWS % 16 == 0 && BM % (16 * WGM) == 0 && BN % (16 * WGN) == 0, "tile shape");
+    extern __shared__ __align__(16) uint8_t lds[];
+
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid / 64;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int frow = lane & 15, kb = lane >> 4;
+
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, M * K, 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, N * K, 0x00020000);
+
+    // this thread's pieces: chunk `ch` of rows lrow, lrow + PASS_ROWS, ...
+    const int lrow = tid >> 3, ch = tid & 7;
+    uint32_t avo[A_CH], bvo[B_CH];
+#pragma unroll
+    for (int c = 0; c < A_CH; c++) {
+        const int r = m0 + lrow + c * PASS_ROWS;
+        avo[c] = r < M ? (uint32_t)r * (uint32_t)K + ch * 16 : NC_BUF_OOB;
+    }
+#pragma unroll
+    for (int c = 0; c < B_CH; c++) {
+        const int r = n0 + lrow + c * PASS_ROWS;
+        bvo[c] = r < N ? (uint32_t)r * (uint32_t)K + ch * 16 : NC_BUF_OOB;
+    }
+    const int lw = lrow * 128 + ((ch ^ NC_SWZ(lrow)) << 4);                 // LDS fill offset of piece 0 (PASS_ROWS keeps the swizzle)
+    const int sw = NC_SWZ(frow);
+    const int rd_lo = frow * 128 + (((2 * kb) ^ sw) << 4), rd_hi = frow * 128 + (((2 * kb + 1) ^ sw) << 4);
+    const int a_rd = wm * (BM / WGM) * 128, b_rd = BM * 128 + wn * (BN / WGN) * 128;
+
+    const int ksteps = (K + 127) / 128, kfull = K / 128;
+    const bool ch_in_tail = ch * 16 >= K % 128;                            // only looked at for the partial last step
+
+    v4f acc[WTM][WTN];
+#pragma unroll
+    for (int i = 0; i < WTM; i++)
+#pragma unroll
+        for (int j = 0; j < WTN; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    v4i ra[2][A_CH], rb[2][B_CH];
+#define BL_LOAD(SLOT, T)                                                                                  \
+    do {                                                                                                  \
+        const int t__ = (T);                                                                              \
+        const bool cut__ = t__ >= ksteps || (t__ == kfull && ch_in_tail);                                 \
+        _Pragma("unroll") for (int c = 0; c < A_CH; c++)                                                  \
+            ra[SLOT][c] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, cut__ ? NC_BUF_OOB : avo[c], t__ * 128, 0); \
+        _Pragma("unroll") for (int c = 0; c < B_CH; c++)                                                  \
+            rb[SLOT][c] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, cut__ ? NC_BUF_OOB : bvo[c], t__ * 128, 0); \
+    } while (0)
+#define BL_FILL(SLOT, BUF)                                                                                \
+    do {                                                                                                  \
+        uint8_t* st__ = lds + (BUF) * STAGE + lw;                                                         \
+        _Pragma("unroll") for (int c = 0; c < A_CH; c++) *(v4i*)(st__ + c * PASS_ROWS * 128) = ra[SLOT][c]; \
+        _Pragma("unroll") for (int c = 0; c < B_CH; c++) *(v4i*)(st__ + BM * 128 + c * PASS_ROWS * 128) = rb[SLOT][c]; \
+    } while (0)
+    auto frag = [&](const uint8_t* base) -> v8i {
+        const v4i lo = *(const v4i*)(base + rd_lo);
+        const v4i hi = *(const v4i*)(base + rd_hi);
+        return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    auto compute = [&](int buf) {
+        const uint8_t* st = lds + buf * STAGE;
+        v8i af[WTM];
+#pragma unroll
+        for (int i = 0; i < WTM; i++) af[i] = frag(st + a_rd + i * 2048);
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            const v8i bf = frag(st + b_rd + j * 2048);
+#pragma unroll
+            for (int i = 0; i < WTM; i++) mfma_f8_acc(acc[i][j], bf, af[i]);
+        }
+    };
+    // Step kt computes from LDS buffer kt & 1, then moves tile kt+1 (register slot (kt+1) & 1, loaded two
+    // steps ago) into the other buffer and refills that slot with tile kt+3.
+#define BL_STEP(KT, BUF)                 \
+    do {                                 \
+        compute(BUF);                    \
+        BL_FILL((BUF) ^ 1, (BUF) ^ 1);   \
+        BL_LOAD((BUF) ^ 1, (KT) + 3);    \
+        __syncthreads();                 \
+        __builtin_amdgcn_sched_barrier(0); \
+    } while (0)
+
+    BL_LOAD(0, 0);
+    BL_LOAD(1, 1);
+    BL_FILL(0, 0);
+    BL_LOAD(0, 2);
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < ksteps; kt += 2) {
+        BL_STEP(kt, 0);
+        BL_STEP(kt + 1, 1);
+    }
+    if (kt < ksteps) compute(0);
+#undef BL_LOAD
+#undef BL_FILL
+#undef BL_STEP
+
+    // the last MFMAs must have left the pipeline before the accumulators are read (16 passes at most)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < WTM; i++)
+#pragma unroll
+        for (int j = 0; j < WTN; j++) asm volatile("" : "+a"(acc[i][j]));
+
+    // epilogue: the (at most four) per-segment weight scales are fetched once
+    const float inv_a = *ep.inv_a;
+    float sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        const int n = n0 + wn * (BN / WGN) + j * 16 + 4 * kb;
+        float inv_b = sc[0];
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            if (i + 1 < ep.segs.nseg && n >= ep.segs.end[i]) inv_b = sc[i + 1];
+#pragma unroll
+        for (int i = 0; i < WTM; i++) {
+            const int m = m0 + wm * (BM / WGM) + i * 16 + frow;
+            if (m >= M || n >= N) continue;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] = (acc[i][j][r] * inv_a) * inv_b;
+            if (OUT_KIND == 0) {
+                bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
+                if (n + 3 < N) *(uint2*)o = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                else
+                    for (int r = 0; r < 4 && n + r < N; r++) o[r] = f32_to_bf16(v[r]);
+            } else {
+                float* o = (float*)ep.out + (size_t)m * ep.ldc + n;
+                for (int r = 0; r < 4 && n + r < N; r++) o[r] = ep.softcap * tanhf(rbf(v[r]) / ep.softcap);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN>
+static int launch_bl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
+    const void* fn = ep.out_kind == 0 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    if (ep.out_kind == 0)
+        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    else
+        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    return 0;
+}
+
 
 // ------------------------------------------------------------------------------------------------
 template <int BM, int BN>
@@ -198,7 +386,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         }
     }
     int rc = 0;
-    if (which != 1) NC_CHECK_ARG(which >= 2 && which <= 4, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    if (which != 1) NC_CHECK_ARG(which >= 2 && which <= 10, "fp8_gemm: unknown kernel selector %d", force_kernel);
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
@@ -216,6 +404,12 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     } else if (which == 2) rc = launch_tile<256, 256>(a, b, ep, M, N, K, s);
     else if (which == 3) rc = launch_tile<256, 128>(a, b, ep, M, N, K, s);
     else if (which == 4) rc = launch_tile<128, 128>(a, b, ep, M, N, K, s);
+    else if (which == 5) rc = launch_bl<128, 128, 2, 2>(a, b, ep, M, N, K, s);
+    else if (which == 6) rc = launch_bl<256, 128, 2, 2>(a, b, ep, M, N, K, s);
+    else if (which == 7) rc = launch_bl<256, 256, 2, 4>(a, b, ep, M, N, K, s);
+    else if (which == 8) rc = launch_bl<128, 256, 2, 2>(a, b, ep, M, N, K, s);
+    else if (which == 9) rc = launch_bl<256, 128, 4, 2>(a, b, ep, M, N, K, s);
+    else if (which == 10) rc = launch_bl<256, 256, 4, 2>(a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");
