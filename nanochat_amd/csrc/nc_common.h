@@ -47,6 +47,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
 }
 
+// two fp32 -> packed bf16 pair with the hardware convert (round to nearest even), low half = first value
+typedef __bf16 nc_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float nc_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16_hw(float lo, float hi) {
+    const nc_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, nc_bf16x2));
+}
+
 // ---------------------------------------------------------------- e4m3fn (OCP) encode
 // |y| must already be clamped to <= 448.  Round to nearest even, subnormals down to 2^-9.
 __device__ __forceinline__ uint32_t e4m3_encode_sw(float y) {

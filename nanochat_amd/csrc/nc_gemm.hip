@@ -8,14 +8,17 @@
 // lane ends up holding four consecutive output columns of one output row, which packs into one 8-byte
 // bf16 store.
 //
-//   gemm_tile_kernel    M large (prefill, isolated Float8Linear): BMxBNx128 tiles, 4 waves in 2x2,
-//                       double-buffered swizzled LDS, global loads of step k+1 overlap the MFMAs of step k.
+//   gemm_bl_kernel      M large (prefill, isolated Float8Linear): BMxBNx128 tiles, double-buffered swizzled LDS fed
+//                       through two register stages of buffer loads, bf16 epilogue staged through LDS.
+//   gemm_tile_kernel    the same tiling with plain global loads (64-bit addressing) for operands past 2 GiB.
 //   M <= 128 (decode) is weight-bandwidth bound and handled by gemm_decode_kernel in nc_gemm_decode.hip.
 #include "nc_common.h"
 #include "nc_kernels.h"
 
-// 16-byte chunk c of LDS row r is kept at chunk slot c ^ NC_SWZ(r) by the buffer-load kernels
-#define NC_SWZ(row) (((row) >> 1) & 7)
+// 16-byte chunk c of LDS row r (128-byte rows) is kept at chunk slot c ^ NC_SWZ(r) by the buffer-load kernels.  Measured on
+// gfx950: with this mapping a fragment read (16 rows per 16 lanes, ds_read_b128) runs at the rate of a lane-linear read
+// (~215 B/clk/CU); XOR with (r & 7) alone, or with (r >> 1) & 7, runs at 60% of that.
+#define NC_SWZ(row) (((row) & 7) ^ (((row) >> 3) & 1))
 #define MFMA_F8(acc, b, a) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4((b), (a), (acc), 0, 0, 0, 0, 0, 0)
 
 struct EpilogueArgs {
@@ -168,6 +171,86 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const uint8_t* __restric
         }
 }
 
+// Epilogue of the buffer-load kernels: scale, convert and store one workgroup tile.
+template <int BM, int BN, int WGM, int WGN, int OUT_KIND>
+__device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN / 16], uint8_t* lds, const EpilogueArgs& ep, float inv_a,
+                                            const float (&sc)[4], int m0, int n0, int M, int N) {
+    constexpr int WTM = BM / WGM / 16, WTN = BN / WGN / 16;
+    constexpr int STAGE = (BM + BN) * 128;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int frow = lane & 15, kb = lane >> 4;
+    if (OUT_KIND == 0) {
+        // bf16 output goes through LDS so that every store instruction writes whole 128-byte lines: each wave parks its
+        // (BM/WGM) x (BN/WGN) block in its own LDS region (16-byte chunk c of row r at chunk c ^ (r & 7)), then reads it
+        // back with one row segment per group of LPR lanes and stores 16 bytes per lane.
+        constexpr int WROWS = BM / WGM, WCOLS = BN / WGN, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
+        static_assert(LPR % 8 == 0 && LPR <= 64 && WGM * WGN * WROWS * ROWB <= 2 * STAGE, "epilogue staging");
+        __syncthreads();                                       // every wave is done with the operand tiles
+        uint8_t* reg = lds + wave * WROWS * ROWB;
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            const int n = n0 + wn * WCOLS + j * 16 + 4 * kb;
+            float inv_b = sc[0];
+#pragma unroll
+            for (int i = 0; i < 3; i++)
+                if (i + 1 < ep.segs.nseg && n >= ep.segs.end[i]) inv_b = sc[i + 1];
+            const int chunk = 2 * j + (kb >> 1);
+#pragma unroll
+            for (int i = 0; i < WTM; i++) {
+                const int row = i * 16 + frow;
+                const v4f a4 = acc[i][j];
+                const uint2 pk = make_uint2(pack_bf16_hw((a4[0] * inv_a) * inv_b, (a4[1] * inv_a) * inv_b),
+                                            pack_bf16_hw((a4[2] * inv_a) * inv_b, (a4[3] * inv_a) * inv_b));
+                *(uint2*)(reg + row * ROWB + ((chunk ^ (row & 7)) << 4) + (kb & 1) * 8) = pk;
+            }
+        }
+        // the region is private to the wave: its own LDS writes only have to land before its reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0xc07f);                    // lgkmcnt(0)
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const bool vec16 = (ep.ldc % 8 == 0) && (((uintptr_t)ep.out & 15) == 0);
+        const int lrow_e = lane / LPR, c = lane % LPR;
+        const int n = n0 + wn * WCOLS + c * 8;
+#pragma unroll
+        for (int it = 0; it < WROWS / RPI; it++) {
+            const int row = it * RPI + lrow_e;
+            const int m = m0 + wm * WROWS + row;
+            const uint4 v = *(const uint4*)(reg + row * ROWB + ((c ^ (row & 7)) << 4));
+            if (m >= M || n >= N) continue;
+            bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
+            if (n + 8 <= N) {
+                if (vec16) *(uint4*)o = v;
+                else {
+                    *(uint2*)o = make_uint2(v.x, v.y);
+                    *(uint2*)(o + 4) = make_uint2(v.z, v.w);
+                }
+            } else {
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                for (int r = 0; r < 8 && n + r < N; r++) o[r] = (bf16_t)(w[r >> 1] >> ((r & 1) * 16));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            const int n = n0 + wn * (BN / WGN) + j * 16 + 4 * kb;
+            float inv_b = sc[0];
+#pragma unroll
+            for (int i = 0; i < 3; i++)
+                if (i + 1 < ep.segs.nseg && n >= ep.segs.end[i]) inv_b = sc[i + 1];
+#pragma unroll
+            for (int i = 0; i < WTM; i++) {
+                const int m = m0 + wm * (BM / WGM) + i * 16 + frow;
+                if (m >= M || n >= N) continue;
+                float* o = (float*)ep.out + (size_t)m * ep.ldc + n;
+                for (int r = 0; r < 4 && n + r < N; r++)
+                    o[r] = ep.softcap * tanhf(rbf((acc[i][j][r] * inv_a) * inv_b) / ep.softcap);
+            }
+        }
+    }
+    if (OUT_KIND == 0) __syncthreads();                        // the staging memory is free again
+}
+
 // ------------------------------------------------------------------------------------------------
 // Buffer-load tile kernel: the same tiling, LDS layout and MFMA mapping as gemm_tile_kernel, with a main
 // loop free of branches.  Global reads go through buffer descriptors, whose hardware range check returns
@@ -300,31 +383,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
     float sc[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
-#pragma unroll
-    for (int j = 0; j < WTN; j++) {
-        const int n = n0 + wn * (BN / WGN) + j * 16 + 4 * kb;
-        float inv_b = sc[0];
-#pragma unroll
-        for (int i = 0; i < 3; i++)
-            if (i + 1 < ep.segs.nseg && n >= ep.segs.end[i]) inv_b = sc[i + 1];
-#pragma unroll
-        for (int i = 0; i < WTM; i++) {
-            const int m = m0 + wm * (BM / WGM) + i * 16 + frow;
-            if (m >= M || n >= N) continue;
-            float v[4];
-#pragma unroll
-            for (int r = 0; r < 4; r++) v[r] = (acc[i][j][r] * inv_a) * inv_b;
-            if (OUT_KIND == 0) {
-                bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
-                if (n + 3 < N) *(uint2*)o = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
-                else
-                    for (int r = 0; r < 4 && n + r < N; r++) o[r] = f32_to_bf16(v[r]);
-            } else {
-                float* o = (float*)ep.out + (size_t)m * ep.ldc + n;
-                for (int r = 0; r < 4 && n + r < N; r++) o[r] = ep.softcap * tanhf(rbf(v[r]) / ep.softcap);
-            }
-        }
-    }
+    bl_epilogue<BM, BN, WGM, WGN, OUT_KIND>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
 template <int BM, int BN, int WGM, int WGN>
@@ -376,17 +435,23 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     if (M == 0) return 0;
     EpilogueArgs ep{inv_a, inv_b, segs, out, out_kind, softcap, ldc};
 
-    // force_kernel: 0 auto, 1 skinny, 2 tile 256x256, 3 tile 256x128, 4 tile 128x128
+    // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256
     int which = force_kernel;
     if (which == 0) {
         if (M <= 128) which = 1;
+        else if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31)) which = 4;   // past the 32-bit buffer offsets
         else {
+            // 256x256 tiles move half the bytes per flop through L2 and LDS but run one workgroup per CU: take them
+            // when their count fills whole rounds of the CUs well, else the 128x128 tiles (two workgroups per CU)
+            int dev = 0, cus = 256;
+            if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-            which = (t256 >= 512) ? 2 : (M >= 2048 ? 3 : 4);
+            const long rounds = (t256 + cus - 1) / cus;
+            which = (M >= 1024 && N >= 512 && 10 * t256 >= 8 * rounds * cus && rounds <= 2) ? 7 : 5;
         }
     }
     int rc = 0;
-    if (which != 1) NC_CHECK_ARG(which >= 2 && which <= 10, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 7, "fp8_gemm: unknown kernel selector %d", force_kernel);
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
@@ -401,15 +466,10 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             return nc_launch_finish_partials((const float*)workspace, used, nullptr, inv_a, inv_b, segs, out, out_kind, softcap, nullptr, M,
                                              N, ldc, s);
         return 0;
-    } else if (which == 2) rc = launch_tile<256, 256>(a, b, ep, M, N, K, s);
-    else if (which == 3) rc = launch_tile<256, 128>(a, b, ep, M, N, K, s);
-    else if (which == 4) rc = launch_tile<128, 128>(a, b, ep, M, N, K, s);
+    } else if (which == 4) rc = launch_tile<128, 128>(a, b, ep, M, N, K, s);
     else if (which == 5) rc = launch_bl<128, 128, 2, 2>(a, b, ep, M, N, K, s);
-    else if (which == 6) rc = launch_bl<256, 128, 2, 2>(a, b, ep, M, N, K, s);
-    else if (which == 7) rc = launch_bl<256, 256, 2, 4>(a, b, ep, M, N, K, s);
-    else if (which == 8) rc = launch_bl<128, 256, 2, 2>(a, b, ep, M, N, K, s);
-    else if (which == 9) rc = launch_bl<256, 128, 4, 2>(a, b, ep, M, N, K, s);
-    else if (which == 10) rc = launch_bl<256, 256, 4, 2>(a, b, ep, M, N, K, s);
+    else if (which == 6) rc = launch_bl<256, 128, 4, 2>(a, b, ep, M, N, K, s);
+    else if (which == 7) rc = launch_bl<256, 256, 4, 2>(a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");

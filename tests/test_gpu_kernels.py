@@ -118,10 +118,11 @@ def make_operands(M, N, K, seed, outliers=True):
 @pytest.mark.parametrize("M,N,K,kernel", [
     (1, 64, 128, 1), (16, 128, 256, 1), (33, 200, 1664, 1), (64, 1664, 1664, 1), (64, 4992, 1664, 1), (64, 1664, 6656, 1),
     (100, 320, 80, 1), (128, 256, 1280, 1),
-    (300, 320, 256, 2), (300, 320, 256, 3), (300, 320, 256, 4), (257, 144, 1664, 4), (512, 512, 80, 3), (256, 256, 128, 2),
-    (129, 64, 2048, 0), (1792, 1664, 1664, 0),
-    (300, 320, 256, 5), (300, 320, 384, 6), (300, 320, 256, 7), (300, 320, 640, 8), (513, 272, 1664, 5),
-    (300, 320, 128, 9), (300, 320, 80, 10), (300, 320, 400, 5), (513, 272, 1664, 7), (640, 528, 912, 6), (257, 144, 16, 5),
+    (300, 320, 256, 4), (257, 144, 1664, 4), (512, 512, 80, 4), (256, 256, 128, 4),
+    (129, 64, 2048, 0), (1792, 1664, 1664, 0), (2048, 1664, 400, 0),
+    (300, 320, 256, 5), (300, 320, 400, 5), (513, 272, 1664, 5), (257, 144, 16, 5), (2100, 1300, 400, 5),
+    (300, 320, 384, 6), (640, 528, 912, 6), (300, 320, 128, 6), (5000, 1100, 144, 6),
+    (300, 320, 256, 7), (300, 320, 80, 7), (513, 272, 1664, 7), (4100, 2100, 272, 7),
 ])
 def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     say(f"gemm M={M} N={N} K={K} kernel={kernel}")
@@ -139,7 +140,7 @@ def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     assert rel_l2(got, exact) < 0.08
 
 
-@pytest.mark.parametrize("kernel,M", [(1, 48), (2, 256), (3, 256), (4, 128), (5, 256), (6, 128), (7, 256), (8, 128), (9, 256), (10, 256)])
+@pytest.mark.parametrize("kernel,M", [(1, 48), (4, 128), (5, 256), (6, 128), (7, 256)])
 def test_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
     say(f"gemm exact powers of two kernel={kernel}")
     g = torch.Generator().manual_seed(9)
