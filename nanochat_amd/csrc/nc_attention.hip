@@ -215,8 +215,12 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         if (threadIdx.x == 0) __hip_atomic_store(&counters[row * Hkv + hk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (amax_ws) {
+        // one publication per workgroup (only the first G*128 threads hold output values)
         am = wave_max(am);
-        if (lane == 0 && am > 0.f) atomicMax(amax_ws, __float_as_uint(am));
+        __syncthreads();
+        if (lane == 0) merge[wave][0][0] = am;
+        __syncthreads();
+        if (threadIdx.x == 0) amax_publish(amax_ws, fmaxf(fmaxf(merge[0][0][0], merge[1][0][0]), fmaxf(merge[2][0][0], merge[3][0][0])));
     }
 }
 

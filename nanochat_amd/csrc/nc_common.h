@@ -162,6 +162,16 @@ __device__ __forceinline__ bool arrive_and_check_last(uint32_t* counter, uint32_
     return last;
 }
 
+// Max-reduce a non-negative fp32 into a device word (fp32 bit patterns of non-negative values order like integers).
+// Atomics on one address serialize at the device coherence point, so the atomic is skipped when the word already
+// holds at least this value.
+__device__ __forceinline__ void amax_publish(uint32_t* ws, float am) {
+    const uint32_t bits = __float_as_uint(am);
+    if (bits == 0u || (bits >> 31)) return;
+    if (__hip_atomic_load(ws, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
+    atomicMax(ws, bits);
+}
+
 // block-wide sum for blockDim.x == 64 * NW, result broadcast to every thread
 template <int NW>
 __device__ __forceinline__ float block_sum(float v, float* red /* >= NW floats of LDS */) {

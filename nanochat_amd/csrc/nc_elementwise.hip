@@ -25,7 +25,7 @@ __device__ __forceinline__ void block_amax_commit(float local_abs_max, uint32_t*
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int i = 1; i < nw; i++) m = fmaxf(m, red[i]);
-        atomicMax(amax_ws, __float_as_uint(m));
+        amax_publish(amax_ws, m);
     }
 }
 

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
         __syncthreads();
         if (tid == 0) {
             am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-            if (am > 0.f) atomicMax(g.out_amax, __float_as_uint(am));
+            amax_publish(g.out_amax, am);
         }
     }
 }
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
         __syncthreads();
         if (threadIdx.x == 0) {
             am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-            if (am > 0.f) atomicMax(out_amax, __float_as_uint(am));
+            amax_publish(out_amax, am);
         }
     }
 }
