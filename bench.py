@@ -202,6 +202,18 @@ def cpu_baseline(budget_s=25.0):
             "s_per_step": round(spent / steps, 3)}
 
 
+def measured_traffic():
+    """HBM bytes per attention launch from the hardware counters (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc runs of this
+    script, scaled by what the same counters read for the --copy-probe-mib pass).  The counters cannot be collected from
+    inside this process, so the figure is read from the summary committed next to the profiles; None if absent."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "attn_partial_d26_b64_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f)["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -210,6 +222,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--profile-steps", type=int, default=16)
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="after the decode steps, run an elementwise pass that reads and writes this many MiB "
+                         "(a kernel of known traffic to scale hardware byte counters with)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (decode shards by batch row; see DESIGN.md). "
@@ -222,7 +237,7 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    K, W, P = args.steps, args.warmup, args.profile_steps
+    K, W, P = args.steps, args.warmup, max(1, args.profile_steps)
     total_new = W + K + P
     prompt_len = CONTEXT - (W + K)            # the last timed step brings the context to 2048
     assert prompt_len >= 1, "steps + warmup must stay below the 2048-token context"
@@ -259,6 +274,14 @@ def main():
     prof = {c: read_profile(lib, c) for c in range(5)}
     lib.nc_profile_enable(0)
     gen.close()
+    if args.copy_probe_mib > 0:
+        n = args.copy_probe_mib * (1 << 20) // 2
+        src = torch.ones(n, dtype=torch.bfloat16, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            torch.mul(src, 1.0, out=dst)       # reads n*2 bytes, writes n*2 bytes
+        torch.cuda.synchronize()
+        del src, dst
     att_ms, _, att_n = prof[0]
     ctx_mid = CONTEXT + P // 2                 # profiled steps sit just past the timed region
     att_bytes_step = attention_bytes_per_step(model, BATCH, ctx_mid)
@@ -288,7 +311,7 @@ def main():
         "ttft_s": round(ttft, 3),
         "roofline": {"bound": "hbm", "kernel": "attn_partial_kernel (+combine) per layer launch",
                      "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK, 4), "traffic": measured_traffic(),
                      "bytes_per_launch": int(att_bytes_launch), "avg_launch_us": round(att_avg_s * 1e6, 2),
                      "launches_timed": att_n},
         "kernel_ms_per_step": per_step_ms,
