@@ -103,6 +103,15 @@ class KVCache:
         self._pos0 += num_tokens
         self._pos_max += num_tokens
 
+    def rewind(self, num_tokens, prev_embedding):
+        """Take back the last advance (the appended rows stay in the tensors and are overwritten by the next
+        append at the same positions); `prev_embedding` is the smear state from before that forward."""
+        assert 0 < num_tokens <= self._pos0
+        self.cache_seqlens -= num_tokens
+        self._pos0 -= num_tokens
+        self._pos_max -= num_tokens
+        self.prev_embedding = prev_embedding
+
     def set_seqlens(self, seqlens):
         """Ragged rows: install per-row lengths (host list or tensor)."""
         t = torch.as_tensor(seqlens, dtype=torch.int32)
@@ -231,12 +240,30 @@ class Engine:
 
         rows = [RowState(tokens.copy()) for _ in range(num_samples)]
         produced = 0
+        # On the GPU the next forward is enqueued on the sampled ids before the host has seen them: the ids travel to a
+        # pinned buffer by an async copy placed ahead of that forward, and the tool-use state machine runs while the
+        # GPU computes.  If the machine then forces a different token for some row, the step is taken back (positions
+        # and smear state) and redone with the forced column -- the outputs are those of the plain loop.
+        ahead = torch.device(device).type == "cuda" and hasattr(self.model, "forward_last")
+        if ahead:
+            host_ids = torch.empty(num_samples, dtype=torch.long, pin_memory=True)
+            ids_ready = torch.cuda.Event()
         while True:
             if max_tokens is not None and produced >= max_tokens:
                 break
             if all(r.completed for r in rows):
                 break
-            sampled = sample_next_token(logits, rng, temperature, top_k)[:, 0].tolist()
+            sampled_dev = sample_next_token(logits, rng, temperature, top_k)
+            run_ahead = ahead and not (max_tokens is not None and produced + 1 >= max_tokens)
+            if run_ahead:
+                host_ids.copy_(sampled_dev[:, 0], non_blocking=True)
+                ids_ready.record()
+                prev_before = kv_decode.prev_embedding
+                logits_ahead = self._last_logits(sampled_dev, kv_decode)
+                ids_ready.synchronize()
+                sampled = host_ids.tolist()
+            else:
+                sampled = sampled_dev[:, 0].tolist()
             column, masks = [], []
             for r, s in zip(rows, sampled):
                 tok, mask = self._step_row(r, s, sp)
@@ -244,6 +271,11 @@ class Engine:
                 masks.append(mask)
             yield column, masks
             produced += 1
+            if run_ahead and column == sampled:
+                logits = logits_ahead
+                continue
+            if run_ahead:
+                kv_decode.rewind(1, prev_before)
             ids = torch.tensor(column, dtype=torch.long, device=device).unsqueeze(1)
             logits = self._last_logits(ids, kv_decode)
 

@@ -385,6 +385,51 @@ def test_engine_generate_sampling_on_gpu(d4_pair):
     assert all(r == g1[0] for r in g1)                           # greedy rows are identical
 
 
+def test_engine_run_ahead_step_is_taken_back_when_a_token_is_forced(d4_pair):
+    """Engine.generate enqueues the next forward on the sampled ids before the host has read them.  When the tool-use
+    machine forces another token the step must be redone: a run whose rows get forced tokens at chosen steps has to
+    match the same run through a model object without the fast path (the plain sample -> host -> forward loop)."""
+    say("Engine.generate: forced tokens vs run-ahead forward")
+    rt, model = d4_pair
+    from nanochat_amd.engine import Engine
+    from test_engine_host import ByteTokenizer
+    tok = ByteTokenizer()
+    tok._special = {k: 32000 + i for i, k in enumerate(tok._special)}
+    tok.get_bos_token_id = lambda: 32005
+
+    class Forcing(Engine):                  # forces a token for row 1 at steps 2 and 3, for every row at step 6
+        def generate(self, *a, **k):
+            self._calls = 0
+            return super().generate(*a, **k)
+
+        def _step_row(self, state, sampled, sp):
+            step, row = divmod(self._calls, 4)
+            self._calls += 1
+            if (row == 1 and step in (2, 3)) or step == 6:
+                state.forced_tokens.append((sampled + 17 + row) % 30000)
+            return super()._step_row(state, sampled, sp)
+
+    class PlainModel:                       # same model, no forward_last: the engine takes the plain loop
+        def __init__(self, m):
+            self.config, self._m = m.config, m
+
+        def get_device(self):
+            return self._m.get_device()
+
+        def forward(self, ids, kv_cache=None):
+            return self._m.forward(ids, kv_cache=kv_cache)
+
+    prompt = [5, 99, 12345, 777, 31000, 42]
+    for temperature, top_k in ((0.0, None), (0.9, 40)):
+        runs = []
+        for m in (model, PlainModel(model)):
+            cols = list(Forcing(m, tok).generate(prompt, num_samples=4, max_tokens=10, temperature=temperature, top_k=top_k, seed=3))
+            runs.append(cols)
+        assert runs[0] == runs[1]
+        assert any(0 in masks for _, masks in runs[0])          # forced tokens did occur
+        assert len(runs[0]) == 10
+
+
 def test_model_refuses_what_it_does_not_implement(d4_pair):
     rt, model = d4_pair
     from nanochat_amd.gpt import GPT, GPTConfig
