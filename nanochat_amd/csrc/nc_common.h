@@ -90,6 +90,13 @@ __device__ __forceinline__ float scale_from_amax(float amax) {
     return (float)(448.0 / d);
 }
 
+// 16-byte load of data that is read once and is larger than the caches (KV cache, weights at decode time): a
+// non-temporal load is not kept on its way in; a pure streaming read measures ~15% more HBM bandwidth with it.
+__device__ __forceinline__ uint4 nt_load16(const void* p) {
+    const v4i r = __builtin_nontemporal_load((const v4i*)p);
+    return make_uint4((uint32_t)r[0], (uint32_t)r[1], (uint32_t)r[2], (uint32_t)r[3]);
+}
+
 // ---------------------------------------------------------------- wave64 reductions
 // DPP row_ror within rows of 16 lanes: all 16 lanes end with the row total.
 template <int CTRL>
