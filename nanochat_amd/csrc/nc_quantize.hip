@@ -17,9 +17,8 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, i
     const int64_t nvec = n / PER_VEC;
     const uint4* xv = (const uint4*)x;
     uint32_t m = 0;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * blockDim.x) {
-        uint4 v = xv[i];
-        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    auto take = [&](const uint4& v) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             if (IS_BF16) {
@@ -31,7 +30,15 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, i
                 m = m > a ? m : a;
             }
         }
+    };
+    // four 16-byte loads in flight per thread
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 3 * stride < nvec; i += 4 * stride) {
+        const uint4 v0 = xv[i], v1 = xv[i + stride], v2 = xv[i + 2 * stride], v3 = xv[i + 3 * stride];
+        take(v0), take(v1), take(v2), take(v3);
     }
+    for (; i < nvec; i += stride) take(xv[i]);
     // tail elements (n not a multiple of the vector width)
     if (blockIdx.x == 0) {
         for (int64_t i = nvec * PER_VEC + threadIdx.x; i < n; i += blockDim.x) {
@@ -48,7 +55,8 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, i
     if (threadIdx.x == 0) {
         uint32_t t = red[0];
         for (int i = 1; i < 4; i++) t = t > red[i] ? t : red[i];
-        atomicMax(amax_bits, t);
+        // atomics on one word serialize: skip the ones that cannot change it
+        if (t > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(amax_bits, t);
     }
 }
 
@@ -137,8 +145,8 @@ int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, floa
     nc_clear_u32(amax_ws, 1, s);
     NcProfScope prof(2, 3.0 * n, s);
     const int per_vec = x_dtype == 0 ? 8 : 4;
-    // 2048 blocks x 256 threads = 8 waves on each of 256 CUs; each block strides the tensor
-    int g1 = grid_for(n / per_vec, 256, 2048);
+    // at most 1024 blocks x 256 threads, four loads per thread and trip; every block ends with one atomic on the same word
+    int g1 = grid_for(n / per_vec, 1024, 1024);
     int g2 = grid_for(n / 16, 256, 4096);
     if (x_dtype == 0) {
         hipLaunchKernelGGL(amax_kernel<true>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
