@@ -18,17 +18,23 @@
 // HBM traffic per (row, kv head): 2 * n_keys * 256 bytes, the algorithmic minimum.
 #include "nc_common.h"
 #include "nc_kernels.h"
+#include "nc_rope.h"
 
 #define NEG_BIG (-1.0e30f)
 #define PART_STRIDE 132     // floats per partial: m, l, pad, pad, acc[128]
 
-template <int G>
-__global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
-                                                           const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
+// FUSED (decode, one new token per row, one split): the workgroup first finishes its own heads of the q|k|v linear
+// (rope_head: partial sums, rotary, QK-norm, value-embedding gate), appends the new key and value to the cache, and
+// attends to them out of LDS; the stand-alone rotary/append kernel and the q buffer drop out of the step.
+template <int G, bool FUSED>
+__global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache,
+                                                           bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
                                                            float* __restrict__ partials, uint32_t* __restrict__ counters,
-                                                           uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, int nsplit) {
+                                                           uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, int nsplit,
+                                                           NcRopeSrc rope) {
     __shared__ float merge[4][G][PART_STRIDE];
+    __shared__ float fresh[FUSED ? G + 2 : 1][128];      // FUSED: the G query heads, then the new key and value
     __shared__ int last_flag;
     const int split = blockIdx.x, hk = blockIdx.y, row = blockIdx.z;
     const int b = row / T, t = row % T;
@@ -42,7 +48,9 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     if (hi > Tmax - 1) hi = Tmax - 1;
     int lo = (window_left < 0) ? 0 : hi - window_left;
     if (lo < 0) lo = 0;
-    const int n_keys = hi - lo + 1;
+    // keys streamed from the cache: [lo, k_stop); the fused kernel takes key hi (its own token) from LDS
+    const int k_stop = FUSED ? hi : hi + 1;
+    const int n_keys = k_stop - lo;
     // contiguous runs, multiples of 4 keys, over nsplit * 4 waves
     const int nw = nsplit * 4;
     int chunk = (n_keys + nw - 1) / nw;
@@ -50,19 +58,40 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     const int gw = split * 4 + wave;
     const int k_begin = lo + gw * chunk;
     int k_end = k_begin + chunk;
-    if (k_end > hi + 1) k_end = hi + 1;
+    if (k_end > k_stop) k_end = k_stop;
+
+    if (FUSED) {
+        // wave w finishes head task w, w+4, ...: tasks 0..G-1 are the query heads, G the key head, G+1 the value head
+        for (int task = wave; task < G + 2; task += 4) {
+            const int hh = task < G ? hk * G + task : (task == G ? H + hk : H + Hkv + hk);
+            float y1, y2;
+            rope_head(rope, row, hi, hh, H, Hkv, lane, y1, y2);
+            fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
+            if (task >= G && hi >= 0 && hi < Tmax) {
+                bf16_t* dst = (task == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + hk) * 128;
+                dst[lane] = f32_to_bf16(y1);
+                dst[lane + 64] = f32_to_bf16(y2);
+            }
+        }
+        __syncthreads();
+    }
 
     // q for the G heads of this kv head, pre-scaled by log2(e) / sqrt(128)
     const float qscale = 1.4426950408889634f * 0.08838834764831845f;
     float qf[G][8];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const uint4 qv = *(const uint4*)(q + ((size_t)row * H + hk * G + g) * 128 + sub * 8);
-        const uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+        if (FUSED) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            qf[g][2 * j] = bf16_lo(w[j]) * qscale;
-            qf[g][2 * j + 1] = bf16_hi(w[j]) * qscale;
+            for (int e = 0; e < 8; e++) qf[g][e] = fresh[g][sub * 8 + e] * qscale;
+        } else {
+            const uint4 qv = *(const uint4*)(q + ((size_t)row * H + hk * G + g) * 128 + sub * 8);
+            const uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                qf[g][2 * j] = bf16_lo(w[j]) * qscale;
+                qf[g][2 * j + 1] = bf16_hi(w[j]) * qscale;
+            }
         }
     }
     float m[G], l[G], acc[G][8];
@@ -71,6 +100,21 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         m[g] = NEG_BIG, l[g] = 0.f;
 #pragma unroll
         for (int d = 0; d < 8; d++) acc[g][d] = 0.f;
+    }
+    if (FUSED) {
+        // the row's own key: the first 16 lanes of wave 0 start their running softmax from it (weight exp2(0) = 1)
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float d = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) d = fmaf(qf[g][e], fresh[G][sub * 8 + e], d);
+            d = row16_sum(d);
+            if (wave == 0 && grp == 0) {
+                m[g] = d, l[g] = 1.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[g][e] = fresh[G + 1][sub * 8 + e];
+            }
+        }
     }
 
     const size_t key_stride = (size_t)Hkv * 128;   // elements between consecutive keys
@@ -232,21 +276,32 @@ static int pick_splits(int B, int T, int Hkv, int max_keys) {
 size_t nc_attn_counter_bytes(int B, int T, int H) { return (((size_t)B * T * H * sizeof(uint32_t)) + 255) & ~(size_t)255; }
 size_t nc_attn_partial_bytes(int B, int T, int H) { return (size_t)B * T * H * 16 * PART_STRIDE * sizeof(float); }
 
-int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
+int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax) {
+    const int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
+    return pick_splits(B, T, Hkv, max_keys);
+}
+
+static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens,
                         int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                         uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
                         int counters_are_zero, hipStream_t s) {
-    NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
+    NC_CHECK_ARG((q || rope) && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
     NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0, "decode_attention: bad shape");
     NC_CHECK_ARG(H % Hkv == 0, "decode_attention: n_head %d not a multiple of n_kv_head %d", H, Hkv);
     const int G = H / Hkv;
     NC_CHECK_ARG(G == 1 || G == 2 || G == 4 || G == 8, "decode_attention: query group size %d not in {1,2,4,8}", G);
     NC_CHECK_ARG((long)B * T <= 65535 && Hkv <= 65535, "decode_attention: more than 65535 query rows in one launch");
-    NC_CHECK_ARG(((uintptr_t)q & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0,
+    NC_CHECK_ARG((!q || ((uintptr_t)q & 15) == 0) && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0,
                  "decode_attention: pointers must be 16-byte aligned");
     int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
     int nsplit = force_splits > 0 ? force_splits : pick_splits(B, T, Hkv, max_keys);
     NC_CHECK_ARG(nsplit >= 1 && nsplit <= 16, "decode_attention: splits must be 1..16");
+    if (rope) {
+        NC_CHECK_ARG(T == 1 && nsplit == 1 && !seqlens_include_new, "decode_attention: the fused q|k|v finish needs T == 1 and one split");
+        NC_CHECK_ARG((rope->qkv || rope->pq.parts) && rope->cos_t && rope->sin_t && rope->rope_len > 0, "decode_attention: rotary source missing");
+        NC_CHECK_ARG(!rope->ve_table || (rope->ve_gate_w && rope->xn && rope->idx && rope->ld_xn >= 12),
+                     "decode_attention: value embedding needs gate weights, xn and idx");
+    }
     if (nsplit > 1) {
         const size_t need = (size_t)B * T * H * nsplit * PART_STRIDE * sizeof(float);
         NC_CHECK_ARG(counters && partials && partial_bytes >= need, "decode_attention: %zu bytes of split workspace needed, %zu given",
@@ -257,9 +312,16 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
     NcProfScope prof(0, 0.0, s);
     float* parts = (float*)partials;
     dim3 grid(nsplit, Hkv, B * T), block(256);
+    const NcRopeSrc none{};
 #define LAUNCH_G(GG)                                                                                                         \
-    hipLaunchKernelGGL(attn_partial_kernel<GG>, grid, block, 0, s, q, k_cache, v_cache, cache_seqlens, window_left,             \
-                       seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit)
+    do {                                                                                                                     \
+        if (rope)                                                                                                            \
+            hipLaunchKernelGGL((attn_partial_kernel<GG, true>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,          \
+                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, *rope); \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((attn_partial_kernel<GG, false>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,         \
+                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, none);  \
+    } while (0)
     if (G == 1) LAUNCH_G(1);
     else if (G == 2) LAUNCH_G(2);
     else if (G == 4) LAUNCH_G(4);
@@ -267,4 +329,21 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
 #undef LAUNCH_G
     NC_CHECK_LAUNCH("decode_attention");
     return 0;
+}
+
+int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
+                        int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
+                        uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
+                        int counters_are_zero, hipStream_t s) {
+    return launch_attention_impl(q, nullptr, const_cast<bf16_t*>(k_cache), const_cast<bf16_t*>(v_cache), cache_seqlens, window_left, out,
+                                 B, T, H, Hkv, Tmax, seqlens_include_new, counters, partials, partial_bytes, amax_ws, force_splits,
+                                 counters_are_zero, s);
+}
+
+// Decode step, one new token per row, cache_seqlens not yet counting it: finish the q|k|v linear (rotary, QK-norm,
+// value embedding), append key and value at cache_seqlens[b], attend.  Needs nc_attn_splits(...) == 1.
+int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
+                              bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* amax_ws, hipStream_t s) {
+    return launch_attention_impl(nullptr, &rope, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, nullptr,
+                                 nullptr, 0, amax_ws, 1, 1, s);
 }

@@ -11,10 +11,7 @@
 // follows (atomicMax on the fp32 bit pattern, valid because the values are non-negative).
 #include "nc_common.h"
 #include "nc_kernels.h"
-
-#define RMS_EPS 1.1920928955078125e-07f   // fp32 machine epsilon: F.rms_norm's default eps
-
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+#include "nc_rope.h"
 
 __device__ __forceinline__ void block_amax_commit(float local_abs_max, uint32_t* amax_ws, float* red) {
     if (!amax_ws) return;
@@ -242,14 +239,9 @@ __global__ __launch_bounds__(256) void relu2_kernel(const bf16_t* __restrict__ h
 //   k heads: same -> k_cache[b, pos+t, h, :]
 //   v heads: v + 3*sigmoid(W_g . xn[:12])[h] * ve[idx, h, :] (if the layer has a value embedding) -> v_cache
 // (gpt.py:89-104, flash_attention.py:167-170)
-__global__ __launch_bounds__(256) void qkv_rope_append_kernel(const bf16_t* __restrict__ qkv, int ld_qkv, NcPartialSrc pq,
-                                                              const bf16_t* __restrict__ xn,
-                                                              int ld_xn, const int64_t* __restrict__ idx, const bf16_t* __restrict__ ve_table,
-                                                              const float* __restrict__ ve_gate_w, const bf16_t* __restrict__ cos_t,
-                                                              const bf16_t* __restrict__ sin_t, int rope_len,
-                                                              const int32_t* __restrict__ cache_seqlens, bf16_t* __restrict__ k_cache,
-                                                              bf16_t* __restrict__ v_cache, bf16_t* __restrict__ q_out, int T, int H,
-                                                              int Hkv, int Tmax, int vocab_rows, int total_waves) {
+__global__ __launch_bounds__(256) void qkv_rope_append_kernel(NcRopeSrc r, const int32_t* __restrict__ cache_seqlens,
+                                                              bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+                                                              bf16_t* __restrict__ q_out, int T, int H, int Hkv, int Tmax, int total_waves) {
     const int lane = threadIdx.x & 63;
     const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (gw >= total_waves) return;
@@ -257,64 +249,17 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(const bf16_t* __re
     const int token = gw / heads, hh = gw % heads;
     const int b = token / T, t = token % T;
     const int pos = cache_seqlens[b] + t;
-    float x1, x2;
-    if (pq.parts) {
-        // the q|k|v linear's output still sits in split partials: add them up, scale, round to bf16
-        const int col = hh * 128 + lane;
-        const float* pp = pq.parts + (size_t)token * pq.ld + col;
-        float a1 = 0.f, a2 = 0.f;
-        for (int sp = 0; sp < pq.nsplit; sp++) {
-            a1 += pp[(size_t)sp * pq.split_stride];
-            a2 += pp[(size_t)sp * pq.split_stride + 64];
-        }
-        const float inv_a = 1.0f / scale_from_amax(__uint_as_float(*pq.a_amax));
-        const float inv_b = pq.inv_b[col >= pq.seg_end1 ? 2 : (col >= pq.seg_end0 ? 1 : 0)];
-        x1 = rbf((a1 * inv_a) * inv_b);
-        x2 = rbf((a2 * inv_a) * inv_b);
-    } else {
-        const bf16_t* src = qkv + (size_t)token * ld_qkv + (size_t)hh * 128;
-        x1 = bf16_to_f32(src[lane]), x2 = bf16_to_f32(src[lane + 64]);
+    float y1, y2;
+    rope_head(r, token, pos, hh, H, Hkv, lane, y1, y2);
+    bf16_t* dst;
+    if (hh < H) dst = q_out + ((size_t)token * H + hh) * 128;
+    else {
+        if (pos < 0 || pos >= Tmax) return;
+        const bool is_k = hh < H + Hkv;
+        dst = (is_k ? k_cache : v_cache) + (((size_t)b * Tmax + pos) * Hkv + (is_k ? hh - H : hh - H - Hkv)) * 128;
     }
-    const bool in_cache = pos >= 0 && pos < Tmax;
-
-    if (hh < H + Hkv) {
-        const int rp = pos < rope_len ? (pos < 0 ? 0 : pos) : rope_len - 1;
-        const float c = bf16_to_f32(cos_t[(size_t)rp * 64 + lane]), s = bf16_to_f32(sin_t[(size_t)rp * 64 + lane]);
-        float y1 = rbf(rbf(x1 * c) + rbf(x2 * s));
-        float y2 = rbf(rbf(x1 * (-s)) + rbf(x2 * c));
-        const float ss = wave_sum(y1 * y1 + y2 * y2);
-        const float rstd = 1.0f / sqrtf(ss / 128.0f + RMS_EPS);
-        y1 = rbf(rbf(y1 * rstd) * 1.2f);
-        y2 = rbf(rbf(y2 * rstd) * 1.2f);
-        if (hh < H) {
-            bf16_t* dst = q_out + ((size_t)token * H + hh) * 128;
-            dst[lane] = f32_to_bf16(y1);
-            dst[lane + 64] = f32_to_bf16(y2);
-        } else if (in_cache) {
-            bf16_t* dst = k_cache + (((size_t)b * Tmax + pos) * Hkv + (hh - H)) * 128;
-            dst[lane] = f32_to_bf16(y1);
-            dst[lane + 64] = f32_to_bf16(y2);
-        }
-    } else {
-        const int hv = hh - H - Hkv;
-        if (ve_table) {
-            float dot = 0.f;
-            const bf16_t* xr = xn + (size_t)token * ld_xn;
-#pragma unroll
-            for (int cidx = 0; cidx < 12; cidx++) dot += bf16_to_f32(xr[cidx]) * rbf(ve_gate_w[hv * 12 + cidx]);
-            const float gate = rbf(3.0f * rbf(sigmoidf_(rbf(dot))));
-            int64_t tok = idx[token];
-            if (tok < 0 || tok >= vocab_rows) tok = 0;
-            const bf16_t* ve = ve_table + ((size_t)tok * Hkv + hv) * 128;
-            x1 = rbf(x1 + rbf(gate * bf16_to_f32(ve[lane])));
-            x2 = rbf(x2 + rbf(gate * bf16_to_f32(ve[lane + 64])));
-        }
-        if (in_cache) {
-            bf16_t* dst = v_cache + (((size_t)b * Tmax + pos) * Hkv + hv) * 128;
-            dst[lane] = f32_to_bf16(x1);
-            dst[lane + 64] = f32_to_bf16(x2);
-        }
-    }
+    dst[lane] = f32_to_bf16(y1);
+    dst[lane + 64] = f32_to_bf16(y2);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -406,8 +351,9 @@ static int launch_rope_impl(const bf16_t* qkv, int ld_qkv, NcPartialSrc pq, cons
     NC_CHECK_ARG(!ve_table || (ve_gate_w && xn && idx && ld_xn >= 12), "qkv_rope_append: value embedding needs gate weights, xn and idx");
     const int total = B * T * (H + 2 * Hkv);
     NcProfScope prof(3, 4.0 * total * 128, s);
-    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, qkv, ld_qkv, pq, xn, ld_xn, idx, ve_table,
-                       ve_gate_w, cos, sin, rope_len, cache_seqlens, k_cache, v_cache, q_out, T, H, Hkv, Tmax, vocab_rows, total);
+    const NcRopeSrc r{qkv, ld_qkv, pq, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin, rope_len, vocab_rows};
+    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, r, cache_seqlens, k_cache, v_cache, q_out, T, H,
+                       Hkv, Tmax, total);
     NC_CHECK_LAUNCH("qkv_rope_append");
     return 0;
 }

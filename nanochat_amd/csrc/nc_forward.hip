@@ -2,11 +2,14 @@
 // Python loop at nanochat/gpt.py:459-524 (and of the module calls it makes into gpt.py:84-153 and
 // fp8.py:202-213).  One call enqueues every kernel of the step; no host synchronisation, no allocation.
 //
-// Per layer, decode (M = B*T <= 128 rows), 9 launches, each making a single dependent trip to memory:
+// Per layer, decode (M = B*T <= 128 rows), 8 launches, each making a single dependent trip to memory:
 //   mix_norm            x += mlp_out(prev) [read from split partials]; x = rl*x + xl*x0; xn = norm(x); amax(xn)
 //   linear q|k|v        quantize xn inside the GEMM; K split over workgroups           -> fp32 partials
-//   qkv_rope_append     sums the partials (three weight scales), rotary, QK-norm, gain, VE gate, KV append -> q, caches
-//   attention           over the cache; amax(y)                                        -> y
+//   attention           each (row, kv head) workgroup first sums its heads' partials (three weight scales), applies
+//                       rotary, QK-norm, gain and the VE gate, appends key and value to the cache, then attends over
+//                       the cache; amax(y)                                             -> y
+//                       (small batches, where attention is split over several workgroups per head, and T > 1 keep the
+//                       stand-alone qkv_rope_append kernel in front)
 //   linear c_proj       quantize y inside                                              -> partials
 //   mix_norm            x += o [from partials]; xn = norm(x); amax(xn)
 //   linear c_fc         quantize xn inside                                             -> partials
@@ -29,6 +32,7 @@
 #include "../../include/nanochat_amd.h"
 #include "nc_common.h"
 #include "nc_kernels.h"
+#include "nc_rope.h"
 
 #define TRY(call)              \
     do {                       \
@@ -196,14 +200,22 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         site++;
         bf16_t* kc = kv->k_cache + (size_t)i * layer_elems;
         bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
-        if (qsrc.parts)
-            TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len, kv->cache_seqlens,
-                                            kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
-        else
-            TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
-                                          kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
-        TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
-                                w.attn_counters, w.attn_parts, w.attn_part_bytes, w.amax + site, 0, 1, s));
+        if (T == 1 && nc_attn_splits(B, 1, Hkv, ly.window_left, kv->max_seq_len) == 1) {
+            // decode: the attention workgroups finish their own q|k|v heads and append to the cache themselves
+            const NcRopeSrc rope{qsrc.parts ? nullptr : w.qkv, qkv_w, qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin,
+                                 m->rope_len, m->padded_vocab};
+            TRY(nc_launch_attention_fused(rope, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, H, Hkv, kv->max_seq_len,
+                                          w.amax + site, s));
+        } else {
+            if (qsrc.parts)
+                TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
+                                                kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
+            else
+                TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
+                                              kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
+            TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
+                                    w.attn_counters, w.attn_parts, w.attn_part_bytes, w.amax + site, 0, 1, s));
+        }
         TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E, &pending_parts));
         pending_add = pending_parts.parts ? nullptr : w.o;
         site++;

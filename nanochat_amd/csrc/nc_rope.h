@@ -1,0 +1,75 @@
+// One head of the q|k|v post-processing of CausalSelfAttention.forward (nanochat/gpt.py:89-104), done by one wave:
+// lane L holds elements L and L+64 of the 128-wide head, which is exactly one rotary pair.
+//   q and k heads: rotary by the position's angle -> rms_norm over the head -> * 1.2
+//   v heads:       v + 3*sigmoid(W_g . xn[:12])[head] * ve[token id, head, :]   (layers with a value embedding)
+// Every value is rounded to bf16 wherever the eager bf16 graph of the reference materialises a tensor.
+// Shared by the stand-alone rotary/append kernel and by the decode attention kernel that does this work itself.
+#pragma once
+#include "nc_common.h"
+#include "nc_kernels.h"
+
+#define RMS_EPS 1.1920928955078125e-07f   // fp32 machine epsilon: F.rms_norm's default eps
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+struct NcRopeSrc {
+    const bf16_t* qkv;        // bf16 [tokens, ld_qkv] output of the q|k|v linear, or nullptr when it is still in partials
+    int ld_qkv;
+    NcPartialSrc pq;
+    const bf16_t* xn;         // normalised layer input (the value-embedding gate reads its first 12 channels)
+    int ld_xn;
+    const int64_t* idx;       // token ids
+    const bf16_t* ve_table;   // nullptr: layer without value embedding
+    const float* ve_gate_w;
+    const bf16_t* cos_t;
+    const bf16_t* sin_t;
+    int rope_len;
+    int vocab_rows;
+};
+
+// hh in [0, H): query head; [H, H+Hkv): key head; [H+Hkv, H+2Hkv): value head.  Returns the finished pair.
+__device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos, int hh, int H, int Hkv, int lane, float& o1, float& o2) {
+    float x1, x2;
+    if (r.pq.parts) {
+        // the linear's output still sits in split partials: add them up, scale, round to bf16
+        const int col = hh * 128 + lane;
+        const float* pp = r.pq.parts + (size_t)token * r.pq.ld + col;
+        float a1 = 0.f, a2 = 0.f;
+        for (int sp = 0; sp < r.pq.nsplit; sp++) {
+            a1 += pp[(size_t)sp * r.pq.split_stride];
+            a2 += pp[(size_t)sp * r.pq.split_stride + 64];
+        }
+        const float inv_a = 1.0f / scale_from_amax(__uint_as_float(*r.pq.a_amax));
+        const float inv_b = r.pq.inv_b[col >= r.pq.seg_end1 ? 2 : (col >= r.pq.seg_end0 ? 1 : 0)];
+        x1 = rbf((a1 * inv_a) * inv_b);
+        x2 = rbf((a2 * inv_a) * inv_b);
+    } else {
+        const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128;
+        x1 = bf16_to_f32(src[lane]), x2 = bf16_to_f32(src[lane + 64]);
+    }
+    if (hh < H + Hkv) {
+        const int rp = pos < r.rope_len ? (pos < 0 ? 0 : pos) : r.rope_len - 1;
+        const float c = bf16_to_f32(r.cos_t[(size_t)rp * 64 + lane]), s = bf16_to_f32(r.sin_t[(size_t)rp * 64 + lane]);
+        float y1 = rbf(rbf(x1 * c) + rbf(x2 * s));
+        float y2 = rbf(rbf(x1 * (-s)) + rbf(x2 * c));
+        const float ss = wave_sum(y1 * y1 + y2 * y2);
+        const float rstd = 1.0f / sqrtf(ss / 128.0f + RMS_EPS);
+        o1 = rbf(rbf(y1 * rstd) * 1.2f);
+        o2 = rbf(rbf(y2 * rstd) * 1.2f);
+    } else {
+        const int hv = hh - H - Hkv;
+        if (r.ve_table) {
+            float dot = 0.f;
+            const bf16_t* xr = r.xn + (size_t)token * r.ld_xn;
+#pragma unroll
+            for (int cidx = 0; cidx < 12; cidx++) dot += bf16_to_f32(xr[cidx]) * rbf(r.ve_gate_w[hv * 12 + cidx]);
+            const float gate = rbf(3.0f * rbf(sigmoidf_(rbf(dot))));
+            int64_t tok = r.idx[token];
+            if (tok < 0 || tok >= r.vocab_rows) tok = 0;
+            const bf16_t* ve = r.ve_table + ((size_t)tok * Hkv + hv) * 128;
+            x1 = rbf(x1 + rbf(gate * bf16_to_f32(ve[lane])));
+            x2 = rbf(x2 + rbf(gate * bf16_to_f32(ve[lane + 64])));
+        }
+        o1 = x1, o2 = x2;
+    }
+}

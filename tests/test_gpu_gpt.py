@@ -58,6 +58,9 @@ def build_pair(cfg_kwargs, seed, trained_like=True):
 D4 = dict(sequence_len=2048, vocab_size=32768, n_layer=4, n_head=2, n_kv_head=2, n_embd=256)
 SMALL_GQA = dict(sequence_len=256, vocab_size=1024, n_layer=5, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
 SMALL_MHA = dict(sequence_len=512, vocab_size=2048, n_layer=6, n_head=3, n_kv_head=3, n_embd=384, window_pattern="SSSL")
+# batch x kv heads >= 512: attention runs one workgroup per (row, kv head) and finishes q|k|v (rotary, append) itself
+WIDE_GQA = dict(sequence_len=128, vocab_size=1024, n_layer=3, n_head=8, n_kv_head=4, n_embd=1024, window_pattern="SL")
+WIDE_MHA = dict(sequence_len=128, vocab_size=1024, n_layer=2, n_head=4, n_kv_head=4, n_embd=512, window_pattern="SL")
 
 
 @pytest.fixture(scope="module")
@@ -284,7 +287,8 @@ def test_cached_decode_equals_cache_free_forward(d4_pair):
     assert (stepped.argmax(-1) == full[:, 15:].argmax(-1)).float().mean().item() > 0.5
 
 
-@pytest.mark.parametrize("cfg_kwargs,B,P,steps", [(SMALL_GQA, 8, 40, 12), (SMALL_MHA, 5, 70, 10)])
+@pytest.mark.parametrize("cfg_kwargs,B,P,steps", [(SMALL_GQA, 8, 40, 12), (SMALL_MHA, 5, 70, 10), (WIDE_GQA, 128, 90, 5),
+                                                  (WIDE_MHA, 128, 3, 6)])
 def test_small_models_batched_decode(cfg_kwargs, B, P, steps):
     say(f"small model {cfg_kwargs['n_embd']}/{cfg_kwargs['n_head']}q{cfg_kwargs['n_kv_head']}kv B={B}")
     rt, model = build_pair(cfg_kwargs, seed=3)
