@@ -45,6 +45,32 @@ __device__ __forceinline__ void block_argmax(float& v, int& i, float* sval, int*
         if (sval[k] > v || (sval[k] == v && sidx[k] < i)) v = sval[k], i = sidx[k];
 }
 
+// f(value, index) over one row of logits, 16-byte loads with four in flight per thread when the row is aligned
+template <typename F>
+__device__ __forceinline__ void scan_row(const float* __restrict__ lr, int V, int tid, F f) {
+    int done = 0;
+    if (((uintptr_t)lr & 15) == 0) {
+        const int nv = V >> 2;
+        const float4* p = (const float4*)lr;
+        int i = tid;
+        for (; i + 3 * SAMPLE_THREADS < nv; i += 4 * SAMPLE_THREADS) {
+            const float4 r0 = p[i], r1 = p[i + SAMPLE_THREADS], r2 = p[i + 2 * SAMPLE_THREADS], r3 = p[i + 3 * SAMPLE_THREADS];
+            const float4 r[4] = {r0, r1, r2, r3};
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int b = 4 * (i + u * SAMPLE_THREADS);
+                f(r[u].x, b), f(r[u].y, b + 1), f(r[u].z, b + 2), f(r[u].w, b + 3);
+            }
+        }
+        for (; i < nv; i += SAMPLE_THREADS) {
+            const float4 r = p[i];
+            f(r.x, 4 * i), f(r.y, 4 * i + 1), f(r.z, 4 * i + 2), f(r.w, 4 * i + 3);
+        }
+        done = nv * 4;
+    }
+    for (int i = done + tid; i < V; i += SAMPLE_THREADS) f(lr[i], i);
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, int V, int ld, float temperature,
                                                                 int top_k, const float* __restrict__ noise, int64_t* __restrict__ out_ids) {
     __shared__ float sval[4];
@@ -61,10 +87,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     if (temperature == 0.0f) {
         float bv = -INFINITY;
         int bi = 0x7fffffff;
-        for (int i = tid; i < V; i += SAMPLE_THREADS) {
-            const float v = lr[i];
+        scan_row(lr, V, tid, [&](float v, int i) {
             if (v > bv || (v == bv && i < bi)) bv = v, bi = i;      // NaN never wins; an all-NaN row yields index 0 below
-        }
+        });
         block_argmax(bv, bi, sval, sidx);
         if (tid == 0) out_ids[row] = (bi == 0x7fffffff) ? 0 : bi;
         return;
@@ -74,7 +99,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
         // full-vocabulary softmax: argmax_i exp((l_i - max)/T) / e_i  ==  argmax_i (l_i/T - max/T - log e_i)
         float mx = -INFINITY;
         int dummy = 0;
-        for (int i = tid; i < V; i += SAMPLE_THREADS) mx = fmaxf(mx, lr[i] / temperature);
+        scan_row(lr, V, tid, [&](float v, int) { mx = fmaxf(mx, v / temperature); });
         block_argmax(mx, dummy, sval, sidx);
         float bv = -INFINITY;
         int bi = 0x7fffffff;
@@ -96,10 +121,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
         __syncthreads();
         const uint32_t prefix = sel_prefix;
         const uint32_t himask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
-        for (int i = tid; i < V; i += SAMPLE_THREADS) {
-            const uint32_t key = fkey(lr[i]);
+        scan_row(lr, V, tid, [&](float v, int) {
+            const uint32_t key = fkey(v);
             if ((key & himask) == prefix) atomicAdd(&hist[(key >> shift) & 0xff], 1u);
-        }
+        });
         __syncthreads();
         if (tid == 0) {
             uint32_t need = sel_need, bin = 255;
