@@ -81,7 +81,7 @@ int nc_rmsnorm(const uint16_t* x, uint16_t* out, int rows, int cols, uint32_t* a
 int nc_embed_norm_smear(const int64_t* idx, const uint16_t* wte, const float* smear_w, const float* smear_lambda,
                         const uint16_t* prev_in, uint16_t* prev_out, uint16_t* x_out, int B, int T, int E, int vocab_rows,
                         nc_stream_t stream) {
-    return nc_launch_embed_norm_smear(idx, wte, smear_w, smear_lambda, prev_in, prev_out, x_out, B, T, E, vocab_rows,
+    return nc_launch_embed_norm_smear(idx, wte, smear_w, smear_lambda, prev_in, prev_out, x_out, nullptr, B, T, E, vocab_rows, nullptr, 0,
                                       (hipStream_t)stream);
 }
 

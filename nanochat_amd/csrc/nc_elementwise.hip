@@ -32,9 +32,13 @@ __device__ __forceinline__ void block_amax_commit(float local_abs_max, uint32_t*
 __global__ __launch_bounds__(256) void embed_norm_smear_kernel(const int64_t* __restrict__ idx, const bf16_t* __restrict__ wte,
                                                                const float* __restrict__ smear_w, const float* __restrict__ smear_lambda,
                                                                const bf16_t* __restrict__ prev_in, bf16_t* __restrict__ prev_out,
-                                                               bf16_t* __restrict__ x_out, int T, int E, int vocab_rows) {
+                                                               bf16_t* __restrict__ x_out, bf16_t* __restrict__ x0_out, int T, int E,
+                                                               int vocab_rows, uint32_t* __restrict__ clear_words, int n_clear) {
     extern __shared__ float rowbuf[];          // [2][E]: this token, previous token (both normalised, bf16 values)
     __shared__ float red[8];
+    // first kernel of a forward pass: it also zeroes the pass's amax slots and arrival counters
+    if (blockIdx.x == 0)
+        for (int i = threadIdx.x; i < n_clear; i += 256) clear_words[i] = 0u;
     const int row = blockIdx.x, b = row / T, t = row % T;
     const bool use_prev_token = (T > 1 && t >= 1);
     const bool use_prev_cache = (T == 1 && prev_in != nullptr);
@@ -69,6 +73,7 @@ __global__ __launch_bounds__(256) void embed_norm_smear_kernel(const int64_t* __
         if (use_prev_token) v = rbf(v + rbf(gate * rowbuf[E + c]));
         else if (use_prev_cache) v = rbf(v + rbf(gate * bf16_to_f32(prev_in[(size_t)b * E + c])));
         x_out[(size_t)row * E + c] = f32_to_bf16(v);
+        if (x0_out) x0_out[(size_t)row * E + c] = f32_to_bf16(v);      // the copy the per-layer residual mix reads (gpt.py:495)
     }
 }
 
@@ -274,13 +279,13 @@ int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t
 }
 
 int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const float* smear_w, const float* smear_lambda,
-                               const bf16_t* prev_in, bf16_t* prev_out, bf16_t* x_out, int B, int T, int E, int vocab_rows,
-                               hipStream_t s) {
+                               const bf16_t* prev_in, bf16_t* prev_out, bf16_t* x_out, bf16_t* x0_out, int B, int T, int E,
+                               int vocab_rows, uint32_t* clear_words, int n_clear, hipStream_t s) {
     NC_CHECK_ARG(idx && wte && smear_w && smear_lambda && prev_out && x_out, "embed_norm_smear: null pointer");
     NC_CHECK_ARG(B > 0 && T > 0 && E >= 24 && E <= 8192, "embed_norm_smear: bad shape B=%d T=%d E=%d", B, T, E);
     NcProfScope prof(3, 4.0 * B * T * E, s);
     hipLaunchKernelGGL(embed_norm_smear_kernel, dim3(B * T), dim3(256), 2 * E * sizeof(float), s, idx, wte, smear_w, smear_lambda,
-                       prev_in, prev_out, x_out, T, E, vocab_rows);
+                       prev_in, prev_out, x_out, x0_out, T, E, vocab_rows, clear_words, clear_words ? n_clear : 0);
     NC_CHECK_LAUNCH("embed_norm_smear");
     return 0;
 }

@@ -25,8 +25,8 @@
 //   a8                    u8   [M,4E]       quantized activations (prefill only)
 //   xl                    bf16 [B,E]        last-position rows (last_only lm_head at T > 1)
 //   inv                   fp32 [4L+1]       activation inverse scales (prefill only)
-//   zeroed                u32               amax slots [4L+1] | attention split counters, cleared by one kernel at
-//                                           the start of the call
+//   zeroed                u32               amax slots [4L+1] | attention split counters, cleared by the embedding
+//                                           kernel at the start of the call
 //   gemm_parts, attn_parts                  split partials of the small-M linears and of attention
 #include <stdio.h>
 #include "../../include/nanochat_amd.h"
@@ -173,12 +173,9 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
     const LinearRunner lin{w, s};
     int site = 0;   // amax / inv slot of the next FP8 linear input
 
-    nc_clear_u32(w.amax, w.zero_words, s);
-    TRY(nc_launch_embed_norm_smear(idx, m->wte, m->smear_w, m->smear_lambda, kv->prev_in, kv->prev_out, w.x, B, T, E,
-                                   m->padded_vocab, s));
     // x0 is the post-smear embedding; layer 0 reads it through both x and x0 (gpt.py:495,500)
-    if (hipMemcpyAsync(w.x0, w.x, (size_t)M * E * sizeof(bf16_t), hipMemcpyDeviceToDevice, s) != hipSuccess)
-        NC_FAIL(-2, "gpt_forward: x0 copy failed");
+    TRY(nc_launch_embed_norm_smear(idx, m->wte, m->smear_w, m->smear_lambda, kv->prev_in, kv->prev_out, w.x, w.x0, B, T, E,
+                                   m->padded_vocab, w.amax, w.zero_words, s));
 
     // output of the previous MLP projection, still to be added into the residual stream: bf16 rows or split partials
     const bf16_t* pending_add = nullptr;

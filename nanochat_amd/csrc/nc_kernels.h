@@ -51,8 +51,8 @@ struct NcPartialSrc {
 // ---- elementwise / norm / rope (nc_elementwise.hip)
 int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s);
 int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const float* smear_w, const float* smear_lambda,
-                               const bf16_t* prev_in, bf16_t* prev_out, bf16_t* x_out, int B, int T, int E, int vocab_rows,
-                               hipStream_t s);
+                               const bf16_t* prev_in, bf16_t* prev_out, bf16_t* x_out, bf16_t* x0_out, int B, int T, int E,
+                               int vocab_rows, uint32_t* clear_words, int n_clear, hipStream_t s);
 int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
                        const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
                        int rows, int cols, uint32_t* amax_ws, hipStream_t s);
