@@ -60,6 +60,29 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     int k_end = k_begin + chunk;
     if (k_end > k_stop) k_end = k_stop;
 
+    const size_t key_stride = (size_t)Hkv * 128;   // elements between consecutive keys
+    const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
+    const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
+
+    constexpr int UNROLL = 8;     // 8 loads x 4 keys = 32 keys (8 KB of K and 8 KB of V) in flight per wave
+    uint4 kr[UNROLL], vr[UNROLL];
+    bool ok[UNROLL];
+    auto fetch = [&](int kb0) {
+#pragma unroll
+        for (int i = 0; i < UNROLL; i++) {
+            const int j = kb0 + 4 * i + grp;
+            ok[i] = j < k_end;
+            kr[i] = ok[i] ? nt_load16(kbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < UNROLL; i++) {
+            const int j = kb0 + 4 * i + grp;
+            vr[i] = ok[i] ? nt_load16(vbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    // the first batch of keys is on its way before anything that needs q
+    if (k_begin < k_end) fetch(k_begin);
+
     if (FUSED) {
         // wave w finishes head task w, w+4, ...: tasks 0..G-1 are the query heads, G the key head, G+1 the value head
         for (int task = wave; task < G + 2; task += 4) {
@@ -117,25 +140,8 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         }
     }
 
-    const size_t key_stride = (size_t)Hkv * 128;   // elements between consecutive keys
-    const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
-    const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
-
-    constexpr int UNROLL = 8;     // 8 loads x 4 keys = 32 keys (8 KB of K and 8 KB of V) in flight per wave
     for (int kb0 = k_begin; kb0 < k_end; kb0 += 4 * UNROLL) {
-        uint4 kr[UNROLL], vr[UNROLL];
-        bool ok[UNROLL];
-#pragma unroll
-        for (int i = 0; i < UNROLL; i++) {
-            const int j = kb0 + 4 * i + grp;
-            ok[i] = j < k_end;
-            kr[i] = ok[i] ? nt_load16(kbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < UNROLL; i++) {
-            const int j = kb0 + 4 * i + grp;
-            vr[i] = ok[i] ? nt_load16(vbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
-        }
+        if (kb0 != k_begin) fetch(kb0);
         float sc[G][UNROLL];
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
