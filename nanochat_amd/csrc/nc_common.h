@@ -169,14 +169,38 @@ __device__ __forceinline__ bool arrive_and_check_last(uint32_t* counter, uint32_
     return last;
 }
 
-// Max-reduce a non-negative fp32 into a device word (fp32 bit patterns of non-negative values order like integers).
-// Atomics on one address serialize at the device coherence point, so the atomic is skipped when the word already
-// holds at least this value.
-__device__ __forceinline__ void amax_publish(uint32_t* ws, float am) {
+// ---------------------------------------------------------------- amax words
+// The tensorwise amax of an activation is max-reduced by its producer kernel into a device word (fp32 bit patterns
+// of non-negative values order like integers) and read by the FP8 linear that quantizes the activation.  Atomics on
+// one address serialize at the device coherence point (~6 ns each across XCDs: 832 workgroups ending together cost
+// ~3.5 us), so the forward pass gives every site NC_AMAX_SLOTS words on separate 128-byte lines: a producer workgroup
+// publishes into the slot its block index selects, a consumer takes the max over the slots.  A pointer to such a
+// site carries tag bit 0 (nc_amax_slotted); an untagged pointer is a single word (the stand-alone entry points).
+// Only amax_read / amax_publish may look through these pointers.
+#define NC_AMAX_SLOTS 8
+#define NC_AMAX_STRIDE 32      // words between slots
+static inline uint32_t* nc_amax_slotted(uint32_t* site) { return (uint32_t*)((uintptr_t)site | 1u); }
+
+__device__ __forceinline__ float amax_read(const uint32_t* h) {
+    const uint32_t* p = (const uint32_t*)((uintptr_t)h & ~(uintptr_t)3);
+    uint32_t m = p[0];
+    if ((uintptr_t)h & 1u) {
+#pragma unroll
+        for (int i = 1; i < NC_AMAX_SLOTS; i++) {
+            const uint32_t v = p[i * NC_AMAX_STRIDE];
+            m = v > m ? v : m;
+        }
+    }
+    return __uint_as_float(m);
+}
+// One call per workgroup.  The atomic is skipped when the word already holds at least the value.
+__device__ __forceinline__ void amax_publish(uint32_t* h, float am) {
     const uint32_t bits = __float_as_uint(am);
     if (bits == 0u || (bits >> 31)) return;
-    if (__hip_atomic_load(ws, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
-    atomicMax(ws, bits);
+    uint32_t* p = (uint32_t*)((uintptr_t)h & ~(uintptr_t)3);
+    if ((uintptr_t)h & 1u) p += ((blockIdx.x + 3u * blockIdx.y + 5u * blockIdx.z) % NC_AMAX_SLOTS) * NC_AMAX_STRIDE;
+    if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
+    atomicMax(p, bits);
 }
 
 // block-wide sum for blockDim.x == 64 * NW, result broadcast to every thread

@@ -37,8 +37,7 @@ __global__ __launch_bounds__(256) void embed_norm_smear_kernel(const int64_t* __
     extern __shared__ float rowbuf[];          // [2][E]: this token, previous token (both normalised, bf16 values)
     __shared__ float red[8];
     // first kernel of a forward pass: it also zeroes the pass's amax slots and arrival counters
-    if (blockIdx.x == 0)
-        for (int i = threadIdx.x; i < n_clear; i += 256) clear_words[i] = 0u;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n_clear; i += gridDim.x * 256) clear_words[i] = 0u;
     const int row = blockIdx.x, b = row / T, t = row % T;
     const bool use_prev_token = (T > 1 && t >= 1);
     const bool use_prev_cache = (T == 1 && prev_in != nullptr);
@@ -129,7 +128,7 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
     const bool writes_x = add || padd.parts || resid_lambda || backout_lambda;
     float p_inv_a = 0.f, p_inv_b = 0.f;
     if (padd.parts) {
-        p_inv_a = 1.0f / scale_from_amax(__uint_as_float(*padd.a_amax));
+        p_inv_a = 1.0f / scale_from_amax(amax_read(padd.a_amax));
         p_inv_b = padd.inv_b[0];
     }
     float v[NV][8];

@@ -25,8 +25,8 @@
 //   a8                    u8   [M,4E]       quantized activations (prefill only)
 //   xl                    bf16 [B,E]        last-position rows (last_only lm_head at T > 1)
 //   inv                   fp32 [4L+1]       activation inverse scales (prefill only)
-//   zeroed                u32               amax slots [4L+1] | attention split counters, cleared by the embedding
-//                                           kernel at the start of the call
+//   zeroed                u32               amax sites [4L+1] x 8 slots on separate lines | attention split counters,
+//                                           cleared by the embedding kernel at the start of the call
 //   gemm_parts, attn_parts                  split partials of the small-M linears and of attention
 #include <stdio.h>
 #include "../../include/nanochat_amd.h"
@@ -59,6 +59,8 @@ struct Workspace {
     uint8_t* a8;
     float* inv;
     uint32_t *amax, *attn_counters;
+    // handle of amax site i (tagged: NC_AMAX_SLOTS words on separate lines, see amax_read / amax_publish)
+    uint32_t* site(int i) const { return nc_amax_slotted(amax + (size_t)i * NC_AMAX_SLOTS * NC_AMAX_STRIDE); }
     int zero_words;
     uint8_t *gemm_parts, *attn_parts;
     size_t gemm_part_bytes, attn_part_bytes;
@@ -84,7 +86,7 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     w.a8 = c.take<uint8_t>(small ? 0 : M * 4 * E);
     w.xl = c.take<bf16_t>((size_t)B * E);
     w.inv = c.take<float>(4 * (size_t)m->n_layer + 1);
-    const size_t amax_words = (4 * (size_t)m->n_layer + 1 + 63) & ~(size_t)63;
+    const size_t amax_words = (4 * (size_t)m->n_layer + 1) * NC_AMAX_SLOTS * NC_AMAX_STRIDE;     // one slotted site per FP8 linear input
     const size_t attn_words = nc_attn_counter_bytes(B, T, m->n_head) / 4;
     uint32_t* zero = c.take<uint32_t>(amax_words + attn_words);
     w.amax = zero;
@@ -127,19 +129,19 @@ struct LinearRunner {
         if (src) *src = NO_PARTIALS;
         if (rows <= 128) {
             int used = 1;
-            TRY(nc_launch_gemm_decode(in, 1, w.amax + site, nullptr, w8, inv_w, segs, out, out_kind, softcap, out_amax, rows, N, K, ldc,
+            TRY(nc_launch_gemm_decode(in, 1, w.site(site), nullptr, w8, inv_w, segs, out, out_kind, softcap, out_amax, rows, N, K, ldc,
                                       (float*)w.gemm_parts, w.gemm_part_bytes, src || out_kind == 2 ? 0 : 1, &used, s));
             if (used == 1) return 0;
             if (src) {
-                *src = NcPartialSrc{(const float*)w.gemm_parts, used, N, (size_t)rows * N, w.amax + site, inv_w,
+                *src = NcPartialSrc{(const float*)w.gemm_parts, used, N, (size_t)rows * N, w.site(site), inv_w,
                                     segs.nseg > 1 ? segs.end[0] : 0x7fffffff, segs.nseg > 2 ? segs.end[1] : 0x7fffffff};
                 return 0;
             }
-            return nc_launch_finish_partials((const float*)w.gemm_parts, used, w.amax + site, nullptr, inv_w, segs, out, out_kind, softcap,
+            return nc_launch_finish_partials((const float*)w.gemm_parts, used, w.site(site), nullptr, inv_w, segs, out, out_kind, softcap,
                                              out_amax, rows, N, ldc, s);
         }
         // large M: explicit convert pass, tiled GEMM; relu^2 (out_kind 2) is a separate kernel there
-        TRY(nc_launch_convert_only(in, (int64_t)rows * K, w.a8, w.inv + site, w.amax + site, s));
+        TRY(nc_launch_convert_only(in, (int64_t)rows * K, w.a8, w.inv + site, w.site(site), s));
         if (out_kind == 2) {
             TRY(nc_launch_gemm(w.a8, w8, w.inv + site, inv_w, segs, w.h, 0, 0.f, rows, N, K, N, 0, nullptr, 0, s));
             return nc_launch_relu2(w.h, (bf16_t*)out, (int64_t)rows * N, out_amax, s);
@@ -189,7 +191,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         NC_CHECK_ARG(ly.w_qkv && ly.inv_qkv && ly.w_attn_proj && ly.w_fc && ly.w_mlp_proj, "gpt_forward: layer %d has no FP8 weights", i);
         // x += mlp_out(prev layer); [save backout]; x = rl*x + xl*x0; xn = norm(x)
         bf16_t* save = (i > 0 && (i - 1) == L / 2) ? w.xb : nullptr;
-        TRY(mix(m->resid_lambdas + i, m->x0_lambdas + i, nullptr, nullptr, save, w.amax + site));
+        TRY(mix(m->resid_lambdas + i, m->x0_lambdas + i, nullptr, nullptr, save, w.site(site)));
         // q|k|v = FP8 linear(xn): one activation quantization, three weight scales
         NcGemmSegs qkv_segs{3, {H * 128, (H + Hkv) * 128, qkv_w, 0}};
         NcPartialSrc qsrc;
@@ -202,7 +204,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
             const NcRopeSrc rope{qsrc.parts ? nullptr : w.qkv, qkv_w, qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin,
                                  m->rope_len, m->padded_vocab};
             TRY(nc_launch_attention_fused(rope, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, H, Hkv, kv->max_seq_len,
-                                          w.amax + site, s));
+                                          w.site(site), s));
         } else {
             if (qsrc.parts)
                 TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
@@ -211,15 +213,15 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
                 TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
                                               kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
             TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
-                                    w.attn_counters, w.attn_parts, w.attn_part_bytes, w.amax + site, 0, 1, s));
+                                    w.attn_counters, w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s));
         }
         TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E, &pending_parts));
         pending_add = pending_parts.parts ? nullptr : w.o;
         site++;
         // x += attn_out; xn = norm(x)
-        TRY(mix(nullptr, nullptr, nullptr, nullptr, nullptr, w.amax + site));
+        TRY(mix(nullptr, nullptr, nullptr, nullptr, nullptr, w.site(site)));
         // h2 = relu(c_fc(xn))^2 with its amax in the next slot
-        TRY(lin.run(w.xn, M, site, ly.w_fc, ly.inv_fc, one_seg(4 * E), w.h2, 2, 0.f, w.amax + site + 1, 4 * E, E, 4 * E, nullptr));
+        TRY(lin.run(w.xn, M, site, ly.w_fc, ly.inv_fc, one_seg(4 * E), w.h2, 2, 0.f, w.site(site + 1), 4 * E, E, 4 * E, nullptr));
         site++;
         TRY(lin.run(w.h2, M, site, ly.w_mlp_proj, ly.inv_mlp_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, 4 * E, E, &pending_parts));
         pending_add = pending_parts.parts ? nullptr : w.o;
@@ -234,7 +236,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
             pending_add = nullptr;
             pending_parts = NO_PARTIALS;
         }
-        TRY(mix(nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.amax + site));
+        TRY(mix(nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.site(site)));
     }
     // lm_head.  Its activation scale is tensorwise over all M rows (that is what the reference quantizes),
     // even when only the last position of every row is projected.

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
 
     float scale = 1.f, inv_a;
     if (A_BF16) {
-        scale = scale_from_amax(__uint_as_float(*g.a_amax));
+        scale = scale_from_amax(amax_read(g.a_amax));
         inv_a = 1.0f / scale;
     } else {
         inv_a = *g.inv_a;
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
                                                               NcGemmSegs segs, void* __restrict__ out, int out_kind, float softcap,
                                                               uint32_t* __restrict__ out_amax, int M, int N, int ldc) {
     __shared__ float red[4];
-    const float inv_a = a_amax ? 1.0f / scale_from_amax(__uint_as_float(*a_amax)) : *inv_a_ptr;
+    const float inv_a = a_amax ? 1.0f / scale_from_amax(amax_read(a_amax)) : *inv_a_ptr;
     const int n4 = N / 4;
     float am = 0.f;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)M * n4; i += (size_t)gridDim.x * 256) {

@@ -65,7 +65,7 @@ template <bool IS_BF16, bool HW_CVT>
 __global__ __launch_bounds__(256) void convert_kernel(const void* __restrict__ x, int64_t n, const uint32_t* __restrict__ amax_bits,
                                                       uint8_t* __restrict__ out, float* __restrict__ scale_out,
                                                       float* __restrict__ inv_out) {
-    const float amax = __uint_as_float(*amax_bits);
+    const float amax = amax_read(amax_bits);
     const float scale = scale_from_amax(amax);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         if (scale_out) *scale_out = scale;

@@ -39,7 +39,7 @@ __device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos
             a1 += pp[(size_t)sp * r.pq.split_stride];
             a2 += pp[(size_t)sp * r.pq.split_stride + 64];
         }
-        const float inv_a = 1.0f / scale_from_amax(__uint_as_float(*r.pq.a_amax));
+        const float inv_a = 1.0f / scale_from_amax(amax_read(r.pq.a_amax));
         const float inv_b = r.pq.inv_b[col >= r.pq.seg_end1 ? 2 : (col >= r.pq.seg_end0 ? 1 : 0)];
         x1 = rbf((a1 * inv_a) * inv_b);
         x2 = rbf((a2 * inv_a) * inv_b);
