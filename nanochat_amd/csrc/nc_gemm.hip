@@ -9,7 +9,8 @@
 // bf16 store.
 //
 //   gemm_bl_kernel      M large (prefill, isolated Float8Linear): BMxBNx128 tiles, double-buffered swizzled LDS fed
-//                       through two register stages of buffer loads, bf16 epilogue staged through LDS.
+//                       through two register stages of buffer loads (for the 128x128 tile the fills and loads are
+//                       placed between the MFMA groups by hand), bf16 epilogue staged through LDS.
 //   gemm_tile_kernel    the same tiling with plain global loads (64-bit addressing) for operands past 2 GiB.
 //   M <= 128 (decode) is weight-bandwidth bound and handled by gemm_decode_kernel in nc_gemm_decode.hip.
 #include "nc_common.h"
@@ -220,7 +221,7 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             if (m >= M || n >= N) continue;
             bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
             if (n + 8 <= N) {
-                if (vec16) *(uint4*)o = v;
+                if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
                 else {
                     *(uint2*)o = make_uint2(v.x, v.y);
                     *(uint2*)(o + 4) = make_uint2(v.z, v.w);
@@ -264,7 +265,12 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
 __device__ __forceinline__ void mfma_f8_acc(v4f& acc, const v8i& b, const v8i& a) {
     asm("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
 }
-template <int BM, int BN, int WGM, int WGN, int OUT_KIND>
+// Same, pinned in program order against every memory operation: used where the LDS fills and global loads of the
+// next steps are placed between groups of MFMAs by hand, so that the LDS, load and matrix pipes work at the same time.
+__device__ __forceinline__ void mfma_f8_acc_ordered(v4f& acc, const v8i& b, const v8i& a) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a) : "memory");
+}
+template <int BM, int BN, int WGM, int WGN, int OUT_KIND, bool INTERLEAVE = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                  EpilogueArgs ep, int M, int N, int K, int tiles_m, int tiles_n) {
     constexpr int NT = 64 * WGM * WGN;
@@ -355,18 +361,57 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
         __syncthreads();                 \
         __builtin_amdgcn_sched_barrier(0); \
     } while (0)
+    // Interleaved step: the fill of the other LDS buffer and the reload of that register slot are cut into WTN
+    // portions, one after each group of WTM MFMAs; B fragments are fetched one group ahead.
+    constexpr int PIECES = A_CH + B_CH, PPG = (PIECES + WTN - 1) / WTN;
+#define BL_STEP_I(KT, BUF)                                                                                     \
+    do {                                                                                                       \
+        const uint8_t* st__ = lds + (BUF) * STAGE;                                                             \
+        uint8_t* fl__ = lds + ((BUF) ^ 1) * STAGE + lw;                                                        \
+        const int t__ = (KT) + 3;                                                                              \
+        const bool cut__ = t__ >= ksteps || (t__ == kfull && ch_in_tail);                                      \
+        v8i af__[WTM], bf__[2];                                                                                \
+        _Pragma("unroll") for (int i = 0; i < WTM; i++) af__[i] = frag(st__ + a_rd + i * 2048);                \
+        bf__[0] = frag(st__ + b_rd);                                                                           \
+        _Pragma("unroll") for (int j = 0; j < WTN; j++) {                                                      \
+            if (j + 1 < WTN) bf__[(j + 1) & 1] = frag(st__ + b_rd + (j + 1) * 2048);                           \
+            _Pragma("unroll") for (int q = 0; q < PPG; q++) {                                                  \
+                const int p = j * PPG + q;                                                                     \
+                const int pa = p < A_CH ? p : 0, pb = (p >= A_CH && p < PIECES) ? p - A_CH : 0;   /* in-range when not taken */ \
+                if (p < A_CH) {                                                                                \
+                    *(v4i*)(fl__ + pa * PASS_ROWS * 128) = ra[(BUF) ^ 1][pa];                                  \
+                    ra[(BUF) ^ 1][pa] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, cut__ ? NC_BUF_OOB : avo[pa], t__ * 128, 0); \
+                } else if (p < PIECES) {                                                                       \
+                    *(v4i*)(fl__ + BM * 128 + pb * PASS_ROWS * 128) = rb[(BUF) ^ 1][pb];                       \
+                    rb[(BUF) ^ 1][pb] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, cut__ ? NC_BUF_OOB : bvo[pb], t__ * 128, 0); \
+                }                                                                                              \
+            }                                                                                                  \
+            _Pragma("unroll") for (int i = 0; i < WTM; i++) mfma_f8_acc_ordered(acc[i][j], bf__[j & 1], af__[i]); \
+        }                                                                                                      \
+        __syncthreads();                                                                                       \
+    } while (0)
 
-    BL_LOAD(0, 0);
-    BL_LOAD(1, 1);
-    BL_FILL(0, 0);
-    BL_LOAD(0, 2);
-    __syncthreads();
     int kt = 0;
-    for (; kt + 1 < ksteps; kt += 2) {
-        BL_STEP(kt, 0);
-        BL_STEP(kt + 1, 1);
+    {
+        BL_LOAD(0, 0);
+        BL_LOAD(1, 1);
+        BL_FILL(0, 0);
+        BL_LOAD(0, 2);
+        __syncthreads();
+        if (INTERLEAVE) {
+            for (; kt + 1 < ksteps; kt += 2) {
+                BL_STEP_I(kt, 0);
+                BL_STEP_I(kt + 1, 1);
+            }
+        } else {
+            for (; kt + 1 < ksteps; kt += 2) {
+                BL_STEP(kt, 0);
+                BL_STEP(kt + 1, 1);
+            }
+        }
+        if (kt < ksteps) compute(0);
     }
-    if (kt < ksteps) compute(0);
+#undef BL_STEP_I
 #undef BL_LOAD
 #undef BL_FILL
 #undef BL_STEP
@@ -386,18 +431,18 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
     bl_epilogue<BM, BN, WGM, WGN, OUT_KIND>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
-template <int BM, int BN, int WGM, int WGN>
+template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE = false>
 static int launch_bl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
-    const void* fn = ep.out_kind == 0 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1>;
+    const void* fn = ep.out_kind == 0 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     if (ep.out_kind == 0)
-        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     else
-        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     return 0;
 }
 
@@ -467,9 +512,9 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
                                              N, ldc, s);
         return 0;
     } else if (which == 4) rc = launch_tile<128, 128>(a, b, ep, M, N, K, s);
-    else if (which == 5) rc = launch_bl<128, 128, 2, 2>(a, b, ep, M, N, K, s);
-    else if (which == 6) rc = launch_bl<256, 128, 4, 2>(a, b, ep, M, N, K, s);
-    else if (which == 7) rc = launch_bl<256, 256, 4, 2>(a, b, ep, M, N, K, s);
+    else if (which == 5) rc = launch_bl<128, 128, 2, 2, true>(a, b, ep, M, N, K, s);
+    else if (which == 6) rc = launch_bl<256, 128, 4, 2, false>(a, b, ep, M, N, K, s);
+    else if (which == 7) rc = launch_bl<256, 256, 4, 2, false>(a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");
