@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(HERE, "libnanochat_amd.so")
 
-SOURCES = ["nc_api.hip", "nc_quantize.hip", "nc_gemm.hip", "nc_elementwise.hip", "nc_attention.hip",
+SOURCES = ["nc_api.hip", "nc_quantize.hip", "nc_gemm.hip", "nc_elementwise.hip", "nc_attention.hip", "nc_attention_prefill.hip",
            "nc_sample.hip", "nc_forward.hip", "nc_profile.hip", "nc_gemm_decode.hip"]
 
 # -packed-fp32-ops off: packed fp32 VALU forms are not to be generated on this hardware pool

@@ -292,6 +292,11 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t*
                         uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
                         int counters_are_zero, hipStream_t s) {
     NC_CHECK_ARG((q || rope) && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
+    // many queries per row: the matrix-core kernel (a workgroup there covers 128 queries; below 16 queries per row
+    // the per-query streaming kernel wastes less)
+    if (!rope && T >= 16 && force_splits <= 0)
+        return nc_launch_attention_prefill(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new,
+                                           amax_ws, s);
     NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0, "decode_attention: bad shape");
     NC_CHECK_ARG(H % Hkv == 0, "decode_attention: n_head %d not a multiple of n_kv_head %d", H, Hkv);
     const int G = H / Hkv;

@@ -78,6 +78,10 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
                         uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
                         int counters_are_zero, hipStream_t s);
 
+// many query positions per row (nc_attention_prefill.hip): flash-attention forward on the bf16 matrix cores
+int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
+                                int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
+                                uint32_t* amax_ws, hipStream_t s);
 int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax);
 struct NcRopeSrc;
 int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,

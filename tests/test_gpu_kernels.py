@@ -468,6 +468,17 @@ def test_attention_prefill_chunk(ops, T, window):
     attn_case(ops, 2, T, 4, 2, 128, [0, 40], window, 0, seed=T)
 
 
+@pytest.mark.parametrize("T,window,H,Hkv,seqlens", [
+    (200, -1, 8, 2, [0, 56]), (300, 64, 3, 3, [0, 212]), (129, 0, 4, 4, [5, 0]), (257, 512, 2, 1, [0, 255]),
+    (128, 31, 4, 2, [384, 1]), (500, 100, 2, 2, [12, 0]), (15, -1, 4, 2, [3, 100]),
+])
+def test_attention_many_queries_per_row(ops, T, window, H, Hkv, seqlens):
+    """T query positions per row over a cache that already holds them (the prefill shape): causal, windowed, GQA,
+    rows at different cache positions, tiles that end inside a 32-key block, a row that fills the cache exactly."""
+    say(f"attention prefill T={T} window={window} H={H}/{Hkv} seq={seqlens}")
+    attn_case(ops, 2, T, H, Hkv, 512, seqlens, window, 0, seed=T + H)
+
+
 def test_attention_through_the_plugin_seam(ops):
     """flash_attn_with_kvcache as the model calls it: in-place insert, caller advances, then decode."""
     say("flash_attn seam")
