@@ -110,6 +110,13 @@ int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16
                         int Tmax, int seqlens_include_new, void* workspace, size_t workspace_bytes,
                         uint32_t* amax_ws, int splits, nc_stream_t stream);
 
+/* KVCache.prefill: nanochat/engine.py:123-137.  Copies the first n_tokens positions of every (layer, row) of one
+ * cache tensor (keys or values), laid out [layers, src_rows, src_tmax, token_bytes], into every row of
+ * [layers, dst_rows, dst_tmax, token_bytes]; src_rows is 1 (broadcast over the destination rows, what the Engine
+ * does after its batch-1 prefill) or dst_rows.  token_bytes = n_kv_head * head_dim * 2, a multiple of 16. */
+int nc_kv_cache_prefill(const void* src, void* dst, int layers, int src_rows, int dst_rows, int src_tmax, int dst_tmax,
+                        int n_tokens, int token_bytes, nc_stream_t stream);
+
 /* (5) softcap * tanh(bf16 logits / softcap) -> fp32: nanochat/gpt.py:511-515. */
 int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_stream_t stream);
 

@@ -12,7 +12,7 @@ EXPORTS = [
     "nc_abi_version", "nc_last_error", "nc_fp8_quantize_tensorwise", "nc_e4m3_encode_with_scale", "nc_fp8_gemm_tn",
     "nc_fp8_small_m_workspace_bytes", "nc_fp8_linear_small_m",
     "nc_rmsnorm", "nc_embed_norm_smear", "nc_mix_norm", "nc_relu2", "nc_qkv_rope_append",
-    "nc_attention_workspace_bytes", "nc_decode_attention", "nc_softcap", "nc_sample",
+    "nc_attention_workspace_bytes", "nc_decode_attention", "nc_kv_cache_prefill", "nc_softcap", "nc_sample",
     "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read",
 ]
 
@@ -58,6 +58,7 @@ def _bind(lib):
         "nc_qkv_rope_append": (i, [p, i, p, i, p, p, p, p, p, i, p, p, p, p, i, i, i, i, i, i, p]),
         "nc_attention_workspace_bytes": (sz, [i, i, i, i]),
         "nc_decode_attention": (i, [p, p, p, p, i, p, i, i, i, i, i, i, p, sz, p, i, p]),
+        "nc_kv_cache_prefill": (i, [p, p, i, i, i, i, i, i, i, p]),
         "nc_softcap": (i, [p, p, i64, f, p]),
         "nc_sample": (i, [p, i, i, i, f, i, p, p, p]),
         "nc_gpt_workspace_bytes": (sz, [C.POINTER(ModelDesc), i, i]),

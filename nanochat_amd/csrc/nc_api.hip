@@ -124,6 +124,11 @@ int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_str
     return nc_launch_softcap(raw, out, n, softcap, (hipStream_t)stream);
 }
 
+int nc_kv_cache_prefill(const void* src, void* dst, int layers, int src_rows, int dst_rows, int src_tmax, int dst_tmax, int n_tokens,
+                        int token_bytes, nc_stream_t stream) {
+    return nc_launch_kv_prefill_copy(src, dst, layers, src_rows, dst_rows, src_tmax, dst_tmax, n_tokens, token_bytes, (hipStream_t)stream);
+}
+
 int nc_sample(const float* logits, int B, int V, int ld, float temperature, int top_k, const float* noise, int64_t* out_ids,
               nc_stream_t stream) {
     return nc_launch_sample(logits, B, V, ld, temperature, top_k, noise, out_ids, (hipStream_t)stream);

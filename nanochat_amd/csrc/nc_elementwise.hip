@@ -267,6 +267,48 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(NcRopeSrc r, const
 }
 
 // ------------------------------------------------------------------------------------------------
+// KVCache.prefill (nanochat/engine.py:123-137): the first n positions of every (layer, row) of a source cache go to
+// every row of a destination cache with a longer time axis; a one-row source is broadcast over the rows.  Each
+// workgroup reads its 16 KB of a source (layer, row) once and writes it to all destination rows with streaming stores.
+__global__ __launch_bounds__(256) void kv_prefill_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t vec_per_row,
+                                                              size_t src_row_stride, size_t dst_row_stride, int src_rows, int dst_rows) {
+    const int layer = blockIdx.y;
+    const size_t v0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const int b_first = src_rows == 1 ? 0 : blockIdx.z, b_last = src_rows == 1 ? dst_rows : blockIdx.z + 1;
+    const uint4* sp = src + ((size_t)layer * src_rows + (src_rows == 1 ? 0 : blockIdx.z)) * src_row_stride;
+    v4i r[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (v0 + i < vec_per_row) r[i] = *(const v4i*)(sp + v0 + i);
+    for (int b = b_first; b < b_last; b++) {
+        uint4* dp = dst + ((size_t)layer * dst_rows + b) * dst_row_stride;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (v0 + i < vec_per_row) __builtin_nontemporal_store(r[i], (v4i*)(dp + v0 + i));
+    }
+}
+
+int nc_launch_kv_prefill_copy(const void* src, void* dst, int layers, int src_rows, int dst_rows, int src_tmax, int dst_tmax,
+                              int n_tokens, int token_bytes, hipStream_t s) {
+    NC_CHECK_ARG(src && dst, "kv_prefill_copy: null pointer");
+    NC_CHECK_ARG(layers > 0 && dst_rows > 0 && (src_rows == 1 || src_rows == dst_rows), "kv_prefill_copy: source rows must be 1 or match");
+    NC_CHECK_ARG(n_tokens >= 0 && n_tokens <= src_tmax && n_tokens <= dst_tmax, "kv_prefill_copy: %d tokens do not fit (%d -> %d)", n_tokens,
+                 src_tmax, dst_tmax);
+    NC_CHECK_ARG(token_bytes > 0 && token_bytes % 16 == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0,
+                 "kv_prefill_copy: token size and pointers must be multiples of 16 bytes");
+    NC_CHECK_ARG(layers <= 65535 && dst_rows <= 65535, "kv_prefill_copy: more than 65535 layers or rows");
+    if (n_tokens == 0) return 0;
+    const size_t vec_per_row = (size_t)n_tokens * token_bytes / 16;
+    const size_t gx = (vec_per_row + 1023) / 1024;
+    NC_CHECK_ARG(gx <= 0x7fffffff, "kv_prefill_copy: row too long");
+    NcProfScope prof(3, 0.0, s);
+    hipLaunchKernelGGL(kv_prefill_copy_kernel, dim3((unsigned)gx, layers, src_rows == 1 ? 1 : dst_rows), dim3(256), 0, s, (const uint4*)src,
+                       (uint4*)dst, vec_per_row, (size_t)src_tmax * token_bytes / 16, (size_t)dst_tmax * token_bytes / 16, src_rows, dst_rows);
+    NC_CHECK_LAUNCH("kv_prefill_copy");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
 static bool row_args_ok(int rows, int cols) { return rows >= 0 && cols > 0 && cols <= 16384; }
 
 int nc_launch_rmsnorm(const bf16_t* x, bf16_t* out, int rows, int cols, uint32_t* amax_ws, hipStream_t s) {

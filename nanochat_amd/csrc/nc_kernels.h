@@ -70,6 +70,9 @@ int nc_launch_qkv_rope_append(const bf16_t* qkv, int ld_qkv, const bf16_t* xn, i
                               int rope_len, const int32_t* cache_seqlens, bf16_t* k_cache, bf16_t* v_cache, bf16_t* q_out,
                               int B, int T, int H, int Hkv, int Tmax, int vocab_rows, hipStream_t s);
 
+int nc_launch_kv_prefill_copy(const void* src, void* dst, int layers, int src_rows, int dst_rows, int src_tmax, int dst_tmax,
+                              int n_tokens, int token_bytes, hipStream_t s);
+
 // ---- attention (nc_attention.hip)
 size_t nc_attn_counter_bytes(int B, int T, int H);
 size_t nc_attn_partial_bytes(int B, int T, int H);

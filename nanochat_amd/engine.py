@@ -126,8 +126,13 @@ class KVCache:
         assert self.n_layers == other.n_layers and self.n_heads == other.n_heads and self.head_dim == other.head_dim
         assert self.max_seq_len >= other.max_seq_len
         n = other.get_pos()
-        self.k_cache[:, :, :n, :, :] = other.k_cache[:, :, :n, :, :]
-        self.v_cache[:, :, :n, :, :] = other.v_cache[:, :, :n, :, :]
+        if self.k_cache.is_cuda:
+            assert other.batch_size in (1, self.batch_size)
+            ops.kv_cache_prefill(self.k_cache, other.k_cache, n)
+            ops.kv_cache_prefill(self.v_cache, other.v_cache, n)
+        else:           # host-side caches (the engine's own logic under test with a mock model)
+            self.k_cache[:, :, :n, :, :] = other.k_cache[:, :, :n, :, :]
+            self.v_cache[:, :, :n, :, :] = other.v_cache[:, :, :n, :, :]
         self.cache_seqlens.fill_(n)
         self._pos0 = self._pos_max = n
         if other.prev_embedding is not None:

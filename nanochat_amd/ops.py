@@ -235,6 +235,18 @@ def decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=-1, seqlens
     return out
 
 
+def kv_cache_prefill(dst, src, n_tokens):
+    """dst[:, :, :n] = src[:, :, :n] for cache tensors (L, B, T, Hkv, D); a one-row src is broadcast (engine.py:129-130)."""
+    _need_cuda(dst, src)
+    if not (dst.is_contiguous() and src.is_contiguous() and dst.dtype == src.dtype == torch.bfloat16):
+        raise ValueError("kv_cache_prefill: contiguous bf16 cache tensors expected")
+    L, Bd, Td, Hkv, D = dst.shape
+    Ls, Bs, Ts, Hs, Ds = src.shape
+    if (Ls, Hs, Ds) != (L, Hkv, D):
+        raise ValueError("kv_cache_prefill: layer / head geometry differs")
+    _lib.check(_lib.lib().nc_kv_cache_prefill(_ptr(src), _ptr(dst), L, Bs, Bd, Ts, Td, int(n_tokens), Hkv * D * 2, _stream()))
+
+
 # ----------------------------------------------------------------------------- (5) softcap / sample
 def softcap(raw_bf16, cap=15.0):
     _need_cuda(raw_bf16)

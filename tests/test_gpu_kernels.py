@@ -430,6 +430,21 @@ def test_qkv_rope_append(ops, H, Hkv, T, with_ve):
     ulp_close(vd.cpu(), vc_want, 0.01)
 
 
+@pytest.mark.parametrize("src_rows,dst_rows,n", [(1, 5, 37), (3, 3, 64), (1, 2, 0), (1, 64, 1)])
+def test_kv_cache_prefill_copy(ops, src_rows, dst_rows, n):
+    """KVCache.prefill (engine.py:123-137): dst[:, :, :n] = src[:, :, :n], a one-row source broadcast over the rows."""
+    say(f"kv cache prefill copy {src_rows}->{dst_rows} n={n}")
+    g = torch.Generator().manual_seed(n)
+    L, Hkv, Ts, Td = 3, 2, 64, 100
+    src = torch.randn(L, src_rows, Ts, Hkv, 128, generator=g).bfloat16()
+    dst = torch.randn(L, dst_rows, Td, Hkv, 128, generator=g).bfloat16()
+    want = dst.clone()
+    want[:, :, :n] = src[:, :, :n]
+    d = dst.to(DEV)
+    ops.kv_cache_prefill(d, src.to(DEV), n)
+    assert torch.equal(d.cpu(), want)
+
+
 # ================================================================== (3) attention
 def attn_case(ops, B, T, H, Hkv, Tmax, seqlens, window, splits, seed=0):
     g = torch.Generator().manual_seed(seed)
