@@ -51,44 +51,10 @@ class RangeTokenizer:
 
 
 def build_model(device, seed=2):
-    """Random init of the d26 architecture directly on the GPU (same distributions as the reference's
-    init_weights, with non-zero projections so every kernel does real work)."""
-    from nanochat_amd.fp8 import convert_to_float8_training, fp8_module_filter
-    from nanochat_amd.gpt import GPT, GPTConfig
-    cfg = GPTConfig(**D26)
-    with torch.device("meta"):
-        model = GPT(cfg)
-    model.to_empty(device=device)
-    g = torch.Generator(device=device).manual_seed(seed)
-    s = 3 ** 0.5 * cfg.n_embd ** -0.5
-    with torch.no_grad():
-        for name, p in model.named_parameters():
-            if name.endswith("wte.weight"):
-                p.normal_(0.0, 0.8, generator=g)
-            elif name == "lm_head.weight":
-                p.normal_(0.0, 0.03, generator=g)
-            elif "value_embeds" in name or "c_q" in name or "c_k" in name or "c_v" in name or "attn.c_proj" in name:
-                p.uniform_(-s, s, generator=g)
-            elif "c_fc" in name:
-                p.uniform_(-0.4 * s, 0.4 * s, generator=g)
-            elif "mlp.c_proj" in name:
-                p.uniform_(-0.5 * s, 0.5 * s, generator=g)
-            elif "gate" in name:
-                p.uniform_(-0.5, 0.5, generator=g)
-            elif name == "resid_lambdas":
-                p.copy_(torch.linspace(1.15, 1.05, cfg.n_layer))
-            elif name == "x0_lambdas":
-                p.copy_(torch.linspace(0.20, 0.05, cfg.n_layer))
-            elif name == "smear_lambda":
-                p.fill_(0.35)
-            elif name == "backout_lambda":
-                p.fill_(0.2)
-            else:
-                raise RuntimeError(f"unhandled parameter {name}")
-        # bf16 weights with FP8 linears
-        model.to(torch.bfloat16)
-    convert_to_float8_training(model, module_filter_fn=fp8_module_filter)
-    return model
+    """Random init of the d26 architecture directly on the GPU, bf16 weights with FP8 linears."""
+    from nanochat_amd.gpt import GPTConfig
+    from nanochat_amd.synthetic import random_init_model
+    return random_init_model(GPTConfig(**D26), device, seed)
 
 
 def attention_bytes_per_step(model, batch, context):

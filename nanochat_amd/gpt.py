@@ -129,6 +129,15 @@ class GPT(nn.Module):
         attn = sum(4 * h * q * min(context_len, w) for w, _ in self.window_sizes)
         return 2 * self.num_matmul_params() + attn
 
+    def estimate_prefill_flops(self, num_tokens):
+        """Causal prefill: token t attends to min(t, window) keys in every layer (gpt.py:362-372)."""
+        h, q = self.config.n_head, self.config.n_embd // self.config.n_head
+        attn = 0
+        for window, _ in self.window_sizes:
+            w = min(window, num_tokens)
+            attn += 4 * h * q * (w * (w + 1) // 2 + (num_tokens - w) * w)
+        return 2 * self.num_matmul_params() * num_tokens + attn
+
     def kv_bytes_per_token(self):
         D = self.config.n_embd // self.config.n_head
         return self.config.n_layer * 2 * self.config.n_kv_head * D * 2
