@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE.json configs[3]): nanochat d26 (n_embd 1664, 13 heads, head_dim 128, 26 layers,
+Workload (the headline decode configuration): nanochat d26 (n_embd 1664, 13 heads, head_dim 128, 26 layers,
 vocab 32768, window pattern SSSL), bf16 weights with FP8 linears, random init seed 2; one prompt of
 random token ids is prefilled at batch 1, the KV cache is replicated to 64 rows, and greedy decoding
 runs through Engine.generate until the context reaches 2048 tokens.  A "step" is one iteration of that
@@ -193,7 +193,7 @@ def main():
                          "(a kernel of known traffic to scale hardware byte counters with)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (decode shards by batch row; see DESIGN.md). "
+        print("bench.py measures one GPU: this build has no multi-GPU path (decode would shard by batch row, one independent copy per GPU). "
               "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     assert torch.cuda.is_available(), "bench.py needs the GPU"

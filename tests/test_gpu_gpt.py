@@ -2,7 +2,7 @@
 against the CPU oracle on the same seeded weights and inputs.
 
 Bars.
-  * Repository init (BASELINE config 1: zero-initialised projections, lm_head std 0.001 -- the weights the
+  * Repository init (the reference's own init_weights: zero-initialised projections, lm_head std 0.001 -- the weights the
     stated tolerance is quoted on): logits within 1e-2 abs of the oracle, greedy ids identical to the
     oracle's wherever the oracle's own top-2 margin exceeds the tolerance (bf16 logits tie often and a
     tie is decided by summation order).
@@ -109,7 +109,7 @@ def margin_aware_compare(got_ids, want_ids, want_logits):
 
 
 def test_repo_init_logits_and_greedy_ids(d4_repo_pair):
-    """BASELINE config 1 weights: logits within 1e-2 abs, greedy ids identical for 64 tokens."""
+    """Repository-init weights: logits within 1e-2 abs, greedy ids identical for 64 tokens."""
     say("d4 repo init: prefill logits + 64 greedy tokens")
     rt, model = d4_repo_pair
     from nanochat_amd.engine import KVCache
