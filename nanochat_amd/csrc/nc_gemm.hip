@@ -13,6 +13,7 @@
 //                       placed between the MFMA groups by hand), bf16 epilogue staged through LDS.
 //   gemm_tile_kernel    the same tiling with plain global loads (64-bit addressing) for operands past 2 GiB.
 //   M <= 128 (decode) is weight-bandwidth bound and handled by gemm_decode_kernel in nc_gemm_decode.hip.
+#include <type_traits>
 #include "nc_common.h"
 #include "nc_kernels.h"
 
@@ -448,6 +449,313 @@ static int launch_bl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep,
 
 
 // ------------------------------------------------------------------------------------------------
+// Direct-to-LDS kernels: 256x256x128 tiles, 8 waves (4 x 2, 64x128 outputs each), one workgroup per CU.  The operand
+// tiles never pass through registers: every wave issues eight 1 KB `buffer_load_dwordx4 ... lds` per K-step, each of
+// which lands 8 rows x 128 bytes in consecutive LDS; the swizzle of the LDS layout (chunk c of row r at slot
+// c ^ NC_SWZ(r)) is applied on the global side, lane (sub, slot) fetching chunk slot ^ NC_SWZ(row) of its row, so each
+// group of 8 lanes still reads one whole 128-byte line.  That removes the ds_write phase (a 64 KB stage costs ~860
+// cycles at the 76 B/clk LDS write rate, next to 2048 cycles of MFMA) and the staging registers.  K must be a multiple
+// of 128 (a K tail would need zero fill inside rows, which the range check of the descriptor cannot give); bf16 output.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+struct DlGeom {
+    int lane, wave, wm, wn, frow, kb;
+    int sub, gch;          // this lane's row inside an 8-row block and the global chunk that belongs in its LDS slot
+    int rd_lo, rd_hi;      // fragment read offsets inside a 16-row block
+};
+__device__ __forceinline__ DlGeom dl_geom() {
+    DlGeom g;
+    g.lane = threadIdx.x & 63, g.wave = threadIdx.x / 64;
+    g.wm = g.wave / 2, g.wn = g.wave % 2;
+    g.frow = g.lane & 15, g.kb = g.lane >> 4;
+    g.sub = g.lane >> 3, g.gch = (g.lane & 7) ^ g.sub ^ (g.wave & 1);
+    const int sw = NC_SWZ(g.frow);
+    g.rd_lo = g.frow * 128 + (((2 * g.kb) ^ sw) << 4), g.rd_hi = g.frow * 128 + (((2 * g.kb + 1) ^ sw) << 4);
+    return g;
+}
+__device__ __forceinline__ v8i dl_frag(const uint8_t* base, const DlGeom& g) {
+    const v4i lo = *(const v4i*)(base + g.rd_lo);
+    const v4i hi = *(const v4i*)(base + g.rd_hi);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+// FIRST starts the accumulation from zero (C operand 0) instead of reading the accumulators.
+__device__ __forceinline__ void mfma_f8_first_ordered(v4f& acc, const v8i& b, const v8i& a) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a) : "memory");
+}
+// One K-step of a wave: 64 rows x (128 or, for a half-width tile, 64) columns from the stage at `st`.
+template <bool HALF, bool FIRST = false>
+__device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, const DlGeom& g) {
+    constexpr int WTN = HALF ? 4 : 8;
+    const uint8_t* a = st + g.wm * 64 * 128;
+    const uint8_t* b = st + 256 * 128 + g.wn * (HALF ? 64 : 128) * 128;
+    v8i af[4], bf[2];
+    bf[0] = dl_frag(b, g);
+#pragma unroll
+    for (int i = 0; i < 4; i++) af[i] = dl_frag(a + i * 2048, g);
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        if (j + 1 < WTN) bf[(j + 1) & 1] = dl_frag(b + (j + 1) * 2048, g);    // one group ahead of its use
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (FIRST) mfma_f8_first_ordered(acc[i][j], bf[j & 1], af[i]);
+            else mfma_f8_acc_ordered(acc[i][j], bf[j & 1], af[i]);
+        }
+    }
+}
+
+// One tile per workgroup, launched tile by tile (any M, N).
+__global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep, int M,
+                                                      int N, int K, int tiles_m, int tiles_n) {
+    constexpr int STAGE = 512 * 128;
+    extern __shared__ __align__(16) uint8_t lds[];
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * 256;
+    const DlGeom g = dl_geom();
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, M * K, 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, N * K, 0x00020000);
+
+    // piece i of this wave is the 1 KB block (wave + 8 i) of the stage: tile rows 8 wave + 64 i + sub, A for i < 4, B after
+    uint32_t vo[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int ra = m0 + 8 * g.wave + 64 * i + g.sub, rb = n0 + 8 * g.wave + 64 * i + g.sub;
+        vo[i] = ra < M ? (uint32_t)ra * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+        vo[4 + i] = rb < N ? (uint32_t)rb * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+    }
+    const int ksteps = K / 128;
+
+    v4f acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto fetch = [&](int t, int buf) {
+        if (t < ksteps) {
+            uint8_t* st = lds + buf * STAGE + g.wave * 1024;
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 4 ? desc_a : desc_b, (lds_ptr_t)(st + i * 8192), 16, vo[i], t * 128, 0, 0);
+        }
+    };
+    // step kt computes from buffer kt & 1 while the loads of step kt + 1 land in the other one; the barrier at its end
+    // says both that those loads are complete for every wave and that nobody reads buffer kt & 1 any more
+    fetch(0, 0);
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < ksteps; kt += 2) {
+        fetch(kt + 1, 1);
+        dl_compute<false>(acc, lds, g);
+        __syncthreads();
+        fetch(kt + 2, 0);
+        dl_compute<false>(acc, lds + STAGE, g);
+        __syncthreads();
+    }
+    if (kt < ksteps) dl_compute<false>(acc, lds, g);
+
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) asm volatile("" : "+a"(acc[i][j]));
+    const float inv_a = *ep.inv_a;
+    float sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
+    bl_epilogue<256, 256, 4, 2, 0>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
+}
+
+// Epilogue of the persistent kernel: the wave's 64 x (128 | 64) block leaves 16 rows at a time through a 4 KB LDS region of
+// its own (past the two operand stages, so the loads of the next tile keep landing meanwhile), every store instruction
+// writing whole 128-byte lines.
+template <bool HALF>
+__device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, const EpilogueArgs& ep, float inv_a, const float (&sc)[4],
+                                             const DlGeom& g, int m0, int n0, int M, int N) {
+    constexpr int WTN = HALF ? 4 : 8, WCOLS = WTN * 16, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
+    const bool vec16 = (ep.ldc % 8 == 0) && (((uintptr_t)ep.out & 15) == 0);
+    const int lrow_e = g.lane / LPR, c = g.lane % LPR;
+    const int n_st = n0 + g.wn * WCOLS + c * 8;
+    float inv_b[WTN];
+#pragma unroll
+    for (int j = 0; j < WTN; j++) {
+        const int n = n0 + g.wn * WCOLS + j * 16 + 4 * g.kb;
+        inv_b[j] = sc[0];
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            if (i + 1 < ep.segs.nseg && n >= ep.segs.end[i]) inv_b[j] = sc[i + 1];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < WTN; j++) {
+            const int chunk = 2 * j + (g.kb >> 1);
+            const v4f a4 = acc[i][j];
+            const uint2 pk = make_uint2(pack_bf16_hw((a4[0] * inv_a) * inv_b[j], (a4[1] * inv_a) * inv_b[j]),
+                                        pack_bf16_hw((a4[2] * inv_a) * inv_b[j], (a4[3] * inv_a) * inv_b[j]));
+            *(uint2*)(reg + g.frow * ROWB + ((chunk ^ (g.frow & 7)) << 4) + (g.kb & 1) * 8) = pk;
+        }
+        // the region is private to the wave: its own LDS writes only have to land before its reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0xc07f);                    // lgkmcnt(0)
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int it = 0; it < 16 / RPI; it++) {
+            const int row = it * RPI + lrow_e;
+            const int m = m0 + g.wm * 64 + i * 16 + row;
+            const uint4 v = *(const uint4*)(reg + row * ROWB + ((c ^ (row & 7)) << 4));
+            if (m >= M || n_st >= N) continue;
+            bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n_st;
+            if (n_st + 8 <= N) {
+                if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
+                else {
+                    *(uint2*)o = make_uint2(v.x, v.y);
+                    *(uint2*)(o + 4) = make_uint2(v.z, v.w);
+                }
+            } else {
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                for (int r = 0; r < 8 && n_st + r < N; r++) o[r] = (bf16_t)(w[r >> 1] >> ((r & 1) * 16));
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads are done before the next 16 rows overwrite the region
+    }
+}
+
+// Persistent form: 8 x 32 workgroups, each walking its own list of tiles as one uninterrupted stream of K-steps (the
+// first loads of the next tile are in flight while the current one is finished and stored).  XCD x (workgroup id % 8)
+// owns `rows_per_xcd` consecutive tile rows; its 32 workgroups form rows_per_xcd x (32 / rows_per_xcd) slots, slot
+// (r, c) owning tile row r and the c-th share of the N range counted in 128-column units.  A share is cut into full
+// 256-column tiles plus, when its unit count is odd, one half-width tile at its end, so no workgroup rounds its work up
+// to whole 256x256 tiles.
+__global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep,
+                                                       int M, int N, int K, int rows_per_xcd, int nu) {
+    constexpr int STAGE = 512 * 128;
+    extern __shared__ __align__(16) uint8_t lds[];
+    const DlGeom g = dl_geom();
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int cols = 32 / rows_per_xcd;
+    const int sc_c = slot % cols, sc_r = slot / cols;
+    const int m0 = (xcd * rows_per_xcd + sc_r) * 256;
+    const int ub = nu * sc_c / cols, ue = nu * (sc_c + 1) / cols;
+    const int count = ue - ub, nitems = (count + 1) / 2;
+    const bool has_half = count & 1;
+    if (nitems == 0) return;
+    auto item = [&](int q, int& n0, bool& half) {
+        half = has_half && q == nitems - 1;
+        n0 = (ub + 2 * q) * 128;
+    };
+
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, M * K, 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, N * K, 0x00020000);
+    const int ksteps = K / 128;
+    uint32_t vo_a[4], vo_b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int ra = m0 + 8 * g.wave + 64 * i + g.sub;
+        vo_a[i] = ra < M ? (uint32_t)ra * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+    }
+    // the fetch cursor runs ahead of the compute cursor, across tile boundaries
+    int fq = 0, fkt = 0, fbuf = 0;
+    bool f_half = false;
+    auto set_fetch_item = [&](int q) {
+        int n0;
+        item(q, n0, f_half);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int rb = n0 + 8 * g.wave + 64 * i + g.sub;
+            vo_b[i] = rb < N ? (uint32_t)rb * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+        }
+    };
+    auto fetch_next = [&]() {
+        if (fq >= nitems) return;
+        uint8_t* st = lds + fbuf * STAGE + g.wave * 1024;
+#pragma unroll
+        for (int i = 0; i < 4; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (lds_ptr_t)(st + i * 8192), 16, vo_a[i], fkt * 128, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 2; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b, (lds_ptr_t)(st + (4 + i) * 8192), 16, vo_b[i], fkt * 128, 0, 0);
+        if (!f_half) {
+#pragma unroll
+            for (int i = 2; i < 4; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b, (lds_ptr_t)(st + (4 + i) * 8192), 16, vo_b[i], fkt * 128, 0, 0);
+        }
+        fbuf ^= 1;
+        if (++fkt == ksteps) {
+            fkt = 0;
+            if (++fq < nitems) set_fetch_item(fq);
+        }
+    };
+
+    const float inv_a = *ep.inv_a;
+    float sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
+    uint8_t* epi = lds + 2 * STAGE + g.wave * 4096;
+
+    // Invariant at the top of every K-step: its own operands have landed (the barrier before it) and the loads of the step
+    // after it are already in flight.  After the barrier that ends a step, its buffer is free and takes the loads of
+    // the step after next; at the end of a tile those are the next tile's, and they travel while the tile is stored.
+    set_fetch_item(0);
+    fetch_next();
+    __syncthreads();
+    fetch_next();
+    int buf = 0;
+    auto tile = [&](int n0, auto half_tag) {
+        constexpr bool HALF = decltype(half_tag)::value;
+        v4f acc[4][8];
+        dl_compute<HALF, true>(acc, lds + buf * STAGE, g);
+        __syncthreads();
+        buf ^= 1;
+        fetch_next();
+        for (int kt = 1; kt < ksteps; kt++) {
+            dl_compute<HALF, false>(acc, lds + buf * STAGE, g);
+            __syncthreads();
+            buf ^= 1;
+            fetch_next();
+        }
+        // the last MFMAs must have left the pipeline before the accumulators are read
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < (HALF ? 4 : 8); j++) asm volatile("" : "+a"(acc[i][j]));
+        int m0_here = m0;
+        asm volatile("" : "+s"(m0_here));          // keeps the store addresses of all tiles from being precomputed (and spilled)
+        dlp_epilogue<HALF>(acc, epi, ep, inv_a, sc, g, m0_here, n0, M, N);
+    };
+    for (int q = 0; q < nitems; q++) {
+        int n0;
+        bool half;
+        item(q, n0, half);
+        if (half) tile(n0, std::true_type{});
+        else tile(n0, std::false_type{});
+    }
+}
+
+static bool dlp_eligible(int M, int N, int K) {
+    const int tiles_m = (M + 255) / 256;
+    if (K % 128 != 0 || tiles_m % 8 != 0) return false;
+    const int rx = tiles_m / 8;
+    return rx >= 1 && rx <= 32 && (rx & (rx - 1)) == 0;
+}
+
+static int launch_dl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
+    NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
+    NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
+    NC_CHECK_ARG(ep.out_kind == 0, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    const size_t lds_bytes = 2 * 512 * 128 + (persistent ? 8 * 4096 : 0);
+    const void* fn = persistent ? (const void*)gemm_dlp_kernel : (const void*)gemm_dl_kernel;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    if (persistent) {
+        NC_CHECK_ARG(dlp_eligible(M, N, K), "fp8_gemm: the persistent kernel needs M/256 (rounded up) to be 8, 16, ... 256 tile rows, got M=%d", M);
+        hipLaunchKernelGGL(gemm_dlp_kernel, dim3(256), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m / 8, (N + 127) / 128);
+    } else {
+        hipLaunchKernelGGL(gemm_dl_kernel, dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
 template <int BM, int BN>
 static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
@@ -496,7 +804,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         }
     }
     int rc = 0;
-    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 7, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 9, "fp8_gemm: unknown kernel selector %d", force_kernel);
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
@@ -515,6 +823,8 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     else if (which == 5) rc = launch_bl<128, 128, 2, 2, true>(a, b, ep, M, N, K, s);
     else if (which == 6) rc = launch_bl<256, 128, 4, 2, false>(a, b, ep, M, N, K, s);
     else if (which == 7) rc = launch_bl<256, 256, 4, 2, false>(a, b, ep, M, N, K, s);
+    else if (which == 8) rc = launch_dl(a, b, ep, M, N, K, false, s);
+    else if (which == 9) rc = launch_dl(a, b, ep, M, N, K, true, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");
