@@ -11,6 +11,8 @@
 //   gemm_bl_kernel      M large (prefill, isolated Float8Linear): BMxBNx128 tiles, double-buffered swizzled LDS fed
 //                       through two register stages of buffer loads (for the 128x128 tile the fills and loads are
 //                       placed between the MFMA groups by hand), bf16 epilogue staged through LDS.
+//   gemm_dl_kernel      256x256x128 tiles whose operands go from global memory straight into LDS (no staging registers,
+//   gemm_dlp_kernel     no LDS fill instructions); the second is the persistent form for shapes of several rounds of tiles.
 //   gemm_tile_kernel    the same tiling with plain global loads (64-bit addressing) for operands past 2 GiB.
 //   M <= 128 (decode) is weight-bandwidth bound and handled by gemm_decode_kernel in nc_gemm_decode.hip.
 #include <type_traits>
@@ -788,19 +790,27 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     if (M == 0) return 0;
     EpilogueArgs ep{inv_a, inv_b, segs, out, out_kind, softcap, ldc};
 
-    // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256
+    // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256,
+    // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent
     int which = force_kernel;
     if (which == 0) {
         if (M <= 128) which = 1;
         else if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31)) which = 4;   // past the 32-bit buffer offsets
         else {
-            // 256x256 tiles move half the bytes per flop through L2 and LDS but run one workgroup per CU: take them
-            // when their count fills whole rounds of the CUs well, else the 128x128 tiles (two workgroups per CU)
             int dev = 0, cus = 256;
-            if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             const long rounds = (t256 + cus - 1) / cus;
-            which = (M >= 1024 && N >= 512 && 10 * t256 >= 8 * rounds * cus && rounds <= 2) ? 7 : 5;
+            if (out_kind == 0 && K % 128 == 0 && 2 * t256 >= cus) {
+                // 256x256 tiles fed straight into LDS whenever they occupy at least half of the CUs (below that the
+                // 128x128 tiles, four times as many, fill the chip better); from two rounds of tiles on, the
+                // persistent form, which neither rounds the last round up nor pays a prologue per tile
+                which = (t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8;
+            } else {
+                // 256x256 tiles move half the bytes per flop through L2 and LDS but run one workgroup per CU: take them
+                // when their count fills whole rounds of the CUs well, else the 128x128 tiles (two workgroups per CU)
+                which = (M >= 1024 && N >= 512 && 10 * t256 >= 8 * rounds * cus && rounds <= 2) ? 7 : 5;
+            }
         }
     }
     int rc = 0;

@@ -123,6 +123,13 @@ def make_operands(M, N, K, seed, outliers=True):
     (300, 320, 256, 5), (300, 320, 400, 5), (513, 272, 1664, 5), (257, 144, 16, 5), (2100, 1300, 400, 5),
     (300, 320, 384, 6), (640, 528, 912, 6), (300, 320, 128, 6), (5000, 1100, 144, 6),
     (300, 320, 256, 7), (300, 320, 80, 7), (513, 272, 1664, 7), (4100, 2100, 272, 7),
+    # direct-to-LDS tiles, launched tile by tile: ragged M and N, one K-step, odd and even step counts
+    (300, 320, 256, 8), (256, 256, 128, 8), (513, 272, 1664, 8), (4100, 2100, 384, 8), (1000, 1000, 512, 8),
+    # the persistent form: 8..64 tile rows, ragged last tile row, N below / not a multiple of the 128-column unit,
+    # fewer units than column slots (idle workgroups), odd and even unit counts per slot
+    (2048, 1664, 256, 9), (2000, 1000, 384, 9), (1800, 72, 128, 9), (4096, 4992, 128, 9), (3900, 6656, 256, 9),
+    (8192, 1664, 384, 9), (8192, 4992, 128, 9), (16384, 392, 256, 9),
+    (2048, 6656, 1664, 0), (8192, 4992, 256, 0),
 ])
 def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     say(f"gemm M={M} N={N} K={K} kernel={kernel}")
@@ -140,7 +147,7 @@ def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     assert rel_l2(got, exact) < 0.08
 
 
-@pytest.mark.parametrize("kernel,M", [(1, 48), (4, 128), (5, 256), (6, 128), (7, 256)])
+@pytest.mark.parametrize("kernel,M", [(1, 48), (4, 128), (5, 256), (6, 128), (7, 256), (8, 256), (9, 2048)])
 def test_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
     say(f"gemm exact powers of two kernel={kernel}")
     g = torch.Generator().manual_seed(9)
@@ -184,6 +191,13 @@ def test_gemm_stacked_weights_use_their_own_scales(ops):
     for kernel, Muse in [(1, 64), (4, 64)]:
         got = ops.fp8_gemm(a8.to(DEV), w8.to(DEV), ia.to(DEV), inv_w.to(DEV), seg_ends=[256, 384, 512], kernel=kernel).cpu()
         assert rel_l2(got, want) < 2e-3
+    # the large-M kernels: the same three segments under 2048 rows (segment ends inside a tile and inside a half tile)
+    a_big = torch.randn(2048, K, generator=g).bfloat16()
+    a8b, iab, _ = fp8_ref.to_fp8(a_big)
+    want_big = torch.cat([fp8_ref.scaled_mm_emulated(a8b, p, iab, inv) for p, inv, _ in q], dim=1)
+    for kernel in (5, 7, 8, 9):
+        got = ops.fp8_gemm(a8b.to(DEV), w8.to(DEV), iab.to(DEV), inv_w.to(DEV), seg_ends=[256, 384, 512], kernel=kernel).cpu()
+        assert rel_l2(got, want_big) < 2e-3, kernel
 
 
 def test_gemm_softcap_epilogue(ops):
