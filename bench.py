@@ -72,8 +72,10 @@ def read_profile(lib, cls):
     return ms.value, units.value, n.value
 
 
-def gemm_rates(device):
-    """FP8 GEMM TFLOP/s at the isolated Float8Linear shapes (M=8192), kernel time by HIP events."""
+def gemm_rates(device, library_gemm=False):
+    """FP8 GEMM TFLOP/s at the isolated Float8Linear shapes (M=8192), kernel time by HIP events.  With library_gemm, the
+    ROCm library GEMM behind torch._scaled_mm (the reference's own call, nanochat/fp8.py:143-153) is timed on the same operands
+    beside it, torch events around the same 60 + 100 launches."""
     from nanochat_amd import _lib, ops
     lib = _lib.lib()
     out = {}
@@ -106,6 +108,24 @@ def gemm_rates(device):
         out[f"K{K}_N{N}"] = {"us": round(ms / n * 1e3, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
                              "quantize_us": round(qms / qn * 1e3, 2),
                              "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1)}
+        if library_gemm:
+            sa, sw = ia.reshape(()).float(), iw.reshape(()).float()
+            a8t, w8t = a8.view(torch.float8_e4m3fn), w8.view(torch.float8_e4m3fn).t()
+
+            def call():
+                return torch._scaled_mm(a8t, w8t, scale_a=sa, scale_b=sw, out_dtype=torch.bfloat16, use_fast_accum=True)
+            for _ in range(60):
+                ref = call()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(100):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 10.0
+            out[f"K{K}_N{N}"]["library_us"] = round(us, 2)
+            out[f"K{K}_N{N}"]["library_tflops"] = round(2.0 * M * N * K / us / 1e6, 1)
+            out[f"K{K}_N{N}"]["rel_l2_vs_library"] = float(((res.float() - ref.float()).norm() / ref.float().norm()).item())
     return out
 
 
@@ -187,6 +207,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--library-gemm", action="store_true", help="also time torch._scaled_mm on the M=8192 GEMM operands")
     ap.add_argument("--profile-steps", type=int, default=16)
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="after the decode steps, run an elementwise pass that reads and writes this many MiB "
@@ -287,7 +308,7 @@ def main():
         "kernel_ms_per_step": per_step_ms,
     }
     if not args.no_gemm:
-        result["fp8_gemm_m8192"] = gemm_rates(device)
+        result["fp8_gemm_m8192"] = gemm_rates(device, args.library_gemm)
     del gen, engine, model
     torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
