@@ -108,6 +108,31 @@ def gemm_rates(device, library_gemm=False):
         out[f"K{K}_N{N}"] = {"us": round(ms / n * 1e3, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
                              "quantize_us": round(qms / qn * 1e3, 2),
                              "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1)}
+        # the two backward GEMMs of the same layer (nanochat/fp8.py:156-192): e5m2 gradient x e4m3 saved operands
+        go = (torch.randn(M, N, device=device, generator=g) * 1e-3).bfloat16()
+
+        def timed(fn, warm=30, n=50):
+            for _ in range(warm):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / n
+        go8, igo, _ = ops.fp8_quantize(go, fp8_dtype=torch.float8_e5m2)
+        wT, goT, xT = ops.fp8_transpose(w8), ops.fp8_transpose(go8), ops.fp8_transpose(a8)
+        gi = torch.empty(M, K, dtype=torch.bfloat16, device=device)
+        gw = torch.empty(N, K, dtype=torch.bfloat16, device=device)
+        dx_us = timed(lambda: ops.fp8_gemm_grad(go8, wT, igo, iw, out=gi))
+        dw_us = timed(lambda: ops.fp8_gemm_grad(goT, xT, igo, ia, out=gw))
+        prep_us = timed(lambda: (ops.fp8_quantize(go, fp8_dtype=torch.float8_e5m2), ops.fp8_transpose(w8), ops.fp8_transpose(go8),
+                                 ops.fp8_transpose(a8)), warm=10, n=20)
+        out[f"K{K}_N{N}"]["backward"] = {"grad_input_us": round(dx_us, 2), "grad_weight_us": round(dw_us, 2),
+                                         "grad_input_tflops": round(2.0 * M * N * K / dx_us / 1e6, 1),
+                                         "grad_weight_tflops": round(2.0 * M * N * K / dw_us / 1e6, 1),
+                                         "quantize_and_transposes_us": round(prep_us, 2)}
         if library_gemm:
             sa, sw = ia.reshape(()).float(), iw.reshape(()).float()
             a8t, w8t = a8.view(torch.float8_e4m3fn), w8.view(torch.float8_e4m3fn).t()

@@ -37,6 +37,18 @@ int nc_fp8_quantize_tensorwise(const void* x, int x_dtype, int64_t n, uint8_t* o
 int nc_e4m3_encode_with_scale(const uint16_t* x, int64_t n, float scale, uint8_t* out, int encoder,
                               nc_stream_t stream);
 
+/* The same with the fp8 format as a parameter: fp8_format 0 = e4m3fn (activations, weights), 1 = e5m2 (OCP, the
+ * encoding of torch.float8_e5m2; saturates at 57344), which nanochat/fp8.py:165 uses for the output gradient. */
+int nc_fp8_quantize_tensorwise_as(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
+                                  float* inv_scale_out, uint32_t* amax_ws, int encoder, nc_stream_t stream);
+int nc_fp8_encode_with_scale(const uint16_t* x, int64_t n, float scale, int fp8_format, uint8_t* out, int encoder,
+                             nc_stream_t stream);
+
+/* dst[cols][rows] = transpose of the fp8 payload src[rows][cols]: the memory rearrangement of _to_col_major and
+ * .t().contiguous() at nanochat/fp8.py:110-118,169,181-182 (the backward GEMMs want the summed index contiguous in
+ * both operands).  rows and cols multiples of 16, pointers 16-byte aligned. */
+int nc_fp8_transpose(const uint8_t* src, int rows, int cols, uint8_t* dst, nc_stream_t stream);
+
 /* (2) FP8 scaled GEMM: torch._scaled_mm as called at nanochat/fp8.py:143-153.
  * out[M,N] = bf16((a[M,K] . b[N,K]^T, fp32 accumulate) * *inv_a * inv_b[seg(n)]).
  * b may stack up to 4 weight matrices along N; seg_ends (HOST array of nseg exclusive column ends)
@@ -57,6 +69,15 @@ int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const
  * bits of max|a|, e.g. produced by nc_rmsnorm / nc_mix_norm / nc_decode_attention), bit-identical to
  * nc_fp8_quantize_tensorwise followed by nc_fp8_gemm_tn.  out_kind 0/1 as above; out_kind 2 writes
  * bf16 relu(bf16(v))^2 (nanochat/gpt.py:139) and max-reduces it into *out_amax.  ksplits 0 = choose. */
+/* The backward GEMMs of nanochat/fp8.py:166-190 (torch._scaled_mm with an e5m2 first operand):
+ * out[M,N] = bf16((a[M,K] . b[N,K]^T, fp32 accumulate) * *inv_a * *inv_b), a in e5m2 (the quantized output gradient or
+ * its transpose), b in e4m3fn (the transposed weight or input payload saved by the forward), K contiguous in both.
+ *   grad_input [B,K']  = nc_fp8_gemm_tn_grad(go[B,N'],   wT[K',N'], ...)   M=B,  N=K', K=N'
+ *   grad_weight[N',K'] = nc_fp8_gemm_tn_grad(goT[N',B],  xT[K',B],  ...)   M=N', N=K', K=B
+ * kernel: 0 auto, 5 (128x128 tiles, any K multiple of 16), 8 / 9 (direct-to-LDS 256x256 tiles, K multiple of 128). */
+int nc_fp8_gemm_tn_grad(const uint8_t* a_e5m2, const uint8_t* b, const float* inv_a, const float* inv_b, void* out, int M,
+                        int N, int K, int ldc, int kernel, nc_stream_t stream);
+
 size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K);
 int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const uint8_t* b, const float* inv_b,
                           const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap,

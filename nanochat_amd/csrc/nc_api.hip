@@ -23,12 +23,27 @@ const char* nc_last_error(void) { return g_error; }
 int nc_fp8_quantize_tensorwise(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_scale_out,
                                uint32_t* amax_ws, int encoder, nc_stream_t stream) {
     NC_CHECK_ARG(encoder == 0 || encoder == 1, "fp8_quantize: encoder must be 0 (hardware) or 1 (software)");
-    return nc_launch_quantize(x, x_dtype, n, out, scale_out, inv_scale_out, amax_ws, encoder, (hipStream_t)stream);
+    return nc_launch_quantize(x, x_dtype, n, 0, out, scale_out, inv_scale_out, amax_ws, encoder, (hipStream_t)stream);
+}
+
+int nc_fp8_quantize_tensorwise_as(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
+                                  float* inv_scale_out, uint32_t* amax_ws, int encoder, nc_stream_t stream) {
+    NC_CHECK_ARG(encoder == 0 || encoder == 1, "fp8_quantize: encoder must be 0 (hardware) or 1 (software)");
+    return nc_launch_quantize(x, x_dtype, n, fp8_format, out, scale_out, inv_scale_out, amax_ws, encoder, (hipStream_t)stream);
+}
+
+int nc_fp8_encode_with_scale(const uint16_t* x, int64_t n, float scale, int fp8_format, uint8_t* out, int encoder, nc_stream_t stream) {
+    NC_CHECK_ARG(encoder == 0 || encoder == 1, "fp8_encode: encoder must be 0 (hardware) or 1 (software)");
+    return nc_launch_encode_with_scale(x, n, scale, fp8_format, out, encoder, (hipStream_t)stream);
+}
+
+int nc_fp8_transpose(const uint8_t* src, int rows, int cols, uint8_t* dst, nc_stream_t stream) {
+    return nc_launch_transpose_u8(src, rows, cols, dst, (hipStream_t)stream);
 }
 
 int nc_e4m3_encode_with_scale(const uint16_t* x, int64_t n, float scale, uint8_t* out, int encoder, nc_stream_t stream) {
     NC_CHECK_ARG(encoder == 0 || encoder == 1, "e4m3_encode: encoder must be 0 (hardware) or 1 (software)");
-    return nc_launch_encode_with_scale(x, n, scale, out, encoder, (hipStream_t)stream);
+    return nc_launch_encode_with_scale(x, n, scale, 0, out, encoder, (hipStream_t)stream);
 }
 
 static int segs_from(const int32_t* seg_ends, int nseg, int N, NcGemmSegs* segs) {
@@ -48,6 +63,12 @@ int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     if (int rc = segs_from(seg_ends, nseg, N, &segs)) return rc;
     return nc_launch_gemm(a, b, inv_a, inv_b, segs, out, out_kind, softcap, M, N, K, ldc, kernel, workspace, workspace_bytes,
                           (hipStream_t)stream);
+}
+
+int nc_fp8_gemm_tn_grad(const uint8_t* a_e5m2, const uint8_t* b, const float* inv_a, const float* inv_b, void* out, int M, int N, int K,
+                        int ldc, int kernel, nc_stream_t stream) {
+    NcGemmSegs segs{1, {N, 0, 0, 0}};
+    return nc_launch_gemm(a_e5m2, b, inv_a, inv_b, segs, out, 0, 0.f, M, N, K, ldc, kernel, nullptr, 0, (hipStream_t)stream, 1);
 }
 
 size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K) {

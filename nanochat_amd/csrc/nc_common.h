@@ -83,11 +83,43 @@ __device__ __forceinline__ uint32_t e4m3_pack4_sw(float a, float b, float c, flo
 }
 __device__ __forceinline__ float clamp448(float y) { return fminf(fmaxf(y, -448.0f), 448.0f); }
 
+// ---------------------------------------------------------------- e5m2 (OCP) encode: the gradient format of nanochat/fp8.py:165
+// |y| must already be clamped to <= 57344.  Round to nearest even, subnormals down to 2^-16.  e5m2 is the top byte of fp16.
+__device__ __forceinline__ uint32_t e5m2_encode_sw(float y) {
+    uint32_t u = __float_as_uint(y);
+    uint32_t sign = (u >> 24) & 0x80u;
+    u &= 0x7fffffffu;
+    uint32_t out;
+    if (u >= 0x38800000u) {                      // >= 2^-14: normal in e5m2
+        u += 0xfffffu + ((u >> 21) & 1u);        // RNE at mantissa bit 21
+        out = (u >> 21) - ((127u - 15u) << 2);
+    } else {                                     // subnormal: multiples of 2^-16
+        float m = __uint_as_float(u) * 65536.0f; // exact
+        out = (uint32_t)__builtin_rintf(m);      // 0..4, ties to even; 4 == 0x04 == 2^-14
+    }
+    return sign | out;
+}
+__device__ __forceinline__ uint32_t e5m2_pack4_hw(float a, float b, float c, float d) {
+    int r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+    return (uint32_t)r;
+}
+__device__ __forceinline__ uint32_t e5m2_pack4_sw(float a, float b, float c, float d) {
+    return e5m2_encode_sw(a) | (e5m2_encode_sw(b) << 8) | (e5m2_encode_sw(c) << 16) | (e5m2_encode_sw(d) << 24);
+}
+// FMT 0 = e4m3fn (max 448), 1 = e5m2 (max 57344)
+template <int FMT> __device__ __forceinline__ float fp8_max() { return FMT == 0 ? 448.0f : 57344.0f; }
+template <int FMT> __device__ __forceinline__ float fp8_clamp(float y) { return fminf(fmaxf(y, -fp8_max<FMT>()), fp8_max<FMT>()); }
+template <int FMT, bool HW> __device__ __forceinline__ uint32_t fp8_pack4(float a, float b, float c, float d) {
+    if (FMT == 0) return HW ? e4m3_pack4_hw(a, b, c, d) : e4m3_pack4_sw(a, b, c, d);
+    return HW ? e5m2_pack4_hw(a, b, c, d) : e5m2_pack4_sw(a, b, c, d);
+}
+
 // scale = fp32(448 / max(fp64(amax), 1e-12)) -- the divide is done in fp64 like the reference
-__device__ __forceinline__ float scale_from_amax(float amax) {
+__device__ __forceinline__ float scale_from_amax(float amax, double fmax = 448.0) {
     double d = (double)amax;
     if (d < 1e-12) d = 1e-12;
-    return (float)(448.0 / d);
+    return (float)(fmax / d);
 }
 
 // 16-byte load of data that is read once and is larger than the caches (KV cache, weights at decode time): a

@@ -265,15 +265,21 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
 // Accumulate in place: tying the result to the accumulator operand keeps every 16x16 tile in the same four
 // accumulation registers for the whole K loop (the builtin lets the register allocator pick a different result
 // tuple, which it repairs with dozens of register copies per K-step once the loop is unrolled).
+// A_FMT is the format of the activation-side operand (the instruction's second source, `blgp`): 0 = e4m3, 1 = e5m2, the
+// gradient format of the backward GEMMs (nanochat/fp8.py:165).  The weight-side operand is always e4m3.
+template <int A_FMT = 0>
 __device__ __forceinline__ void mfma_f8_acc(v4f& acc, const v8i& b, const v8i& a) {
-    asm("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+    if (A_FMT == 0) asm("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+    else asm("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+a"(acc) : "v"(b), "v"(a));
 }
 // Same, pinned in program order against every memory operation: used where the LDS fills and global loads of the
 // next steps are placed between groups of MFMAs by hand, so that the LDS, load and matrix pipes work at the same time.
+template <int A_FMT = 0>
 __device__ __forceinline__ void mfma_f8_acc_ordered(v4f& acc, const v8i& b, const v8i& a) {
-    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a) : "memory");
+    if (A_FMT == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a) : "memory");
+    else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+a"(acc) : "v"(b), "v"(a) : "memory");
 }
-template <int BM, int BN, int WGM, int WGN, int OUT_KIND, bool INTERLEAVE = false>
+template <int BM, int BN, int WGM, int WGN, int OUT_KIND, bool INTERLEAVE = false, int A_FMT = 0>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                  EpilogueArgs ep, int M, int N, int K, int tiles_m, int tiles_n) {
     constexpr int NT = 64 * WGM * WGN;
@@ -351,7 +357,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
         for (int j = 0; j < WTN; j++) {
             const v8i bf = frag(st + b_rd + j * 2048);
 #pragma unroll
-            for (int i = 0; i < WTM; i++) mfma_f8_acc(acc[i][j], bf, af[i]);
+            for (int i = 0; i < WTM; i++) mfma_f8_acc<A_FMT>(acc[i][j], bf, af[i]);
         }
     };
     // Step kt computes from LDS buffer kt & 1, then moves tile kt+1 (register slot (kt+1) & 1, loaded two
@@ -389,7 +395,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
                     rb[(BUF) ^ 1][pb] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, cut__ ? NC_BUF_OOB : bvo[pb], t__ * 128, 0); \
                 }                                                                                              \
             }                                                                                                  \
-            _Pragma("unroll") for (int i = 0; i < WTM; i++) mfma_f8_acc_ordered(acc[i][j], bf__[j & 1], af__[i]); \
+            _Pragma("unroll") for (int i = 0; i < WTM; i++) mfma_f8_acc_ordered<A_FMT>(acc[i][j], bf__[j & 1], af__[i]); \
         }                                                                                                      \
         __syncthreads();                                                                                       \
     } while (0)
@@ -434,18 +440,18 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
     bl_epilogue<BM, BN, WGM, WGN, OUT_KIND>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
-template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE = false>
+template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE = false, int A_FMT = 0>
 static int launch_bl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
-    const void* fn = ep.out_kind == 0 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE>;
+    const void* fn = ep.out_kind == 0 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     if (ep.out_kind == 0)
-        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     else
-        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     return 0;
 }
 
@@ -481,11 +487,13 @@ __device__ __forceinline__ v8i dl_frag(const uint8_t* base, const DlGeom& g) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
 // FIRST starts the accumulation from zero (C operand 0) instead of reading the accumulators.
+template <int A_FMT = 0>
 __device__ __forceinline__ void mfma_f8_first_ordered(v4f& acc, const v8i& b, const v8i& a) {
-    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a) : "memory");
+    if (A_FMT == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a) : "memory");
+    else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 blgp:1" : "=a"(acc) : "v"(b), "v"(a) : "memory");
 }
 // One K-step of a wave: 64 rows x (128 or, for a half-width tile, 64) columns from the stage at `st`.
-template <bool HALF, bool FIRST = false>
+template <bool HALF, bool FIRST = false, int A_FMT = 0>
 __device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, const DlGeom& g) {
     constexpr int WTN = HALF ? 4 : 8;
     const uint8_t* a = st + g.wm * 64 * 128;
@@ -499,13 +507,14 @@ __device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, 
         if (j + 1 < WTN) bf[(j + 1) & 1] = dl_frag(b + (j + 1) * 2048, g);    // one group ahead of its use
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            if (FIRST) mfma_f8_first_ordered(acc[i][j], bf[j & 1], af[i]);
-            else mfma_f8_acc_ordered(acc[i][j], bf[j & 1], af[i]);
+            if (FIRST) mfma_f8_first_ordered<A_FMT>(acc[i][j], bf[j & 1], af[i]);
+            else mfma_f8_acc_ordered<A_FMT>(acc[i][j], bf[j & 1], af[i]);
         }
     }
 }
 
 // One tile per workgroup, launched tile by tile (any M, N).
+template <int A_FMT>
 __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep, int M,
                                                       int N, int K, int tiles_m, int tiles_n) {
     constexpr int STAGE = 512 * 128;
@@ -548,13 +557,13 @@ __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict_
     int kt = 0;
     for (; kt + 1 < ksteps; kt += 2) {
         fetch(kt + 1, 1);
-        dl_compute<false>(acc, lds, g);
+        dl_compute<false, false, A_FMT>(acc, lds, g);
         __syncthreads();
         fetch(kt + 2, 0);
-        dl_compute<false>(acc, lds + STAGE, g);
+        dl_compute<false, false, A_FMT>(acc, lds + STAGE, g);
         __syncthreads();
     }
-    if (kt < ksteps) dl_compute<false>(acc, lds, g);
+    if (kt < ksteps) dl_compute<false, false, A_FMT>(acc, lds, g);
 
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
@@ -629,6 +638,7 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
 // (r, c) owning tile row r and the c-th share of the N range counted in 128-column units.  A share is cut into full
 // 256-column tiles plus, when its unit count is odd, one half-width tile at its end, so no workgroup rounds its work up
 // to whole 256x256 tiles.
+template <int A_FMT>
 __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep,
                                                        int M, int N, int K, int rows_per_xcd, int nu) {
     constexpr int STAGE = 512 * 128;
@@ -703,12 +713,12 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
     auto tile = [&](int n0, auto half_tag) {
         constexpr bool HALF = decltype(half_tag)::value;
         v4f acc[4][8];
-        dl_compute<HALF, true>(acc, lds + buf * STAGE, g);
+        dl_compute<HALF, true, A_FMT>(acc, lds + buf * STAGE, g);
         __syncthreads();
         buf ^= 1;
         fetch_next();
         for (int kt = 1; kt < ksteps; kt++) {
-            dl_compute<HALF, false>(acc, lds + buf * STAGE, g);
+            dl_compute<HALF, false, A_FMT>(acc, lds + buf * STAGE, g);
             __syncthreads();
             buf ^= 1;
             fetch_next();
@@ -739,20 +749,21 @@ static bool dlp_eligible(int M, int N, int K) {
     return rx >= 1 && rx <= 32 && (rx & (rx - 1)) == 0;
 }
 
+template <int A_FMT>
 static int launch_dl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
     NC_CHECK_ARG(ep.out_kind == 0, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
     const size_t lds_bytes = 2 * 512 * 128 + (persistent ? 8 * 4096 : 0);
-    const void* fn = persistent ? (const void*)gemm_dlp_kernel : (const void*)gemm_dl_kernel;
+    const void* fn = persistent ? (const void*)gemm_dlp_kernel<A_FMT> : (const void*)gemm_dl_kernel<A_FMT>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     if (persistent) {
         NC_CHECK_ARG(dlp_eligible(M, N, K), "fp8_gemm: the persistent kernel needs M/256 (rounded up) to be 8, 16, ... 256 tile rows, got M=%d", M);
-        hipLaunchKernelGGL(gemm_dlp_kernel, dim3(256), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m / 8, (N + 127) / 128);
+        hipLaunchKernelGGL(gemm_dlp_kernel<A_FMT>, dim3(256), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m / 8, (N + 127) / 128);
     } else {
-        hipLaunchKernelGGL(gemm_dl_kernel, dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+        hipLaunchKernelGGL(gemm_dl_kernel<A_FMT>, dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     }
     return 0;
 }
@@ -772,7 +783,7 @@ static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& e
 
 int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
                    void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, void* workspace,
-                   size_t workspace_bytes, hipStream_t s) {
+                   size_t workspace_bytes, hipStream_t s, int a_fmt) {
     NC_CHECK_ARG(a && b && inv_a && inv_b && out, "fp8_gemm: null pointer");
     NC_CHECK_ARG(M >= 0 && N > 0 && K > 0, "fp8_gemm: bad shape M=%d N=%d K=%d", M, N, K);
     NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
@@ -787,8 +798,27 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     NC_CHECK_ARG(segs.end[segs.nseg - 1] == N, "fp8_gemm: last segment must end at N");
     if (out_kind == 0)
         NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "fp8_gemm: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
+    NC_CHECK_ARG(a_fmt == 0 || a_fmt == 1, "fp8_gemm: the format of a must be 0 (e4m3fn) or 1 (e5m2)");
     if (M == 0) return 0;
     EpilogueArgs ep{inv_a, inv_b, segs, out, out_kind, softcap, ldc};
+    if (a_fmt == 1) {
+        // gradient operand (the backward GEMMs): bf16 output through the 128x128 buffer-load tile or the 256x256 direct-to-LDS tiles
+        NC_CHECK_ARG(out_kind == 0, "fp8_gemm: an e5m2 operand goes with bf16 output");
+        NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: e5m2 operands need M*K and N*K below 2^31");
+        int which = force_kernel;
+        if (which == 0) {
+            int dev = 0, cus = 256;
+            if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+            which = (K % 128 == 0 && 2 * t256 >= cus) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
+        }
+        NC_CHECK_ARG(which == 5 || which == 8 || which == 9, "fp8_gemm: kernels 5, 8 and 9 take an e5m2 operand, not %d", force_kernel);
+        NcProfScope prof(1, 2.0 * M * N * K, s);
+        int rc = which == 5 ? launch_bl<128, 128, 2, 2, true, 1>(a, b, ep, M, N, K, s) : launch_dl<1>(a, b, ep, M, N, K, which == 9, s);
+        if (rc) return rc;
+        NC_CHECK_LAUNCH("fp8_gemm");
+        return 0;
+    }
 
     // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256,
     // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent
@@ -833,8 +863,8 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     else if (which == 5) rc = launch_bl<128, 128, 2, 2, true>(a, b, ep, M, N, K, s);
     else if (which == 6) rc = launch_bl<256, 128, 4, 2, false>(a, b, ep, M, N, K, s);
     else if (which == 7) rc = launch_bl<256, 256, 4, 2, false>(a, b, ep, M, N, K, s);
-    else if (which == 8) rc = launch_dl(a, b, ep, M, N, K, false, s);
-    else if (which == 9) rc = launch_dl(a, b, ep, M, N, K, true, s);
+    else if (which == 8) rc = launch_dl<0>(a, b, ep, M, N, K, false, s);
+    else if (which == 9) rc = launch_dl<0>(a, b, ep, M, N, K, true, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");

@@ -9,10 +9,11 @@ typedef uint16_t bf16_t;
 
 // ---- quantize (nc_quantize.hip)
 void nc_clear_u32(uint32_t* p, int n, hipStream_t s);
-int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_out,
+int nc_launch_quantize(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* out, float* scale_out, float* inv_out,
                        uint32_t* amax_ws, int encoder, hipStream_t s);
+int nc_launch_transpose_u8(const uint8_t* src, int R, int C, uint8_t* dst, hipStream_t s);
 int nc_launch_convert_only(const void* x, int64_t n, uint8_t* out, float* inv_out, const uint32_t* amax_ws, hipStream_t s);
-int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, uint8_t* out, int encoder, hipStream_t s);
+int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, int fmt, uint8_t* out, int encoder, hipStream_t s);
 
 // ---- GEMM (nc_gemm.hip)
 struct NcGemmSegs {      // column segments of B, each with its own weight inv-scale
@@ -22,7 +23,7 @@ struct NcGemmSegs {      // column segments of B, each with its own weight inv-s
 // out_kind: 0 = bf16 [M,ldc];  1 = fp32 [M,ldc] of softcap*tanh(bf16(v)/softcap)
 int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
                    void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, void* workspace,
-                   size_t workspace_bytes, hipStream_t s);
+                   size_t workspace_bytes, hipStream_t s, int a_fmt = 0);   // a_fmt: 0 e4m3fn, 1 e5m2 (kernels 5, 8, 9)
 
 // small-M path (nc_gemm_decode.hip): A is e4m3 (+inv_a) or bf16 (+amax, quantized inside the kernel)
 // out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax.

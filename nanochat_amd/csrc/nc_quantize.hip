@@ -61,12 +61,12 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, i
 }
 
 // ---------------------------------------------------------------- pass 2: convert
-template <bool IS_BF16, bool HW_CVT>
+template <bool IS_BF16, bool HW_CVT, int FMT = 0>
 __global__ __launch_bounds__(256) void convert_kernel(const void* __restrict__ x, int64_t n, const uint32_t* __restrict__ amax_bits,
                                                       uint8_t* __restrict__ out, float* __restrict__ scale_out,
                                                       float* __restrict__ inv_out) {
     const float amax = amax_read(amax_bits);
-    const float scale = scale_from_amax(amax);
+    const float scale = scale_from_amax(amax, fp8_max<FMT>());
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         if (scale_out) *scale_out = scale;
         *inv_out = 1.0f / scale;
@@ -95,17 +95,17 @@ __global__ __launch_bounds__(256) void convert_kernel(const void* __restrict__ x
         uint32_t o[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            float y0 = clamp448(f[4 * j] * scale), y1 = clamp448(f[4 * j + 1] * scale);
-            float y2 = clamp448(f[4 * j + 2] * scale), y3 = clamp448(f[4 * j + 3] * scale);
-            o[j] = HW_CVT ? e4m3_pack4_hw(y0, y1, y2, y3) : e4m3_pack4_sw(y0, y1, y2, y3);
+            float y0 = fp8_clamp<FMT>(f[4 * j] * scale), y1 = fp8_clamp<FMT>(f[4 * j + 1] * scale);
+            float y2 = fp8_clamp<FMT>(f[4 * j + 2] * scale), y3 = fp8_clamp<FMT>(f[4 * j + 3] * scale);
+            o[j] = fp8_pack4<FMT, HW_CVT>(y0, y1, y2, y3);
         }
         ((uint4*)out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
     }
     if (blockIdx.x == 0) {
         for (int64_t i = n16 * 16 + threadIdx.x; i < n; i += blockDim.x) {
             float v = IS_BF16 ? bf16_to_f32(((const bf16_t*)x)[i]) : ((const float*)x)[i];
-            float y = clamp448(v * scale);
-            out[i] = (uint8_t)(HW_CVT ? (e4m3_pack4_hw(y, 0.f, 0.f, 0.f) & 0xffu) : e4m3_encode_sw(y));
+            float y = fp8_clamp<FMT>(v * scale);
+            out[i] = (uint8_t)(fp8_pack4<FMT, HW_CVT>(y, 0.f, 0.f, 0.f) & 0xffu);
         }
     }
 }
@@ -116,12 +116,12 @@ __global__ void clear_u32_kernel(uint32_t* p, int n) {
 }
 
 // Encode with a caller-given scale (no amax pass): used to check the encoder exhaustively.
-template <bool HW_CVT>
+template <bool HW_CVT, int FMT>
 __global__ void encode_with_scale_kernel(const bf16_t* __restrict__ x, int64_t n, float scale, uint8_t* __restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
-        float y = clamp448(bf16_to_f32(x[i]) * scale);
-        out[i] = (uint8_t)(HW_CVT ? (e4m3_pack4_hw(y, 0.f, 0.f, 0.f) & 0xffu) : e4m3_encode_sw(y));
+        float y = fp8_clamp<FMT>(bf16_to_f32(x[i]) * scale);
+        out[i] = (uint8_t)(fp8_pack4<FMT, HW_CVT>(y, 0.f, 0.f, 0.f) & 0xffu);
     }
 }
 
@@ -136,11 +136,30 @@ void nc_clear_u32(uint32_t* p, int n, hipStream_t s) {
     hipLaunchKernelGGL(clear_u32_kernel, dim3((n + 63) / 64), dim3(64), 0, s, p, n);
 }
 
-int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_out,
+template <int FMT>
+static void launch_quantize_fmt(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_out, uint32_t* amax_ws,
+                                int encoder, int g1, int g2, hipStream_t s) {
+    if (x_dtype == 0) {
+        hipLaunchKernelGGL(amax_kernel<true>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
+        if (encoder == 0)
+            hipLaunchKernelGGL((convert_kernel<true, true, FMT>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+        else
+            hipLaunchKernelGGL((convert_kernel<true, false, FMT>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+    } else {
+        hipLaunchKernelGGL(amax_kernel<false>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
+        if (encoder == 0)
+            hipLaunchKernelGGL((convert_kernel<false, true, FMT>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+        else
+            hipLaunchKernelGGL((convert_kernel<false, false, FMT>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
+    }
+}
+
+int nc_launch_quantize(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* out, float* scale_out, float* inv_out,
                        uint32_t* amax_ws, int encoder, hipStream_t s) {
     NC_CHECK_ARG(n >= 0, "fp8_quantize: negative element count");
     NC_CHECK_ARG(inv_out && amax_ws && (n == 0 || (x && out)), "fp8_quantize: null pointer");
     NC_CHECK_ARG(x_dtype == 0 || x_dtype == 1, "fp8_quantize: dtype must be 0 (bf16) or 1 (fp32)");
+    NC_CHECK_ARG(fmt == 0 || fmt == 1, "fp8_quantize: format must be 0 (e4m3fn) or 1 (e5m2)");
     NC_CHECK_ARG(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "fp8_quantize: pointers must be 16-byte aligned");
     nc_clear_u32(amax_ws, 1, s);
     NcProfScope prof(2, 3.0 * n, s);
@@ -148,19 +167,8 @@ int nc_launch_quantize(const void* x, int x_dtype, int64_t n, uint8_t* out, floa
     // at most 1024 blocks x 256 threads, four loads per thread and trip; every block ends with one atomic on the same word
     int g1 = grid_for(n / per_vec, 1024, 1024);
     int g2 = grid_for(n / 16, 256, 4096);
-    if (x_dtype == 0) {
-        hipLaunchKernelGGL(amax_kernel<true>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
-        if (encoder == 0)
-            hipLaunchKernelGGL((convert_kernel<true, true>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
-        else
-            hipLaunchKernelGGL((convert_kernel<true, false>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
-    } else {
-        hipLaunchKernelGGL(amax_kernel<false>, dim3(g1), dim3(256), 0, s, x, n, amax_ws);
-        if (encoder == 0)
-            hipLaunchKernelGGL((convert_kernel<false, true>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
-        else
-            hipLaunchKernelGGL((convert_kernel<false, false>), dim3(g2), dim3(256), 0, s, x, n, amax_ws, out, scale_out, inv_out);
-    }
+    if (fmt == 0) launch_quantize_fmt<0>(x, x_dtype, n, out, scale_out, inv_out, amax_ws, encoder, g1, g2, s);
+    else launch_quantize_fmt<1>(x, x_dtype, n, out, scale_out, inv_out, amax_ws, encoder, g1, g2, s);
     NC_CHECK_LAUNCH("fp8_quantize");
     return 0;
 }
@@ -174,14 +182,70 @@ int nc_launch_convert_only(const void* x, int64_t n, uint8_t* out, float* inv_ou
     return 0;
 }
 
-int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, uint8_t* out, int encoder, hipStream_t s) {
-    NC_CHECK_ARG(x && out && n >= 0, "e4m3_encode: bad arguments");
+int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, int fmt, uint8_t* out, int encoder, hipStream_t s) {
+    NC_CHECK_ARG(x && out && n >= 0, "fp8_encode: bad arguments");
+    NC_CHECK_ARG(fmt == 0 || fmt == 1, "fp8_encode: format must be 0 (e4m3fn) or 1 (e5m2)");
     int g = (int)((n + 255) / 256);
     if (g == 0) return 0;
-    if (encoder == 0)
-        hipLaunchKernelGGL(encode_with_scale_kernel<true>, dim3(g), dim3(256), 0, s, x, n, scale, out);
-    else
-        hipLaunchKernelGGL(encode_with_scale_kernel<false>, dim3(g), dim3(256), 0, s, x, n, scale, out);
-    NC_CHECK_LAUNCH("e4m3_encode");
+    if (fmt == 0) {
+        if (encoder == 0) hipLaunchKernelGGL((encode_with_scale_kernel<true, 0>), dim3(g), dim3(256), 0, s, x, n, scale, out);
+        else hipLaunchKernelGGL((encode_with_scale_kernel<false, 0>), dim3(g), dim3(256), 0, s, x, n, scale, out);
+    } else {
+        if (encoder == 0) hipLaunchKernelGGL((encode_with_scale_kernel<true, 1>), dim3(g), dim3(256), 0, s, x, n, scale, out);
+        else hipLaunchKernelGGL((encode_with_scale_kernel<false, 1>), dim3(g), dim3(256), 0, s, x, n, scale, out);
+    }
+    NC_CHECK_LAUNCH("fp8_encode");
     return 0;
 }
+
+// ---------------------------------------------------------------- byte-matrix transpose
+// dst[c][r] = src[r][c] for an fp8 payload: the memory rearrangement behind _to_col_major and .t().contiguous() at
+// nanochat/fp8.py:110-118,169,181-182 (the backward GEMMs need the reduction index contiguous in both operands).
+// 128x128 tiles: 16-byte global accesses on both sides (whole 128-byte row segments), 4x4 byte blocks transposed in
+// registers with v_perm_b32 between two LDS copies of the tile.
+#define TP_PITCH 144
+__global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t* __restrict__ src, int R, int C, uint8_t* __restrict__ dst) {
+    __shared__ __align__(16) uint8_t ta[128 * TP_PITCH], tb[128 * TP_PITCH];
+    const int r0 = blockIdx.y * 128, c0 = blockIdx.x * 128, t = threadIdx.x;
+    const int lrow = t >> 3, lc16 = (t & 7) * 16;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = lrow + 32 * i;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (r0 + row < R && c0 + lc16 < C) v = *(const uint4*)(src + (size_t)(r0 + row) * C + c0 + lc16);
+        *(uint4*)(ta + row * TP_PITCH + lc16) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int blk = t + 256 * i, rb = blk >> 5, cb = blk & 31;      // 4x4 block: rows 4 rb.., columns 4 cb..
+        uint32_t d[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) d[k] = *(const uint32_t*)(ta + (4 * rb + k) * TP_PITCH + 4 * cb);
+        const uint32_t t0 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400), t1 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602);
+        const uint32_t u0 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400), u1 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602);
+        const uint32_t o[4] = {__builtin_amdgcn_perm(u0, t0, 0x05040100), __builtin_amdgcn_perm(u0, t0, 0x07060302),
+                               __builtin_amdgcn_perm(u1, t1, 0x05040100), __builtin_amdgcn_perm(u1, t1, 0x07060302)};
+#pragma unroll
+        for (int k = 0; k < 4; k++) *(uint32_t*)(tb + (4 * cb + k) * TP_PITCH + 4 * rb) = o[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = lrow + 32 * i;          // a column of src
+        if (c0 + row < C && r0 + lc16 < R)
+            *(uint4*)(dst + (size_t)(c0 + row) * R + r0 + lc16) = *(const uint4*)(tb + row * TP_PITCH + lc16);
+    }
+}
+
+int nc_launch_transpose_u8(const uint8_t* src, int R, int C, uint8_t* dst, hipStream_t s) {
+    NC_CHECK_ARG(R >= 0 && C >= 0, "fp8_transpose: negative shape");
+    if (R == 0 || C == 0) return 0;
+    NC_CHECK_ARG(src && dst, "fp8_transpose: null pointer");
+    NC_CHECK_ARG(R % 16 == 0 && C % 16 == 0, "fp8_transpose: rows=%d and cols=%d must be multiples of 16", R, C);
+    NC_CHECK_ARG(((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0, "fp8_transpose: pointers must be 16-byte aligned");
+    hipLaunchKernelGGL(transpose_u8_kernel, dim3((C + 127) / 128, (R + 127) / 128), dim3(256), 0, s, src, R, C, dst);
+    NC_CHECK_LAUNCH("fp8_transpose");
+    return 0;
+}
+

@@ -1,17 +1,45 @@
-"""Float8Linear on MI355X: tensorwise e4m3 quantization + FP8 MFMA GEMM, forward only.
+"""Float8Linear on MI355X: tensorwise fp8 quantization + FP8 MFMA GEMMs.
 
 Same public surface as nanochat/fp8.py (Float8Linear :195-227, Float8LinearConfig :230-240,
 convert_to_float8_training :243-266).  Differences that do not change results:
   * the weight is quantized once and kept (payload + inverse scale) until the parameter's storage or
-    version counter changes; the reference re-quantizes it on every call (fp8.py:136), which for a
-    frozen weight produces the same bytes;
-  * there is no backward: this is the inference path.
+    version counter changes; the reference re-quantizes it on every call (fp8.py:136), which for an
+    unchanged weight produces the same bytes;
+  * without autograd (inference) no tensors are saved and the call is three launches; with autograd the
+    three GEMMs of _Float8Matmul (fp8.py:123-192) run: e4m3 x e4m3 forward, e5m2 x e4m3 for both gradients.
 """
 import torch
 import torch.nn as nn
 
 from . import ops
 from .common import COMPUTE_DTYPE
+
+
+class _Float8Matmul(torch.autograd.Function):
+    """input_2d [B,K] @ weight[N,K]^T with the reference's three FP8 GEMMs (nanochat/fp8.py:123-192)."""
+
+    @staticmethod
+    def forward(ctx, input_2d, weight, module):
+        a8, inv_a, _ = ops.fp8_quantize(input_2d)
+        w8, inv_w = module._weight_fp8()
+        ctx.save_for_backward(a8, inv_a, w8, inv_w)
+        return ops.fp8_gemm(a8, w8, inv_a, inv_w)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a8, inv_a, w8, inv_w = ctx.saved_tensors
+        if grad_output.dtype != torch.bfloat16:
+            raise ValueError("Float8Linear: the GPU path computes in bf16")
+        # gradients in e5m2 (wider range), saved operands in e4m3 (fp8.py:163-165)
+        go8, inv_go, _ = ops.fp8_quantize(grad_output.contiguous(), fp8_dtype=torch.float8_e5m2)
+        grad_input = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            # grad_input [B,K] = grad_output [B,N] @ weight [N,K]: the summed index N must be contiguous in both (fp8.py:166-177)
+            grad_input = ops.fp8_gemm_grad(go8, ops.fp8_transpose(w8), inv_go, inv_w)
+        if ctx.needs_input_grad[1]:
+            # grad_weight [N,K] = grad_output^T [N,B] @ input [B,K]: B contiguous in both (fp8.py:179-190)
+            grad_weight = ops.fp8_gemm_grad(ops.fp8_transpose(go8), ops.fp8_transpose(a8), inv_go, inv_a)
+        return grad_input, grad_weight, None
 
 
 class Float8Linear(nn.Linear):
@@ -22,12 +50,12 @@ class Float8Linear(nn.Linear):
         key = (w.data_ptr(), w._version, w.dtype, tuple(w.shape))
         cached = getattr(self, "_fp8_cache", None)
         if cached is None or cached[0] != key:
-            payload, inv, _ = ops.fp8_quantize(w.detach())
+            with torch.no_grad():
+                payload, inv, _ = ops.fp8_quantize(w.detach())
             cached = (key, payload, inv.reshape(1))
             self._fp8_cache = cached
         return cached[1], cached[2]
 
-    @torch.no_grad()
     def forward(self, input):
         if not input.is_cuda:
             raise RuntimeError("Float8Linear runs on the GPU only; there is no CPU fallback")
@@ -36,9 +64,12 @@ class Float8Linear(nn.Linear):
             raise ValueError("Float8Linear: the GPU path computes in bf16")
         orig_shape = input.shape
         x2 = input.reshape(-1, orig_shape[-1])
-        a8, inv_a, _ = ops.fp8_quantize(x2)
-        w8, inv_w = self._weight_fp8()
-        out = ops.fp8_gemm(a8, w8, inv_a, inv_w)
+        if torch.is_grad_enabled() and (x2.requires_grad or self.weight.requires_grad):
+            out = _Float8Matmul.apply(x2, self.weight, self)
+        else:
+            a8, inv_a, _ = ops.fp8_quantize(x2)
+            w8, inv_w = self._weight_fp8()
+            out = ops.fp8_gemm(a8, w8, inv_a, inv_w)
         out = out.reshape(*orig_shape[:-1], out.shape[-1])
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)

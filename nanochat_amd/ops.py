@@ -37,22 +37,69 @@ def _amax_slot(device):
 
 
 # ----------------------------------------------------------------------------- (1) quantize
-def fp8_quantize(x, encoder=0):
-    """Tensorwise e4m3 quantization of a bf16/fp32 tensor (nanochat/fp8.py:81-107).
+_FP8_FORMATS = {torch.float8_e4m3fn: 0, torch.float8_e5m2: 1}
 
-    Returns (payload float8_e4m3fn with x's shape, inv_scale fp32 0-dim, scale fp32 0-dim)."""
+
+def fp8_quantize(x, encoder=0, fp8_dtype=torch.float8_e4m3fn):
+    """Tensorwise fp8 quantization of a bf16/fp32 tensor (nanochat/fp8.py:81-107): e4m3fn, or e5m2 for gradients.
+
+    Returns (payload of fp8_dtype with x's shape, inv_scale fp32 0-dim, scale fp32 0-dim)."""
     _need_cuda(x)
     if x.dtype not in (torch.bfloat16, torch.float32):
         raise ValueError(f"fp8_quantize: dtype {x.dtype} not supported (bf16 or fp32)")
+    if fp8_dtype not in _FP8_FORMATS:
+        raise ValueError(f"fp8_quantize: format {fp8_dtype} not supported (float8_e4m3fn or float8_e5m2)")
     x = x.contiguous()
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     scales = torch.empty(2, dtype=torch.float32, device=x.device)
     ws = _amax_slot(x.device)
-    rc = _lib.lib().nc_fp8_quantize_tensorwise(_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _ptr(out),
-                                               C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4),
-                                               _ptr(ws), encoder, _stream())
+    rc = _lib.lib().nc_fp8_quantize_tensorwise_as(_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _FP8_FORMATS[fp8_dtype],
+                                                  _ptr(out), C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4),
+                                                  _ptr(ws), encoder, _stream())
     _lib.check(rc)
-    return out.view(torch.float8_e4m3fn), scales[1], scales[0]
+    return out.view(fp8_dtype), scales[1], scales[0]
+
+
+def fp8_encode_with_scale(x_bf16, scale, fp8_dtype, encoder=0):
+    """The saturating cast alone, with a given scale (nanochat/fp8.py:100-103); returns uint8 payload bytes."""
+    _need_cuda(x_bf16)
+    assert x_bf16.dtype == torch.bfloat16
+    x = x_bf16.contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.lib().nc_fp8_encode_with_scale(_ptr(x), x.numel(), float(scale), _FP8_FORMATS[fp8_dtype], _ptr(out), encoder, _stream()))
+    return out
+
+
+def fp8_transpose(x8):
+    """[R,C] fp8 payload -> [C,R] contiguous (the rearrangement of _to_col_major / .t().contiguous(), nanochat/fp8.py:110-118)."""
+    _need_cuda(x8)
+    if x8.dim() != 2 or x8.element_size() != 1:
+        raise ValueError("fp8_transpose: a 2-D one-byte tensor is required")
+    x8 = x8.contiguous()
+    R, Cc = x8.shape
+    out = torch.empty(Cc, R, dtype=x8.dtype, device=x8.device)
+    _lib.check(_lib.lib().nc_fp8_transpose(_ptr(x8), R, Cc, _ptr(out), _stream()))
+    return out
+
+
+def fp8_gemm_grad(a_e5m2, w8, inv_a, inv_w, kernel=0, out=None):
+    """out[M,N] = bf16((a_e5m2[M,K] @ w8[N,K]^T, fp32 acc) * inv_a * inv_w): the backward GEMMs of nanochat/fp8.py:166-190,
+    first operand in e5m2, second in e4m3fn, the summed index contiguous in both."""
+    _need_cuda(a_e5m2, w8, inv_a, inv_w)
+    if a_e5m2.dim() != 2 or w8.dim() != 2 or a_e5m2.shape[1] != w8.shape[1]:
+        raise ValueError(f"fp8_gemm_grad: shapes {tuple(a_e5m2.shape)} x {tuple(w8.shape)}^T do not match")
+    if a_e5m2.element_size() != 1 or w8.element_size() != 1:
+        raise ValueError("fp8_gemm_grad: operands must be fp8 (one byte per element)")
+    a_e5m2, w8 = a_e5m2.contiguous(), w8.contiguous()
+    M, K = a_e5m2.shape
+    N = w8.shape[0]
+    inv_a = inv_a.reshape(-1).float()
+    inv_w = inv_w.reshape(-1).float()
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=a_e5m2.device)
+    _lib.check(_lib.lib().nc_fp8_gemm_tn_grad(_ptr(a_e5m2), _ptr(w8), _ptr(inv_a), _ptr(inv_w), _ptr(out), M, N, K, out.stride(0), kernel,
+                                              _stream()))
+    return out
 
 
 def e4m3_encode_with_scale(x_bf16, scale, encoder=0):

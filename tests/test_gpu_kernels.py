@@ -328,6 +328,122 @@ def test_float8linear_module_forward(ops):
     assert rel_l2(got2, want * 2) < 2e-3
 
 
+# ================================================================== (2b) gradient format, transpose, backward GEMMs
+@pytest.mark.parametrize("encoder", [0, 1])
+@pytest.mark.parametrize("scale", [1.0, 0.37, 57344.0 / 5.1875, 3.0e-3, 1.7e4, 5.7344e16])
+def test_e5m2_encoder_exhaustive_all_bf16(ops, encoder, scale):
+    say(f"e5m2 encoder exhaustive scale={scale} encoder={encoder}")
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    x = x[torch.isfinite(x.float())]
+    want = (x.float() * np.float32(scale)).clamp(-57344, 57344).to(torch.float8_e5m2).view(torch.uint8)
+    got = ops.fp8_encode_with_scale(x.to(DEV), scale, torch.float8_e5m2, encoder=encoder).cpu()
+    assert torch.equal(got, want)
+    assert torch.equal(got, fp8_ref.e5m2_encode_bits((x.float() * np.float32(scale)).clamp(-57344, 57344)))
+
+
+@pytest.mark.parametrize("shape,dtype,mag", [((8192, 1664), torch.bfloat16, 1e-3), ((64, 6656), torch.bfloat16, 1.0), ((333, 77), torch.bfloat16, 30.0),
+                                             ((1664, 1664), torch.float32, 1e-6), ((1,), torch.bfloat16, 1.0), ((0,), torch.bfloat16, 1.0)])
+def test_quantize_e5m2_matches_oracle_bitwise(ops, shape, dtype, mag):
+    say(f"quantize e5m2 {shape} {dtype}")
+    g = torch.Generator().manual_seed(hash(shape) % 1000 + 1)
+    x = torch.randn(shape, generator=g) * mag
+    if x.numel() > 100:
+        x = torch.where(torch.rand(shape, generator=g) < 0.001, x * 50, x)     # gradients are heavy-tailed
+    x = x.to(dtype)
+    payload, inv, scale = ops.fp8_quantize(x.to(DEV), fp8_dtype=torch.float8_e5m2)
+    assert payload.dtype == torch.float8_e5m2
+    if x.numel() == 0:
+        assert payload.numel() == 0 and scale.item() == np.float32(57344.0 / 1e-12)
+        return
+    want_p, want_inv, want_s = fp8_ref.to_fp8(x, torch.float8_e5m2)
+    assert f32_bits(scale.item()) == f32_bits(want_s.item())
+    assert f32_bits(inv.item()) == f32_bits(want_inv.item())
+    assert torch.equal(payload.view(torch.uint8).cpu(), want_p.view(torch.uint8))
+
+
+@pytest.mark.parametrize("R,C", [(128, 128), (16, 16), (48, 272), (2048, 1664), (1664, 6656), (8192, 400), (144, 8192)])
+def test_fp8_transpose_is_exact(ops, R, C):
+    say(f"transpose {R}x{C}")
+    g = torch.Generator().manual_seed(R + C)
+    x = torch.randint(0, 256, (R, C), generator=g, dtype=torch.uint8)
+    got = ops.fp8_transpose(x.to(DEV)).cpu()
+    assert got.shape == (C, R) and torch.equal(got, x.t().contiguous())
+    with pytest.raises((AssertionError, ValueError)):
+        ops.fp8_transpose(torch.zeros(24, 40, dtype=torch.uint8, device=DEV))        # not multiples of 16
+
+
+@pytest.mark.parametrize("M,N,K,kernel", [
+    (300, 320, 256, 5), (64, 128, 400, 5), (513, 272, 1664, 5), (2100, 1300, 48, 5),
+    (300, 320, 256, 8), (513, 272, 1664, 8), (4100, 2100, 384, 8),
+    (2048, 1664, 256, 9), (2000, 1000, 384, 9), (8192, 4992, 128, 9),
+    (64, 1664, 6656, 0), (2048, 6656, 1664, 0), (1664, 6656, 2048, 0), (8192, 1664, 256, 0),
+])
+def test_grad_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
+    say(f"grad gemm M={M} N={N} K={K} kernel={kernel}")
+    g = torch.Generator().manual_seed(M * 3 + N + K)
+    a = torch.randn(M, K, generator=g) * 1e-3
+    a = torch.where(torch.rand(M, K, generator=g) < 0.001, a * 50, a).bfloat16()
+    w = ((torch.rand(N, K, generator=g) * 2 - 1) * math.sqrt(3.0 / K)).bfloat16()
+    a8, ia, _ = fp8_ref.to_fp8(a, torch.float8_e5m2)
+    w8, iw, _ = fp8_ref.to_fp8(w)
+    want = ((a8.float() @ w8.float().t()) * ia * iw).bfloat16()
+    got = ops.fp8_gemm_grad(a8.to(DEV), w8.to(DEV), ia.to(DEV), iw.to(DEV), kernel=kernel).cpu()
+    assert got.shape == (M, N) and got.dtype == torch.bfloat16
+    err = rel_l2(got, want)
+    assert err <= 2e-2, err
+    assert err <= 2e-3, err           # same fp8 inputs: only summation order and one bf16 rounding differ
+
+
+@pytest.mark.parametrize("kernel,M", [(5, 256), (8, 256), (9, 2048)])
+def test_grad_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
+    say(f"grad gemm exact kernel={kernel}")
+    g = torch.Generator().manual_seed(10)
+    N, K = 192, 384
+    a = (torch.randint(0, 2, (M, K), generator=g).float() * 2 - 1) * 2.0 ** torch.randint(-3, 3, (M, K), generator=g).float()
+    w = (torch.randint(0, 2, (N, K), generator=g).float() * 2 - 1) * 2.0 ** torch.randint(-3, 3, (N, K), generator=g).float()
+    a[0, 0] = 7.0
+    w[0, 0] = 7.0
+    a8, ia, _ = fp8_ref.to_fp8(a.bfloat16(), torch.float8_e5m2)
+    w8, iw, _ = fp8_ref.to_fp8(w.bfloat16())
+    got = ops.fp8_gemm_grad(a8.to(DEV), w8.to(DEV), ia.to(DEV), iw.to(DEV), kernel=kernel).cpu()
+    assert torch.equal(got, (a @ w.t()).bfloat16())                  # exact products and sums: the true product itself
+
+
+@pytest.mark.parametrize("B,K,N", [(256, 256, 384), (2048, 1664, 1664), (4096, 1664, 6656), (64, 6656, 1664), (48, 128, 144)])
+def test_float8linear_backward_matches_oracle(ops, B, K, N):
+    """Float8Linear under autograd: output, grad_input and grad_weight against the CPU restatement of
+    _Float8Matmul (nanochat/fp8.py:123-192) fed the same tensors."""
+    say(f"Float8Linear backward B={B} K={K} N={N}")
+    from nanochat_amd.fp8 import Float8Linear
+    g = torch.Generator().manual_seed(B + K + N)
+    x = torch.randn(B, K, generator=g).bfloat16()
+    w = ((torch.rand(N, K, generator=g) * 2 - 1) * math.sqrt(3.0 / K))
+    go = (torch.randn(B, N, generator=g) * 1e-3)
+    go = torch.where(torch.rand(B, N, generator=g) < 0.001, go * 50, go).bfloat16()
+    lin = Float8Linear(K, N, bias=False).to(DEV)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    xg = x.to(DEV).requires_grad_(True)
+    out = lin(xg)
+    out.backward(go.to(DEV))
+    a8, ia, _ = fp8_ref.to_fp8(x)
+    w8, iw, _ = fp8_ref.to_fp8(w)                                    # the fp32 master weight is what gets quantized
+    want_out = fp8_ref.scaled_mm_emulated(a8, w8, ia, iw)
+    want_gi, want_gw, _, _ = fp8_ref.float8_matmul_backward(go, a8, ia, w8, iw)
+    assert rel_l2(out.detach().cpu(), want_out) <= 2e-3
+    assert xg.grad.dtype == torch.bfloat16 and lin.weight.grad.dtype == lin.weight.dtype
+    assert rel_l2(xg.grad.cpu(), want_gi) <= 2e-3
+    assert rel_l2(lin.weight.grad.cpu(), want_gw.float()) <= 2e-3
+    # and the unquantized gradients, at fp8 noise level
+    assert rel_l2(xg.grad.cpu(), go.float() @ w) < 0.1
+    assert rel_l2(lin.weight.grad.cpu(), go.float().t() @ x.float()) < 0.1
+    # a second step after an in-place weight update re-quantizes the weight
+    with torch.no_grad():
+        lin.weight.mul_(0.5)
+    out2 = lin(x.to(DEV))
+    assert rel_l2(out2.detach().cpu().float() * 2, want_out) <= 2e-2
+
+
 # ================================================================== (4) row kernels
 def ulp_close(got, want, max_frac_off=0.002):
     """bf16 tensors equal except for rare one-ulp differences (fp32 summation order)."""

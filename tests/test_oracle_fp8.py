@@ -176,3 +176,63 @@ def test_float8_linear_shapes_and_filter():
     assert rel < 0.06      # e4m3 has 3 mantissa bits: ~3-4% rms error is expected
     assert fp8_ref.fp8_module_filter(256, 1024) and not fp8_ref.fp8_module_filter(12, 2)
     assert not fp8_ref.fp8_module_filter(24, 1) and not fp8_ref.fp8_module_filter(130, 256)
+
+
+# ---------------------------------------------------------------- gradient format and the backward GEMMs (nanochat/fp8.py:156-192)
+def test_e5m2_cast_pinned_by_integer_encoder_exhaustively():
+    """Every bf16 value the clamp lets through, and random fp32 values: torch's e5m2 cast (the library routine the reference
+    calls at fp8.py:103) against an integer restatement of OCP e5m2 round-to-nearest-even."""
+    allb = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    x = allb[allb.abs() <= fp8_ref.E5M2_MAX]
+    assert torch.equal(x.to(torch.float8_e5m2).view(torch.uint8), fp8_ref.e5m2_encode_bits(x))
+    g = torch.Generator().manual_seed(0)
+    y = (torch.randn(500_000, generator=g) * torch.exp(torch.randn(500_000, generator=g) * 6)).clamp(-fp8_ref.E5M2_MAX, fp8_ref.E5M2_MAX)
+    assert torch.equal(y.to(torch.float8_e5m2).view(torch.uint8), fp8_ref.e5m2_encode_bits(y))
+    # ties to even, the subnormal boundary and the saturation point
+    probe = torch.tensor([1.125, 1.375, 2.0 ** -16, 2.0 ** -17, 1.5 * 2.0 ** -16, 57344.0, 60000.0])
+    assert probe.clamp(max=fp8_ref.E5M2_MAX).to(torch.float8_e5m2).float().tolist() == [1.0, 1.5, 2.0 ** -16, 0.0, 2.0 ** -15, 57344.0, 57344.0]
+
+
+def test_to_fp8_e5m2_closed_form_and_invariants():
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(4096, generator=g) * 3).bfloat16()
+    p, inv, scale = fp8_ref.to_fp8(x, torch.float8_e5m2)
+    amax = x.float().abs().max().double()
+    assert scale.item() == np.float32(57344.0 / amax.item()) and inv.item() == np.float32(1.0) / np.float32(scale.item())
+    assert (p.view(torch.uint8) & 0x7F).max().item() == 0x7B                 # the largest entry lands on 57344
+    p2, _, _ = fp8_ref.to_fp8(-x, torch.float8_e5m2)
+    assert torch.equal(p.view(torch.uint8) ^ 0x80, p2.view(torch.uint8))
+    z, _, sz = fp8_ref.to_fp8(torch.zeros(64).bfloat16(), torch.float8_e5m2)
+    assert z.view(torch.uint8).sum().item() == 0 and sz.item() == np.float32(57344.0 / 1e-12)
+
+
+def test_backward_restatement_against_library_and_exact_case():
+    g = torch.Generator().manual_seed(2)
+    B, K, N = 64, 128, 96
+    x = torch.randn(B, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    go = (torch.randn(B, N, generator=g) * 1e-3).bfloat16()
+    a8, ia, _ = fp8_ref.to_fp8(x)
+    w8, iw, _ = fp8_ref.to_fp8(w)
+    gi, gw, go8, igo = fp8_ref.float8_matmul_backward(go, a8, ia, w8, iw)
+    gi_lib, gw_lib = fp8_ref.float8_matmul_backward_library(go, a8, ia, w8, iw)      # the reference's own three calls, on CPU
+    for got, want in ((gi, gi_lib), (gw, gw_lib)):
+        assert got.shape == want.shape and got.dtype == torch.bfloat16
+        rel = ((got.float() - want.float()).norm() / want.float().norm()).item()
+        assert rel < 2e-3, rel                                                       # same fp8 inputs: summation order + one bf16 rounding
+    # against the unquantized gradients, fp8 noise only
+    gi_exact = go.float() @ w.float()
+    gw_exact = go.float().t() @ x.float()
+    assert ((gi.float() - gi_exact).norm() / gi_exact.norm()).item() < 0.1
+    assert ((gw.float() - gw_exact).norm() / gw_exact.norm()).item() < 0.1
+    # signed powers of two with power-of-two scales: every product and partial sum is exact, so the result is the exact gradient
+    sgn = lambda *s: torch.randint(0, 2, s, generator=g).float() * 2 - 1
+    xe = sgn(B, K) * 2.0 ** torch.randint(-2, 3, (B, K), generator=g).float()
+    we = sgn(N, K) * 2.0 ** torch.randint(-2, 3, (N, K), generator=g).float()
+    ge = sgn(B, N) * 2.0 ** torch.randint(-2, 3, (B, N), generator=g).float()
+    xe[0, 0], we[0, 0], ge[0, 0] = 7.0, 7.0, 7.0                                     # amax 7: 448/7 = 64 and 57344/7 = 8192
+    a8, ia, _ = fp8_ref.to_fp8(xe.bfloat16())
+    w8, iw, _ = fp8_ref.to_fp8(we.bfloat16())
+    gi, gw, _, _ = fp8_ref.float8_matmul_backward(ge.bfloat16(), a8, ia, w8, iw)
+    assert torch.equal(gi, (ge @ we).bfloat16()) and torch.equal(gw, (ge.t() @ xe).bfloat16())
+
