@@ -773,10 +773,8 @@ template <int BM, int BN>
 static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
-    static bool configured = false;   // per instantiation; the attribute is per function, not per device state
     hipError_t e = hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, BN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-    (void)configured;
     hipLaunchKernelGGL((gemm_tile_kernel<BM, BN>), dim3(tiles_m * tiles_n), dim3(256), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     return 0;
 }
