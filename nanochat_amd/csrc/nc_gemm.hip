@@ -252,7 +252,8 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             }
         }
     }
-    if (OUT_KIND == 0) __syncthreads();                        // the staging memory is free again
+    // no barrier and no wait here: the kernel ends, and a wave may retire with its stores still on their way, which frees the
+    // CU for the next workgroup while the output drains
 }
 
 // ------------------------------------------------------------------------------------------------
