@@ -809,7 +809,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             int dev = 0, cus = 256;
             if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-            which = (K % 128 == 0 && 2 * t256 >= cus) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
+            which = (K % 128 == 0 && 8 * t256 >= 5 * cus) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
         }
         NC_CHECK_ARG(which == 5 || which == 8 || which == 9, "fp8_gemm: kernels 5, 8 and 9 take an e5m2 operand, not %d", force_kernel);
         NcProfScope prof(1, 2.0 * M * N * K, s);
@@ -830,8 +830,8 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             const long rounds = (t256 + cus - 1) / cus;
-            if (out_kind == 0 && K % 128 == 0 && 2 * t256 >= cus) {
-                // 256x256 tiles fed straight into LDS whenever they occupy at least half of the CUs (below that the
+            if (out_kind == 0 && K % 128 == 0 && 8 * t256 >= 5 * cus) {
+                // 256x256 tiles fed straight into LDS whenever they occupy at least 5/8 of the CUs (below that the
                 // 128x128 tiles, four times as many, fill the chip better); from two rounds of tiles on, the
                 // persistent form, which neither rounds the last round up nor pays a prologue per tile
                 which = (t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8;
