@@ -273,18 +273,19 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(NcRopeSrc r, const
 __global__ __launch_bounds__(256) void kv_prefill_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t vec_per_row,
                                                               size_t src_row_stride, size_t dst_row_stride, int src_rows, int dst_rows) {
     const int layer = blockIdx.y;
-    const size_t v0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    // piece i of a thread is vector v0 + 256 i: every load and store instruction of a wave covers 1 KB of consecutive bytes
+    const size_t v0 = (size_t)blockIdx.x * 1024 + threadIdx.x;
     const int b_first = src_rows == 1 ? 0 : blockIdx.z, b_last = src_rows == 1 ? dst_rows : blockIdx.z + 1;
     const uint4* sp = src + ((size_t)layer * src_rows + (src_rows == 1 ? 0 : blockIdx.z)) * src_row_stride;
     v4i r[4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
-        if (v0 + i < vec_per_row) r[i] = *(const v4i*)(sp + v0 + i);
+        if (v0 + 256 * i < vec_per_row) r[i] = *(const v4i*)(sp + v0 + 256 * i);
     for (int b = b_first; b < b_last; b++) {
         uint4* dp = dst + ((size_t)layer * dst_rows + b) * dst_row_stride;
 #pragma unroll
         for (int i = 0; i < 4; i++)
-            if (v0 + i < vec_per_row) __builtin_nontemporal_store(r[i], (v4i*)(dp + v0 + i));
+            if (v0 + 256 * i < vec_per_row) __builtin_nontemporal_store(r[i], (v4i*)(dp + v0 + 256 * i));
     }
 }
 
