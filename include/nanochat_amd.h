@@ -78,6 +78,12 @@ int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const
 int nc_fp8_gemm_tn_grad(const uint8_t* a_e5m2, const uint8_t* b, const float* inv_a, const float* inv_b, void* out, int M,
                         int N, int K, int ldc, int kernel, nc_stream_t stream);
 
+/* The MLP's first linear with its activation (nanochat/gpt.py:138-139, c_fc then relu().square()) for M > 128 rows:
+ * out[M,N] = bf16(relu(bf16(v))^2), v as in nc_fp8_gemm_tn, and atomicMax(*out_amax, fp32 bits of max(out)) so that the
+ * next tensorwise quantization needs no amax pass; the caller clears *out_amax.  kernel: 0 auto, 5..9. */
+int nc_fp8_gemm_tn_relu2(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, void* out,
+                         uint32_t* out_amax, int M, int N, int K, int ldc, int kernel, nc_stream_t stream);
+
 size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K);
 int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const uint8_t* b, const float* inv_b,
                           const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap,

@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(_HERE, "libnanochat_amd.so")
 
 EXPORTS = [
     "nc_abi_version", "nc_last_error", "nc_fp8_quantize_tensorwise", "nc_e4m3_encode_with_scale", "nc_fp8_gemm_tn",
-    "nc_fp8_quantize_tensorwise_as", "nc_fp8_encode_with_scale", "nc_fp8_transpose", "nc_fp8_gemm_tn_grad",
+    "nc_fp8_quantize_tensorwise_as", "nc_fp8_encode_with_scale", "nc_fp8_transpose", "nc_fp8_gemm_tn_grad", "nc_fp8_gemm_tn_relu2",
     "nc_fp8_small_m_workspace_bytes", "nc_fp8_linear_small_m",
     "nc_rmsnorm", "nc_embed_norm_smear", "nc_mix_norm", "nc_relu2", "nc_qkv_rope_append",
     "nc_attention_workspace_bytes", "nc_decode_attention", "nc_kv_cache_prefill", "nc_softcap", "nc_sample",
@@ -53,6 +53,7 @@ def _bind(lib):
         "nc_fp8_encode_with_scale": (i, [p, i64, f, i, p, i, p]),
         "nc_fp8_transpose": (i, [p, i, i, p, p]),
         "nc_fp8_gemm_tn_grad": (i, [p, p, p, p, p, i, i, i, i, i, p]),
+        "nc_fp8_gemm_tn_relu2": (i, [p, p, p, p, p, p, i, i, i, i, i, p]),
         "nc_fp8_gemm_tn": (i, [p, p, p, p, p, i, p, i, f, i, i, i, i, i, p, sz, p]),
         "nc_fp8_small_m_workspace_bytes": (sz, [i, i, i]),
         "nc_fp8_linear_small_m": (i, [p, p, p, p, p, i, p, i, f, p, i, i, i, i, p, sz, i, p]),

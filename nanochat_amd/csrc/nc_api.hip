@@ -71,6 +71,12 @@ int nc_fp8_gemm_tn_grad(const uint8_t* a_e5m2, const uint8_t* b, const float* in
     return nc_launch_gemm(a_e5m2, b, inv_a, inv_b, segs, out, 0, 0.f, M, N, K, ldc, kernel, nullptr, 0, (hipStream_t)stream, 1);
 }
 
+int nc_fp8_gemm_tn_relu2(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, void* out, uint32_t* out_amax, int M,
+                         int N, int K, int ldc, int kernel, nc_stream_t stream) {
+    NcGemmSegs segs{1, {N, 0, 0, 0}};
+    return nc_launch_gemm(a, b, inv_a, inv_b, segs, out, 2, 0.f, M, N, K, ldc, kernel, nullptr, 0, (hipStream_t)stream, 0, out_amax);
+}
+
 size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K) {
     if (M < 1 || M > 128 || N < 1 || K < 1) return 0;
     return nc_gemm_decode_partial_bytes(M, N, K);

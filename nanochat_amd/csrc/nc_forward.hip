@@ -143,6 +143,9 @@ struct LinearRunner {
         // large M: explicit convert pass, tiled GEMM; relu^2 (out_kind 2) is a separate kernel there
         TRY(nc_launch_convert_only(in, (int64_t)rows * K, w.a8, w.inv + site, w.site(site), s));
         if (out_kind == 2) {
+            // relu^2 and its amax in the GEMM's epilogue; past the 32-bit buffer offsets, the plain-load kernel and a separate pass
+            if ((long)rows * K < (1L << 31) && (long)N * K < (1L << 31))
+                return nc_launch_gemm(w.a8, w8, w.inv + site, inv_w, segs, out, 2, 0.f, rows, N, K, ldc, 0, nullptr, 0, s, 0, out_amax);
             TRY(nc_launch_gemm(w.a8, w8, w.inv + site, inv_w, segs, w.h, 0, 0.f, rows, N, K, N, 0, nullptr, 0, s));
             return nc_launch_relu2(w.h, (bf16_t*)out, (int64_t)rows * N, out_amax, s);
         }

@@ -30,10 +30,28 @@ struct EpilogueArgs {
     const float* inv_b;
     NcGemmSegs segs;
     void* out;
-    int out_kind;
+    int out_kind;            // 0 bf16, 1 fp32 softcap, 2 bf16 relu(v)^2 with the amax of the result published to out_amax
     float softcap;
     int ldc;
+    uint32_t* out_amax;
 };
+
+// relu(bf16(v))^2, to be rounded to bf16 by the caller's pack: the two eager ops of nanochat/gpt.py:139 on a bf16 tensor
+__device__ __forceinline__ float relu2_of(float v) {
+    const float h = fmaxf(rbf(v), 0.f);
+    return h * h;
+}
+// largest of eight non-negative bf16 values in a 16-byte vector, the first `count` of them
+__device__ __forceinline__ float max_bf16x8(const uint4& v, int count) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t m = 0;
+#pragma unroll
+    for (int r = 0; r < 8; r++) {
+        const uint32_t b = (w[r >> 1] >> ((r & 1) * 16)) & 0xffffu;
+        if (r < count) m = b > m ? b : m;             // non-negative bf16: integer order is value order
+    }
+    return __uint_as_float(m << 16);
+}
 
 __device__ __forceinline__ float seg_scale(const EpilogueArgs& e, int col) {
     int s = 0;
@@ -190,6 +208,8 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
         // back with one row segment per group of LPR lanes and stores 16 bytes per lane.
         constexpr int WROWS = BM / WGM, WCOLS = BN / WGN, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
         static_assert(LPR % 8 == 0 && LPR <= 64 && WGM * WGN * WROWS * ROWB <= 2 * STAGE, "epilogue staging");
+        const bool relu2 = ep.out_kind == 2;
+        float am = 0.f;
         __syncthreads();                                       // every wave is done with the operand tiles
         uint8_t* reg = lds + wave * WROWS * ROWB;
 #pragma unroll
@@ -204,8 +224,13 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             for (int i = 0; i < WTM; i++) {
                 const int row = i * 16 + frow;
                 const v4f a4 = acc[i][j];
-                const uint2 pk = make_uint2(pack_bf16_hw((a4[0] * inv_a) * inv_b, (a4[1] * inv_a) * inv_b),
-                                            pack_bf16_hw((a4[2] * inv_a) * inv_b, (a4[3] * inv_a) * inv_b));
+                float o4[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    o4[r] = (a4[r] * inv_a) * inv_b;
+                    if (relu2) o4[r] = relu2_of(o4[r]);
+                }
+                const uint2 pk = make_uint2(pack_bf16_hw(o4[0], o4[1]), pack_bf16_hw(o4[2], o4[3]));
                 *(uint2*)(reg + row * ROWB + ((chunk ^ (row & 7)) << 4) + (kb & 1) * 8) = pk;
             }
         }
@@ -222,6 +247,7 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             const int m = m0 + wm * WROWS + row;
             const uint4 v = *(const uint4*)(reg + row * ROWB + ((c ^ (row & 7)) << 4));
             if (m >= M || n >= N) continue;
+            if (relu2) am = fmaxf(am, max_bf16x8(v, N - n));
             bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
             if (n + 8 <= N) {
                 if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
@@ -233,6 +259,10 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
                 for (int r = 0; r < 8 && n + r < N; r++) o[r] = (bf16_t)(w[r >> 1] >> ((r & 1) * 16));
             }
+        }
+        if (relu2) {
+            am = wave_max(am);
+            if (lane == 0) amax_publish(ep.out_amax, am);
         }
     } else {
 #pragma unroll
@@ -446,10 +476,10 @@ static int launch_bl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep,
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
-    const void* fn = ep.out_kind == 0 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>;
+    const void* fn = ep.out_kind != 1 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-    if (ep.out_kind == 0)
+    if (ep.out_kind != 1)
         hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     else
         hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
@@ -586,6 +616,8 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
                                              const DlGeom& g, int m0, int n0, int M, int N) {
     constexpr int WTN = HALF ? 4 : 8, WCOLS = WTN * 16, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
     const bool vec16 = (ep.ldc % 8 == 0) && (((uintptr_t)ep.out & 15) == 0);
+    const bool relu2 = ep.out_kind == 2;
+    float am = 0.f;
     const int lrow_e = g.lane / LPR, c = g.lane % LPR;
     const int n_st = n0 + g.wn * WCOLS + c * 8;
     float inv_b[WTN];
@@ -603,8 +635,13 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
         for (int j = 0; j < WTN; j++) {
             const int chunk = 2 * j + (g.kb >> 1);
             const v4f a4 = acc[i][j];
-            const uint2 pk = make_uint2(pack_bf16_hw((a4[0] * inv_a) * inv_b[j], (a4[1] * inv_a) * inv_b[j]),
-                                        pack_bf16_hw((a4[2] * inv_a) * inv_b[j], (a4[3] * inv_a) * inv_b[j]));
+            float o4[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                o4[r] = (a4[r] * inv_a) * inv_b[j];
+                if (relu2) o4[r] = relu2_of(o4[r]);
+            }
+            const uint2 pk = make_uint2(pack_bf16_hw(o4[0], o4[1]), pack_bf16_hw(o4[2], o4[3]));
             *(uint2*)(reg + g.frow * ROWB + ((chunk ^ (g.frow & 7)) << 4) + (g.kb & 1) * 8) = pk;
         }
         // the region is private to the wave: its own LDS writes only have to land before its reads
@@ -617,6 +654,7 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
             const int m = m0 + g.wm * 64 + i * 16 + row;
             const uint4 v = *(const uint4*)(reg + row * ROWB + ((c ^ (row & 7)) << 4));
             if (m >= M || n_st >= N) continue;
+            if (relu2) am = fmaxf(am, max_bf16x8(v, N - n_st));
             bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n_st;
             if (n_st + 8 <= N) {
                 if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
@@ -630,6 +668,10 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads are done before the next 16 rows overwrite the region
+    }
+    if (relu2) {
+        am = wave_max(am);
+        if (g.lane == 0) amax_publish(ep.out_amax, am);
     }
 }
 
@@ -754,7 +796,7 @@ template <int A_FMT>
 static int launch_dl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
-    NC_CHECK_ARG(ep.out_kind == 0, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
+    NC_CHECK_ARG(ep.out_kind != 1, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
     const size_t lds_bytes = 2 * 512 * 128 + (persistent ? 8 * 4096 : 0);
     const void* fn = persistent ? (const void*)gemm_dlp_kernel<A_FMT> : (const void*)gemm_dl_kernel<A_FMT>;
@@ -782,24 +824,26 @@ static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& e
 
 int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
                    void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, void* workspace,
-                   size_t workspace_bytes, hipStream_t s, int a_fmt) {
+                   size_t workspace_bytes, hipStream_t s, int a_fmt, uint32_t* out_amax) {
     NC_CHECK_ARG(a && b && inv_a && inv_b && out, "fp8_gemm: null pointer");
     NC_CHECK_ARG(M >= 0 && N > 0 && K > 0, "fp8_gemm: bad shape M=%d N=%d K=%d", M, N, K);
     NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
     NC_CHECK_ARG(ldc >= N, "fp8_gemm: ldc=%d < N=%d", ldc, N);
     NC_CHECK_ARG(((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0, "fp8_gemm: operands must be 16-byte aligned");
-    NC_CHECK_ARG(out_kind == 0 || out_kind == 1, "fp8_gemm: out_kind must be 0 (bf16) or 1 (softcapped fp32)");
+    NC_CHECK_ARG(out_kind >= 0 && out_kind <= 2, "fp8_gemm: out_kind must be 0 (bf16), 1 (softcapped fp32) or 2 (bf16 relu^2 + amax)");
+    NC_CHECK_ARG(out_kind != 2 || (out_amax && M > 128 && (long)M * K < (1L << 31) && (long)N * K < (1L << 31) && (force_kernel == 0 || force_kernel >= 5)),
+                 "fp8_gemm: the relu^2 epilogue needs an amax word, M > 128, operands below 2 GiB and a buffer-load kernel");
     NC_CHECK_ARG(segs.nseg >= 1 && segs.nseg <= 4, "fp8_gemm: 1..4 column segments supported, got %d", segs.nseg);
     for (int i = 0; i < segs.nseg; i++) {
         NC_CHECK_ARG(segs.end[i] % 4 == 0 || segs.end[i] == N, "fp8_gemm: segment end %d must be a multiple of 4", segs.end[i]);
         NC_CHECK_ARG(i == 0 || segs.end[i] > segs.end[i - 1], "fp8_gemm: segment ends must increase");
     }
     NC_CHECK_ARG(segs.end[segs.nseg - 1] == N, "fp8_gemm: last segment must end at N");
-    if (out_kind == 0)
+    if (out_kind != 1)
         NC_CHECK_ARG(((uintptr_t)out & 7) == 0 && ldc % 4 == 0, "fp8_gemm: bf16 output needs 8-byte alignment and ldc %% 4 == 0");
     NC_CHECK_ARG(a_fmt == 0 || a_fmt == 1, "fp8_gemm: the format of a must be 0 (e4m3fn) or 1 (e5m2)");
     if (M == 0) return 0;
-    EpilogueArgs ep{inv_a, inv_b, segs, out, out_kind, softcap, ldc};
+    EpilogueArgs ep{inv_a, inv_b, segs, out, out_kind, softcap, ldc, out_amax};
     if (a_fmt == 1) {
         // gradient operand (the backward GEMMs): bf16 output through the 128x128 buffer-load tile or the 256x256 direct-to-LDS tiles
         NC_CHECK_ARG(out_kind == 0, "fp8_gemm: an e5m2 operand goes with bf16 output");
@@ -830,7 +874,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             const long rounds = (t256 + cus - 1) / cus;
-            if (out_kind == 0 && K % 128 == 0 && 8 * t256 >= 5 * cus) {
+            if (out_kind != 1 && K % 128 == 0 && 8 * t256 >= 5 * cus) {
                 // 256x256 tiles fed straight into LDS whenever they occupy at least 5/8 of the CUs (below that the
                 // 128x128 tiles, four times as many, fill the chip better); from two rounds of tiles on, the
                 // persistent form, which neither rounds the last round up nor pays a prologue per tile

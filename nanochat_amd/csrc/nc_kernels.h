@@ -20,10 +20,11 @@ struct NcGemmSegs {      // column segments of B, each with its own weight inv-s
     int nseg;
     int end[4];          // exclusive column end of each segment
 };
-// out_kind: 0 = bf16 [M,ldc];  1 = fp32 [M,ldc] of softcap*tanh(bf16(v)/softcap)
+// out_kind: 0 = bf16 [M,ldc];  1 = fp32 [M,ldc] of softcap*tanh(bf16(v)/softcap);  2 = bf16 relu(bf16(v))^2 + amax (M > 128)
 int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, NcGemmSegs segs,
                    void* out, int out_kind, float softcap, int M, int N, int K, int ldc, int force_kernel, void* workspace,
-                   size_t workspace_bytes, hipStream_t s, int a_fmt = 0);   // a_fmt: 0 e4m3fn, 1 e5m2 (kernels 5, 8, 9)
+                   size_t workspace_bytes, hipStream_t s, int a_fmt = 0,    // a_fmt: 0 e4m3fn, 1 e5m2 (kernels 5, 8, 9)
+                   uint32_t* out_amax = nullptr);                            // out_kind 2: bf16 relu(v)^2, amax of it published here
 
 // small-M path (nc_gemm_decode.hip): A is e4m3 (+inv_a) or bf16 (+amax, quantized inside the kernel)
 // out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax.

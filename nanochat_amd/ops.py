@@ -156,6 +156,20 @@ def fp8_gemm(a8, w8, inv_a, inv_w, seg_ends=None, softcap=None, kernel=0, out=No
     return out
 
 
+def fp8_gemm_relu2(a8, w8, inv_a, inv_w, kernel=0):
+    """relu(a8 @ w8^T * scales)^2 in bf16 for M > 128 rows, and an int32 tensor with the fp32 bits of its maximum
+    (nanochat/gpt.py:138-139 with the amax of the next quantization fused in)."""
+    _need_cuda(a8, w8, inv_a, inv_w)
+    a8, w8 = a8.contiguous(), w8.contiguous()
+    M, K = a8.shape
+    N = w8.shape[0]
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=a8.device)
+    amax = torch.zeros(1, dtype=torch.int32, device=a8.device)
+    _lib.check(_lib.lib().nc_fp8_gemm_tn_relu2(_ptr(a8), _ptr(w8), _ptr(inv_a.reshape(-1).float()), _ptr(inv_w.reshape(-1).float()),
+                                               _ptr(out), _ptr(amax), M, N, K, out.stride(0), kernel, _stream()))
+    return out, amax
+
+
 def fp8_linear_small_m(a_bf16, amax_bits, w8, inv_w, seg_ends=None, softcap=None, relu2=False, ksplits=0):
     """Float8Linear.forward for M <= 128 rows in one launch: a_bf16 [M,K] is quantized inside the GEMM with the
     tensorwise scale of amax_bits (int32 tensor holding the fp32 bits of max|a|).  Returns the output, and with

@@ -320,6 +320,44 @@ def test_small_models_batched_decode(cfg_kwargs, B, P, steps):
     assert_within_floor(G, S, Dd, rel_l2(Dd, S), (S - Dd).abs().max().item(), "prefill + batched decode")
 
 
+LONG_GQA = dict(sequence_len=1024, vocab_size=1024, n_layer=4, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
+LONG_MHA = dict(sequence_len=2048, vocab_size=2048, n_layer=3, n_head=3, n_kv_head=3, n_embd=384, window_pattern="SSL")
+
+
+@pytest.mark.parametrize("cfg_kwargs,B,P,trained_like", [(LONG_GQA, 1, 200, True), (LONG_GQA, 2, 150, True), (LONG_MHA, 1, 700, True),
+                                                         (LONG_MHA, 1, 1100, False), (LONG_GQA, 1, 520, False)])
+def test_long_prefill_matches_oracle(cfg_kwargs, B, P, trained_like):
+    """More than 128 rows in one forward: the tiled FP8 GEMMs (with the relu^2 epilogue), the convert pass, the stand-alone rotary
+    kernel and the matrix-core attention, all positions' logits against the oracle; then two decode steps on that cache."""
+    say(f"long prefill {cfg_kwargs['n_embd']}/{cfg_kwargs['n_head']}q{cfg_kwargs['n_kv_head']}kv B={B} P={P} trained_like={trained_like}")
+    rt, model = build_pair(cfg_kwargs, seed=5, trained_like=trained_like)
+    from nanochat_amd.engine import KVCache
+    cfg = rt.cfg
+    g = torch.Generator().manual_seed(6)
+    prompt = torch.randint(0, cfg.vocab_size, (B, P), generator=g)
+    steps = [torch.randint(0, cfg.vocab_size, (B, 1), generator=g) for _ in range(2)]
+
+    def run(r):
+        c = decode_ref.new_cache(cfg, B, P + 2, torch.bfloat16)
+        outs = [gpt_ref.forward(r, prompt, c)]
+        for nxt in steps:
+            outs.append(gpt_ref.forward(r, nxt, c))
+        return torch.cat(outs, dim=1)
+    floor_rel, floor_max, want, want_def = oracle_floor(rt, run)
+    cache = KVCache(B, cfg.n_kv_head, P + 2, 128, cfg.n_layer, DEV, torch.bfloat16)
+    got = [model(prompt.to(DEV), kv_cache=cache).cpu()]
+    for nxt in steps:
+        got.append(model(nxt.to(DEV), kv_cache=cache).cpu())
+    got = torch.cat(got, dim=1)
+    assert got.shape == want.shape == (B, P + 2, cfg.vocab_size)
+    if trained_like:
+        assert_within_floor(got, want, want_def, floor_rel, floor_max, "long prefill logits")
+    else:
+        worst = min((got - want).abs().max().item(), (got - want_def).abs().max().item())
+        assert worst <= LOGIT_TOL, worst
+    assert cache.get_pos() == P + 2
+
+
 def test_ragged_rows():
     """Per-row cache lengths (outside the reference's GPT.forward, inside FA3's signature): every row
     must equal the same row run alone."""

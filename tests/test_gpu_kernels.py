@@ -200,6 +200,26 @@ def test_gemm_stacked_weights_use_their_own_scales(ops):
         assert rel_l2(got, want_big) < 2e-3, kernel
 
 
+@pytest.mark.parametrize("M,N,K,kernel", [(300, 320, 256, 5), (513, 272, 400, 5), (300, 320, 256, 7), (300, 320, 256, 8), (1000, 1000, 512, 8),
+                                          (2048, 1664, 256, 9), (2000, 1000, 384, 9), (1792, 6656, 1664, 0), (2048, 6656, 256, 0)])
+def test_gemm_relu2_epilogue_and_amax(ops, M, N, K, kernel):
+    say(f"gemm relu2 M={M} N={N} K={K} kernel={kernel}")
+    a, w = make_operands(M, N, K, seed=M + N + K)
+    a8, ia, _ = fp8_ref.to_fp8(a)
+    w8, iw, _ = fp8_ref.to_fp8(w)
+    raw = fp8_ref.scaled_mm_emulated(a8, w8, ia, iw)                    # bf16, as the eager c_fc output
+    want = F.relu(raw).square()                                         # gpt.py:139 on the bf16 tensor
+    got, amax = ops.fp8_gemm_relu2(a8.to(DEV), w8.to(DEV), ia.to(DEV), iw.to(DEV), kernel=kernel)
+    got = got.cpu()
+    assert got.dtype == torch.bfloat16 and (got >= 0).all()
+    assert rel_l2(got, want) <= 2e-3
+    # the published amax is the maximum of what was written, bit for bit (no element outside [M,N] contributes)
+    assert amax.cpu().view(torch.float32).item() == got.float().max().item()
+    # consistent with the plain kernel: same accumulation, activation applied to its bf16 result
+    plain = ops.fp8_gemm(a8.to(DEV), w8.to(DEV), ia.to(DEV), iw.reshape(1).to(DEV), kernel=kernel).cpu()
+    assert torch.equal(got, F.relu(plain).square())
+
+
 def test_gemm_softcap_epilogue(ops):
     say("gemm softcap")
     a, w = make_operands(64, 1024, 256, 11)
