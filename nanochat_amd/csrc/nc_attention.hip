@@ -23,9 +23,11 @@
 #define NEG_BIG (-1.0e30f)
 #define PART_STRIDE 132     // floats per partial: m, l, pad, pad, acc[128]
 
-// FUSED (decode, one new token per row, one split): the workgroup first finishes its own heads of the q|k|v linear
+// FUSED (decode, one new token per row): the workgroup first finishes its own heads of the q|k|v linear
 // (rope_head: partial sums, rotary, QK-norm, value-embedding gate), appends the new key and value to the cache, and
-// attends to them out of LDS; the stand-alone rotary/append kernel and the q buffer drop out of the step.
+// attends to them out of LDS; the stand-alone rotary/append kernel and the q buffer drop out of the step.  With several
+// splits every split finishes the heads for itself (a few KB of partial sums); split 0 alone appends and counts the
+// row's own key, the others stream only older keys, so nobody reads the position that is being written.
 template <int G, bool FUSED>
 __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache,
                                                            bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             float y1, y2;
             rope_head(rope, row, hi, hh, H, Hkv, lane, y1, y2);
             fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
-            if (task >= G && hi >= 0 && hi < Tmax) {
+            if (task >= G && split == 0 && hi >= 0 && hi < Tmax) {
                 bf16_t* dst = (task == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + hk) * 128;
                 dst[lane] = f32_to_bf16(y1);
                 dst[lane + 64] = f32_to_bf16(y2);
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
 #pragma unroll
             for (int e = 0; e < 8; e++) d = fmaf(qf[g][e], fresh[G][sub * 8 + e], d);
             d = row16_sum(d);
-            if (wave == 0 && grp == 0) {
+            if (split == 0 && wave == 0 && grp == 0) {
                 m[g] = d, l[g] = 1.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) acc[g][e] = fresh[G + 1][sub * 8 + e];
@@ -308,7 +310,7 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t*
     int nsplit = force_splits > 0 ? force_splits : pick_splits(B, T, Hkv, max_keys);
     NC_CHECK_ARG(nsplit >= 1 && nsplit <= 16, "decode_attention: splits must be 1..16");
     if (rope) {
-        NC_CHECK_ARG(T == 1 && nsplit == 1 && !seqlens_include_new, "decode_attention: the fused q|k|v finish needs T == 1 and one split");
+        NC_CHECK_ARG(T == 1 && !seqlens_include_new, "decode_attention: the fused q|k|v finish needs one new token per row, not yet counted");
         NC_CHECK_ARG((rope->qkv || rope->pq.parts) && rope->cos_t && rope->sin_t && rope->rope_len > 0, "decode_attention: rotary source missing");
         NC_CHECK_ARG(!rope->ve_table || (rope->ve_gate_w && rope->xn && rope->idx && rope->ld_xn >= 12),
                      "decode_attention: value embedding needs gate weights, xn and idx");
@@ -352,9 +354,10 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
 }
 
 // Decode step, one new token per row, cache_seqlens not yet counting it: finish the q|k|v linear (rotary, QK-norm,
-// value embedding), append key and value at cache_seqlens[b], attend.  Needs nc_attn_splits(...) == 1.
+// value embedding), append key and value at cache_seqlens[b], attend.  counters / partials as for nc_launch_attention.
 int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
-                              bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* amax_ws, hipStream_t s) {
-    return launch_attention_impl(nullptr, &rope, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, nullptr,
-                                 nullptr, 0, amax_ws, 1, 1, s);
+                              bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* counters, void* partials, size_t partial_bytes,
+                              uint32_t* amax_ws, int force_splits, int counters_are_zero, hipStream_t s) {
+    return launch_attention_impl(nullptr, &rope, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, counters,
+                                 partials, partial_bytes, amax_ws, force_splits, counters_are_zero, s);
 }

@@ -202,12 +202,12 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         site++;
         bf16_t* kc = kv->k_cache + (size_t)i * layer_elems;
         bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
-        if (T == 1 && nc_attn_splits(B, 1, Hkv, ly.window_left, kv->max_seq_len) == 1) {
+        if (T == 1) {
             // decode: the attention workgroups finish their own q|k|v heads and append to the cache themselves
             const NcRopeSrc rope{qsrc.parts ? nullptr : w.qkv, qkv_w, qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin,
                                  m->rope_len, m->padded_vocab};
             TRY(nc_launch_attention_fused(rope, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, H, Hkv, kv->max_seq_len,
-                                          w.site(site), s));
+                                          w.attn_counters, w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s));
         } else {
             if (qsrc.parts)
                 TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,

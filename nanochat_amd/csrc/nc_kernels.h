@@ -90,7 +90,8 @@ int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf
 int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax);
 struct NcRopeSrc;
 int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
-                              bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* amax_ws, hipStream_t s);
+                              bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* counters, void* partials, size_t partial_bytes,
+                              uint32_t* amax_ws, int force_splits, int counters_are_zero, hipStream_t s);
 
 // ---- sampling (nc_sample.hip)
 int nc_launch_softcap(const bf16_t* raw, float* out, int64_t n, float softcap, hipStream_t s);
