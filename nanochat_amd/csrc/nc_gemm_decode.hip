@@ -301,18 +301,18 @@ int nc_launch_finish_partials(const float* parts, int nsplit, const uint32_t* a_
     return 0;
 }
 
-// How many K splits a [M<=128] x [N,K] linear is cut into: one 512-wide K chunk per workgroup (a single round
-// of loads) as long as that keeps the partial traffic moderate; big-N layers need fewer to fill the machine.
 // How many K splits a [M<=128] x [N,K] linear is cut into.  Measured on d26 shapes at M=64: a workgroup that
-// covers one 512-wide K chunk (a single round of loads) finishes in ~6 us, every further chunk it walks adds
-// ~3 us of exposed latency, so K is split down to one chunk per workgroup (at most 16 splits).  Only a layer
-// with hundreds of column blocks of its own (lm_head) runs unsplit with the epilogue in the GEMM.
+// covers one 512-wide K chunk (a single round of loads) finishes in ~6 us and every further chunk it walks adds
+// ~3 us of exposed latency, so K is split over workgroups.  Only a layer with hundreds of column blocks of its own
+// (lm_head) runs unsplit with the epilogue in the GEMM.
 int nc_gemm_decode_splits(int N, int K) {
     const int nblk = (N + 63) / 64;
     const int nksteps = (K + 127) / 128;
     if (N % 4 != 0 || nblk >= 256) return 1;
-    int ks = (nksteps + 3) / 4;
-    if (ks > 8) ks = 8;      // more splits than 8 cost the consumer more in partial sums to read than the GEMM gains (K = 6656: 13 -> 8 splits, +2 % tokens/s)
+    // as many splits as keep the launch within one round of the 256 CUs (a second round of workgroups costs more than longer
+    // K runs), and at most 8: beyond that the consumer pays more for the partial sums it has to read than the GEMM gains
+    int ks = 256 / nblk;
+    if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;
     const int kps = (nksteps + ks - 1) / ks;
     return (nksteps + kps - 1) / kps;
