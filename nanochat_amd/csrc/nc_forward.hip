@@ -97,7 +97,7 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
         const int shapes[5][2] = {{(int)qkv_w, (int)E}, {(int)E, m->n_head * 128}, {(int)(4 * E), (int)E}, {(int)E, (int)(4 * E)},
                                   {m->vocab_size, (int)E}};
         for (auto& sh : shapes) {
-            const size_t n = nc_gemm_decode_partial_bytes((int)M, sh[0], sh[1]);
+            const size_t n = nc_gemm_decode_partial_bytes_auto((int)M, sh[0], sh[1]);
             gneed = n > gneed ? n : gneed;
         }
     }

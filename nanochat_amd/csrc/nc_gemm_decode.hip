@@ -318,8 +318,17 @@ int nc_gemm_decode_splits(int N, int K) {
     return (nksteps + kps - 1) / kps;
 }
 
-size_t nc_gemm_decode_partial_bytes(int M, int N, int K) {
+// room for the partial sums of the split count nc_gemm_decode_splits() picks (what a forward pass needs)
+size_t nc_gemm_decode_partial_bytes_auto(int M, int N, int K) {
     const int ks = nc_gemm_decode_splits(N, K);
+    return ks > 1 ? (size_t)ks * M * N * sizeof(float) : 0;
+}
+
+// room for the partial sums of any split count a caller may ask for (at most 16, and no more than there are K-steps)
+size_t nc_gemm_decode_partial_bytes(int M, int N, int K) {
+    if (N % 4 != 0) return 0;
+    const int nksteps = (K + 127) / 128;
+    const int ks = nksteps < 16 ? nksteps : 16;
     return ks > 1 ? (size_t)ks * M * N * sizeof(float) : 0;
 }
 
@@ -335,6 +344,7 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     NC_CHECK_ARG(((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0, "fp8_gemm: operands must be 16-byte aligned");
     const int nksteps = (K + 127) / 128;
     if (ksplits <= 0) ksplits = nc_gemm_decode_splits(N, K);
+    NC_CHECK_ARG(ksplits <= 16, "fp8_gemm(decode): at most 16 K splits, got %d", ksplits);
     if (ksplits > nksteps) ksplits = nksteps;
     int kps = (nksteps + ksplits - 1) / ksplits;
     ksplits = (nksteps + kps - 1) / kps;

@@ -30,7 +30,8 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
 // out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax.
 // With K split over workgroups the raw fp32 sums land in `partials` [ksplits][M][N] and a consumer finishes them.
 int nc_gemm_decode_splits(int N, int K);
-size_t nc_gemm_decode_partial_bytes(int M, int N, int K);
+size_t nc_gemm_decode_partial_bytes(int M, int N, int K);        // any split count up to 16
+size_t nc_gemm_decode_partial_bytes_auto(int M, int N, int K);   // the split count nc_gemm_decode_splits() picks
 int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
                           const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
                           int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s);
