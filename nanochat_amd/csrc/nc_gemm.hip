@@ -202,13 +202,13 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
     const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
     const int wm = wave / WGN, wn = wave % WGN;
     const int frow = lane & 15, kb = lane >> 4;
-    if (OUT_KIND == 0) {
+    if (OUT_KIND != 1) {
         // bf16 output goes through LDS so that every store instruction writes whole 128-byte lines: each wave parks its
         // (BM/WGM) x (BN/WGN) block in its own LDS region (16-byte chunk c of row r at chunk c ^ (r & 7)), then reads it
         // back with one row segment per group of LPR lanes and stores 16 bytes per lane.
         constexpr int WROWS = BM / WGM, WCOLS = BN / WGN, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
         static_assert(LPR % 8 == 0 && LPR <= 64 && WGM * WGN * WROWS * ROWB <= 2 * STAGE, "epilogue staging");
-        const bool relu2 = ep.out_kind == 2;
+        constexpr bool relu2 = OUT_KIND == 2;
         float am = 0.f;
         __syncthreads();                                       // every wave is done with the operand tiles
         uint8_t* reg = lds + wave * WROWS * ROWB;
@@ -471,19 +471,24 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
     bl_epilogue<BM, BN, WGM, WGN, OUT_KIND>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
+template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE, int A_FMT, int OUT_KIND>
+static int launch_bl_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
+    const void* fn = (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, OUT_KIND, INTERLEAVE, A_FMT>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, OUT_KIND, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b,
+                       ep, M, N, K, tiles_m, tiles_n);
+    return 0;
+}
 template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE = false, int A_FMT = 0>
 static int launch_bl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
-    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
-    const void* fn = ep.out_kind != 1 ? (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT> : (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>;
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-    if (ep.out_kind != 1)
-        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 0, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
-    else
-        hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, 1, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
-    return 0;
+    if (ep.out_kind == 0) return launch_bl_as<BM, BN, WGM, WGN, INTERLEAVE, A_FMT, 0>(a, b, ep, M, N, K, s);
+    NC_CHECK_ARG(A_FMT == 0, "fp8_gemm: an e5m2 operand goes with plain bf16 output");
+    if (ep.out_kind == 1) return launch_bl_as<BM, BN, WGM, WGN, INTERLEAVE, 0, 1>(a, b, ep, M, N, K, s);
+    return launch_bl_as<BM, BN, WGM, WGN, INTERLEAVE, 0, 2>(a, b, ep, M, N, K, s);
 }
 
 
@@ -545,7 +550,7 @@ __device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, 
 }
 
 // One tile per workgroup, launched tile by tile (any M, N).
-template <int A_FMT>
+template <int A_FMT, bool RELU2>
 __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep, int M,
                                                       int N, int K, int tiles_m, int tiles_n) {
     constexpr int STAGE = 512 * 128;
@@ -605,18 +610,18 @@ __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict_
     float sc[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
-    bl_epilogue<256, 256, 4, 2, 0>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
+    bl_epilogue<256, 256, 4, 2, RELU2 ? 2 : 0>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
 // Epilogue of the persistent kernel: the wave's 64 x (128 | 64) block leaves 16 rows at a time through a 4 KB LDS region of
 // its own (past the two operand stages, so the loads of the next tile keep landing meanwhile), every store instruction
 // writing whole 128-byte lines.
-template <bool HALF>
+template <bool HALF, bool RELU2>
 __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, const EpilogueArgs& ep, float inv_a, const float (&sc)[4],
                                              const DlGeom& g, int m0, int n0, int M, int N) {
     constexpr int WTN = HALF ? 4 : 8, WCOLS = WTN * 16, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
     const bool vec16 = (ep.ldc % 8 == 0) && (((uintptr_t)ep.out & 15) == 0);
-    const bool relu2 = ep.out_kind == 2;
+    constexpr bool relu2 = RELU2;
     float am = 0.f;
     const int lrow_e = g.lane / LPR, c = g.lane % LPR;
     const int n_st = n0 + g.wn * WCOLS + c * 8;
@@ -681,7 +686,7 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
 // (r, c) owning tile row r and the c-th share of the N range counted in 128-column units.  A share is cut into full
 // 256-column tiles plus, when its unit count is odd, one half-width tile at its end, so no workgroup rounds its work up
 // to whole 256x256 tiles.
-template <int A_FMT>
+template <int A_FMT, bool RELU2>
 __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep,
                                                        int M, int N, int K, int rows_per_xcd, int nu) {
     constexpr int STAGE = 512 * 128;
@@ -774,7 +779,7 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
             for (int j = 0; j < (HALF ? 4 : 8); j++) asm volatile("" : "+a"(acc[i][j]));
         int m0_here = m0;
         asm volatile("" : "+s"(m0_here));          // keeps the store addresses of all tiles from being precomputed (and spilled)
-        dlp_epilogue<HALF>(acc, epi, ep, inv_a, sc, g, m0_here, n0, M, N);
+        dlp_epilogue<HALF, RELU2>(acc, epi, ep, inv_a, sc, g, m0_here, n0, M, N);
     };
     for (int q = 0; q < nitems; q++) {
         int n0;
@@ -792,23 +797,31 @@ static bool dlp_eligible(int M, int N, int K) {
     return rx >= 1 && rx <= 32 && (rx & (rx - 1)) == 0;
 }
 
+template <int A_FMT, bool RELU2>
+static int launch_dl_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    const size_t lds_bytes = 2 * 512 * 128 + (persistent ? 8 * 4096 : 0);
+    const void* fn = persistent ? (const void*)gemm_dlp_kernel<A_FMT, RELU2> : (const void*)gemm_dl_kernel<A_FMT, RELU2>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    if (persistent)
+        hipLaunchKernelGGL((gemm_dlp_kernel<A_FMT, RELU2>), dim3(256), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m / 8, (N + 127) / 128);
+    else
+        hipLaunchKernelGGL((gemm_dl_kernel<A_FMT, RELU2>), dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    return 0;
+}
+
+// the relu^2 epilogue is a variant of its own so that the plain kernels keep their register budget
 template <int A_FMT>
 static int launch_dl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
     NC_CHECK_ARG(ep.out_kind != 1, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
-    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-    const size_t lds_bytes = 2 * 512 * 128 + (persistent ? 8 * 4096 : 0);
-    const void* fn = persistent ? (const void*)gemm_dlp_kernel<A_FMT> : (const void*)gemm_dl_kernel<A_FMT>;
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-    if (persistent) {
+    if (persistent)
         NC_CHECK_ARG(dlp_eligible(M, N, K), "fp8_gemm: the persistent kernel needs M/256 (rounded up) to be 8, 16, ... 256 tile rows, got M=%d", M);
-        hipLaunchKernelGGL(gemm_dlp_kernel<A_FMT>, dim3(256), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m / 8, (N + 127) / 128);
-    } else {
-        hipLaunchKernelGGL(gemm_dl_kernel<A_FMT>, dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
-    }
-    return 0;
+    if (A_FMT == 0 && ep.out_kind == 2) return launch_dl_as<0, true>(a, b, ep, M, N, K, persistent, s);
+    NC_CHECK_ARG(ep.out_kind == 0, "fp8_gemm: the relu^2 epilogue goes with an e4m3 first operand");
+    return launch_dl_as<A_FMT, false>(a, b, ep, M, N, K, persistent, s);
 }
 
 // ------------------------------------------------------------------------------------------------
