@@ -487,3 +487,81 @@ def test_model_refuses_what_it_does_not_implement(d4_pair):
     tiny = KVCache(1, 2, 3, 128, 4, DEV, torch.bfloat16)
     with pytest.raises(AssertionError):
         model(idx, kv_cache=tiny)                                # 4 tokens into a 3-slot cache
+
+
+# ------------------------------------------------------------------------------------------------
+# Full size (d26, 64 rows, context to 2048): no oracle can be run at this size in test time, so the checks are
+# properties that hold whatever the size.
+def test_full_size_d26_batch64_properties():
+    say("d26 batch 64 full-size properties")
+    from nanochat_amd.engine import KVCache
+    from nanochat_amd.synthetic import config_for_depth, random_init_model
+    cfg = config_for_depth(26)
+    model = random_init_model(cfg, DEV, seed=2)
+    B, P = 64, 1792
+    g = torch.Generator().manual_seed(7)
+    prompt = torch.randint(0, cfg.vocab_size, (1, P), generator=g).to(DEV)
+    pre = KVCache(1, cfg.n_kv_head, P, 128, cfg.n_layer, DEV, torch.bfloat16)
+    first = model.forward_last(prompt, kv_cache=pre)
+    assert first.shape == (1, cfg.vocab_size) and torch.isfinite(first).all()
+    dec = KVCache(B, cfg.n_kv_head, 2048, 128, cfg.n_layer, DEV, torch.bfloat16)
+    dec.prefill(pre)
+    # (1) replicated rows fed the same tokens compute the same thing: logits identical across the 64 rows, bit for bit
+    tok = first.argmax(-1, keepdim=True).expand(B, 1).contiguous()
+    steps = []
+    for _ in range(3):
+        logits = model.forward_last(tok, kv_cache=dec)
+        assert logits.shape == (B, cfg.vocab_size) and torch.isfinite(logits).all()
+        assert torch.equal(logits, logits[:1].expand(B, -1)), "rows of one replicated prompt diverged"
+        steps.append(logits[0].clone())
+        tok = logits.argmax(-1, keepdim=True)
+    assert dec.get_pos() == P + 3 and dec.cache_seqlens.tolist() == [P + 3] * B
+    # (2) cached decode equals one forward over the longer sequence: position P of a (P+1)-token prefill sees the same
+    # keys and values as the first decode step (different kernels, same mathematics; fp8 and bf16 rounding apart)
+    longer = torch.cat([prompt, first.argmax(-1, keepdim=True)], dim=1)
+    pre2 = KVCache(1, cfg.n_kv_head, P + 1, 128, cfg.n_layer, DEV, torch.bfloat16)
+    full = model.forward_last(longer, kv_cache=pre2)[0]
+    rel = rel_l2(steps[0], full)
+    print(f"d26: decode step vs (P+1)-token prefill rel-L2 {rel:.4f}, argmax {steps[0].argmax().item()} / {full.argmax().item()}")
+    assert rel < 0.1
+    # the appended cache rows agree with the prefill's rows for the same position up to fp8 noise (the tensorwise scale of
+    # a 64-row decode batch is not that of a 1793-row prefill, so not bit for bit)
+    for layer in (0, cfg.n_layer - 1):
+        assert rel_l2(dec.k_cache[layer, 0, P], pre2.k_cache[layer, 0, P]) < 0.1
+        assert rel_l2(dec.v_cache[layer, 0, P], pre2.v_cache[layer, 0, P]) < 0.1
+    # (3) a row with a different token diverges from the others, and does not disturb them: rows are independent
+    # apart from the shared tensorwise scales
+    tok2 = tok.clone()
+    tok2[5, 0] = (tok2[5, 0] + 1234) % cfg.vocab_size
+    snap = dec.cache_seqlens.clone()
+    l_mixed = model.forward_last(tok2, kv_cache=dec)
+    assert not torch.equal(l_mixed[5], l_mixed[0])
+    assert torch.equal(l_mixed[0], l_mixed[63]) and torch.equal(snap + 1, dec.cache_seqlens)
+
+
+@pytest.mark.parametrize("K,N", [(1664, 4992), (1664, 1664), (1664, 6656), (6656, 1664)])
+def test_full_size_float8linear_shapes_against_fp32_matmul(K, N):
+    """The isolated Float8Linear shapes at M = 8192, forward and both backward GEMMs, against torch's fp32 matmul of the
+    same fp8 payloads on the GPU (the CPU oracle covers smaller sizes; payloads are checked bit for bit elsewhere)."""
+    say(f"full-size Float8Linear M=8192 K={K} N={N}")
+    from nanochat_amd import ops
+    M = 8192
+    g = torch.Generator(device=DEV).manual_seed(K + N)
+    a = torch.randn(M, K, device=DEV, generator=g)
+    a = torch.where(torch.rand(M, K, device=DEV, generator=g) < 0.001, a * 20, a).bfloat16()
+    w = ((torch.rand(N, K, device=DEV, generator=g) * 2 - 1) * (3.0 / K) ** 0.5).bfloat16()
+    go = (torch.randn(M, N, device=DEV, generator=g) * 1e-3).bfloat16()
+    a8, ia, _ = ops.fp8_quantize(a)
+    w8, iw, _ = ops.fp8_quantize(w)
+    go8, igo, _ = ops.fp8_quantize(go, fp8_dtype=torch.float8_e5m2)
+    torch.backends.cuda.matmul.allow_tf32 = False
+    af, wf, gf = a8.float(), w8.float(), go8.float()
+    out = ops.fp8_gemm(a8, w8, ia, iw.reshape(1))
+    assert rel_l2(out, (af @ wf.t()) * ia * iw) <= 3e-3
+    gi = ops.fp8_gemm_grad(go8, ops.fp8_transpose(w8), igo, iw)
+    assert rel_l2(gi, (gf @ wf) * igo * iw) <= 3e-3
+    gw = ops.fp8_gemm_grad(ops.fp8_transpose(go8), ops.fp8_transpose(a8), igo, ia)
+    assert rel_l2(gw, (gf.t() @ af) * igo * ia) <= 3e-3
+    # linearity in the scales: doubling an inverse scale doubles the result exactly (power of two)
+    out2 = ops.fp8_gemm(a8, w8, ia * 2, iw.reshape(1))
+    assert torch.equal(out2.float(), out.float() * 2)
