@@ -565,3 +565,51 @@ def test_full_size_float8linear_shapes_against_fp32_matmul(K, N):
     # linearity in the scales: doubling an inverse scale doubles the result exactly (power of two)
     out2 = ops.fp8_gemm(a8, w8, ia * 2, iw.reshape(1))
     assert torch.equal(out2.float(), out.float() * 2)
+
+
+def test_full_size_d32_gqa_batch128_ragged_rows():
+    """d32 with 16 query / 4 kv heads, 128 rows of lengths in [64, 2048): rows that hold the same history and get the same
+    token give the same logits wherever they sit in the batch, a row's result does not depend on what the other rows hold
+    beyond the shared tensorwise scales, and the whole batch agrees with running a few rows in a batch of their own."""
+    say("d32 GQA batch 128 ragged full-size properties")
+    from nanochat_amd.engine import KVCache
+    from nanochat_amd.synthetic import config_for_depth, random_init_model
+    cfg = config_for_depth(32, n_kv_head=4)
+    assert (cfg.n_embd, cfg.n_head, cfg.n_kv_head) == (2048, 16, 4)
+    model = random_init_model(cfg, DEV, seed=3)
+    B, Tmax = 128, 2048
+    g = torch.Generator().manual_seed(8)
+    lens = torch.randint(64, 2048, (B,), generator=g).tolist()
+    lens[1], lens[77], lens[126] = lens[0], lens[0], lens[5]          # duplicates of rows 0 and 5
+    gd = torch.Generator(device=DEV).manual_seed(9)
+    cache = KVCache(B, cfg.n_kv_head, Tmax, 128, cfg.n_layer, DEV, torch.bfloat16)
+    cache.k_cache.normal_(0.0, 1.0, generator=gd)
+    cache.v_cache.normal_(0.0, 1.0, generator=gd)
+    for dup, src in ((1, 0), (77, 0), (126, 5)):
+        cache.k_cache[:, dup] = cache.k_cache[:, src]
+        cache.v_cache[:, dup] = cache.v_cache[:, src]
+    prev = torch.randn(B, 1, cfg.n_embd, device=DEV, generator=gd).bfloat16()
+    prev[1], prev[77], prev[126] = prev[0], prev[0], prev[5]
+    cache.set_seqlens(lens)
+    cache.prev_embedding = prev.clone()
+    tok = torch.randint(0, cfg.vocab_size, (B, 1), generator=g).to(DEV)
+    tok[1], tok[77], tok[126] = tok[0], tok[0], tok[5]
+    k_before = cache.k_cache[:, :, :64].clone()
+    logits = model.forward_last(tok, kv_cache=cache)
+    assert logits.shape == (B, cfg.vocab_size) and torch.isfinite(logits).all()
+    assert cache.cache_seqlens.tolist() == [n + 1 for n in lens]
+    assert torch.equal(logits[0], logits[1]) and torch.equal(logits[0], logits[77]) and torch.equal(logits[5], logits[126])
+    assert not torch.equal(logits[0], logits[5])
+    assert torch.equal(cache.k_cache[:, :, :64], k_before)                     # the append touched position len only
+    # the same rows in a batch of four: same mathematics, other tensorwise scales
+    pick = [0, 5, 40, 127]
+    small = KVCache(len(pick), cfg.n_kv_head, Tmax, 128, cfg.n_layer, DEV, torch.bfloat16)
+    for i, b in enumerate(pick):
+        small.k_cache[:, i] = cache.k_cache[:, b]
+        small.v_cache[:, i] = cache.v_cache[:, b]
+    small.set_seqlens([lens[b] for b in pick])
+    small.prev_embedding = prev[pick].clone()
+    l4 = model.forward_last(tok[pick], kv_cache=small)
+    rel = rel_l2(l4, logits[pick])
+    print(f"d32 GQA: rows in a batch of 4 vs in the batch of 128: rel-L2 {rel:.4f}")
+    assert rel < 0.1
