@@ -153,11 +153,24 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
             if (padd.parts) {
                 float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 const float* pp = padd.parts + (size_t)blockIdx.x * padd.ld + c;
-                for (int sp = 0; sp < padd.nsplit; sp++) {
-                    const float4 a0 = *(const float4*)(pp + (size_t)sp * padd.split_stride);
-                    const float4 a1 = *(const float4*)(pp + (size_t)sp * padd.split_stride + 4);
-                    acc8[0] += a0.x, acc8[1] += a0.y, acc8[2] += a0.z, acc8[3] += a0.w;
-                    acc8[4] += a1.x, acc8[5] += a1.y, acc8[6] += a1.z, acc8[7] += a1.w;
+                // eight splits at a time: all their loads are issued before the first sum (a loop with a run-time trip count
+                // makes one round trip to memory per split); the sums keep the split order
+                for (int sp0 = 0; sp0 < padd.nsplit; sp0 += 8) {
+                    float4 a0[8], a1[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const bool on = sp0 + u < padd.nsplit;
+                        const float* q = pp + (size_t)(on ? sp0 + u : sp0) * padd.split_stride;
+                        a0[u] = *(const float4*)q;
+                        a1[u] = *(const float4*)(q + 4);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        if (sp0 + u < padd.nsplit) {
+                            acc8[0] += a0[u].x, acc8[1] += a0[u].y, acc8[2] += a0[u].z, acc8[3] += a0[u].w;
+                            acc8[4] += a1[u].x, acc8[5] += a1[u].y, acc8[6] += a1[u].z, acc8[7] += a1[u].w;
+                        }
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < 8; j++) v[it][j] = rbf(v[it][j] + rbf((acc8[j] * p_inv_a) * p_inv_b));

@@ -249,9 +249,15 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)M * n4; i += (size_t)gridDim.x * 256) {
         const int m = (int)(i / n4), n = (int)(i % n4) * 4;
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int s = 0; s < nsplit; s++) {
-            const float4 p = *(const float4*)(parts + (size_t)s * split_stride + (size_t)m * N + n);
-            a.x += p.x, a.y += p.y, a.z += p.z, a.w += p.w;
+        // eight splits at a time: loads first, sums after in split order (one round trip to memory, not one per split)
+        const float* pp = parts + (size_t)m * N + n;
+        for (int s0 = 0; s0 < nsplit; s0 += 8) {
+            float4 p[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) p[u] = *(const float4*)(pp + (size_t)(s0 + u < nsplit ? s0 + u : s0) * split_stride);
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (s0 + u < nsplit) a.x += p[u].x, a.y += p[u].y, a.z += p[u].z, a.w += p[u].w;
         }
         int sg = 0;
 #pragma unroll

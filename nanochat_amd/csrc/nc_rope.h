@@ -35,9 +35,17 @@ __device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos
         const int col = hh * 128 + lane;
         const float* pp = r.pq.parts + (size_t)token * r.pq.ld + col;
         float a1 = 0.f, a2 = 0.f;
-        for (int sp = 0; sp < r.pq.nsplit; sp++) {
-            a1 += pp[(size_t)sp * r.pq.split_stride];
-            a2 += pp[(size_t)sp * r.pq.split_stride + 64];
+        // eight splits at a time, loads first, sums after in split order (see mix_norm_vec_kernel)
+        for (int sp0 = 0; sp0 < r.pq.nsplit; sp0 += 8) {
+            float t1[8], t2[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const size_t o = (size_t)(sp0 + u < r.pq.nsplit ? sp0 + u : sp0) * r.pq.split_stride;
+                t1[u] = pp[o], t2[u] = pp[o + 64];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (sp0 + u < r.pq.nsplit) a1 += t1[u], a2 += t2[u];
         }
         const float inv_a = 1.0f / scale_from_amax(amax_read(r.pq.a_amax));
         const float inv_b = r.pq.inv_b[col >= r.pq.seg_end1 ? 2 : (col >= r.pq.seg_end0 ? 1 : 0)];
