@@ -7,8 +7,8 @@
 // Layout: q [B*T, H, 128] bf16; k_cache, v_cache [B, Tmax, Hkv, 128] bf16 (one layer).
 // A key is 256 contiguous bytes; consecutive keys of one head are Hkv*256 bytes apart.
 //
-// Mapping: a wave owns a contiguous run of keys of one (row, kv head).  16 lanes share one key, 16 bytes
-// (8 dims) each, so one 64-lane load instruction fetches four whole keys as four 256-byte segments.  The
+// Mapping: a wave owns a contiguous run of keys of one (row, kv head) or (row, pair of neighbouring kv heads).  16 lanes
+// share one key of one head, 16 bytes (8 dims) each, so one 64-lane load instruction fetches four 256-byte segments.  The
 // 16-lane dot product is finished with DPP row rotations; each 16-lane group runs its own online softmax
 // over the keys it sees (no cross-lane traffic in the loop), and the four groups, then the four waves of
 // the workgroup, then the splits (by whichever split-workgroup finishes last, through a counter), are
@@ -28,20 +28,30 @@
 // attends to them out of LDS; the stand-alone rotary/append kernel and the q buffer drop out of the step.  With several
 // splits every split finishes the heads for itself (a few KB of partial sums); split 0 alone appends and counts the
 // row's own key, the others stream only older keys, so nobody reads the position that is being written.
-template <int G, bool FUSED>
+// HP kv heads per workgroup (1 or 2).  With HP = 2 the two heads are neighbours in memory, a lane group of 32 covers
+// both heads of one key (512 contiguous bytes) and a load instruction fetches two keys: the same bytes per instruction in
+// runs twice as long, which streams ~8 % faster when there are enough workgroups left.  A lane still serves one head
+// (hsel), so the register budget does not change; an odd head count leaves the second half of the last pair idle.
+template <int G, bool FUSED, int HP>
 __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache,
                                                            bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
                                                            float* __restrict__ partials, uint32_t* __restrict__ counters,
                                                            uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, int nsplit,
                                                            NcRopeSrc rope) {
-    __shared__ float merge[4][G][PART_STRIDE];
-    __shared__ float fresh[FUSED ? G + 2 : 1][128];      // FUSED: the G query heads, then the new key and value
+    constexpr int KPI = 4 / HP;                          // keys per load instruction
+    constexpr int TASKS = (G + 2) * HP;                  // FUSED: per head the G query heads, then the new key and value
+    __shared__ float merge[4][HP * G][PART_STRIDE];
+    __shared__ float fresh[FUSED ? TASKS : 1][128];
     __shared__ int last_flag;
-    const int split = blockIdx.x, hk = blockIdx.y, row = blockIdx.z;
+    const int split = blockIdx.x, hp = blockIdx.y, row = blockIdx.z;
     const int b = row / T, t = row % T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int grp = lane >> 4, sub = lane & 15;
+    const int hsel = grp & (HP - 1), ksel = grp / HP;    // which head of the pair, which key of the instruction
+    const int hk = hp * HP + hsel;                       // this lane's kv head
+    const bool head_ok = hk < Hkv;
+    const int n_heads_here = (hp * HP + HP <= Hkv) ? HP : Hkv - hp * HP;
 
     // visible keys [lo, hi]
     int pos = cache_seqlens[b];
@@ -63,22 +73,23 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     if (k_end > k_stop) k_end = k_stop;
 
     const size_t key_stride = (size_t)Hkv * 128;   // elements between consecutive keys
-    const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
-    const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + sub * 8;
+    const int hk_addr = head_ok ? hk : hp * HP;    // an idle half-pair reads nothing; the address only has to be valid
+    const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk_addr) * 128 + sub * 8;
+    const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk_addr) * 128 + sub * 8;
 
-    constexpr int UNROLL = 8;     // 8 loads x 4 keys = 32 keys (8 KB of K and 8 KB of V) in flight per wave
+    constexpr int UNROLL = 8;     // 8 loads of 1 KB each for K and for V in flight per wave (32 keys of one head, or 16 keys of two)
     uint4 kr[UNROLL], vr[UNROLL];
     bool ok[UNROLL];
     auto fetch = [&](int kb0) {
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
-            const int j = kb0 + 4 * i + grp;
-            ok[i] = j < k_end;
+            const int j = kb0 + KPI * i + ksel;
+            ok[i] = j < k_end && head_ok;
             kr[i] = ok[i] ? nt_load16(kbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
-            const int j = kb0 + 4 * i + grp;
+            const int j = kb0 + KPI * i + ksel;
             vr[i] = ok[i] ? nt_load16(vbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
         }
     };
@@ -86,20 +97,23 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     if (k_begin < k_end) fetch(k_begin);
 
     if (FUSED) {
-        // wave w finishes head task w, w+4, ...: tasks 0..G-1 are the query heads, G the key head, G+1 the value head
-        for (int task = wave; task < G + 2; task += 4) {
-            const int hh = task < G ? hk * G + task : (task == G ? H + hk : H + Hkv + hk);
+        // wave w finishes head task w, w+4, ...: per head of the pair, tasks 0..G-1 are the query heads, G the key head,
+        // G+1 the value head
+        for (int task = wave; task < (G + 2) * n_heads_here; task += 4) {
+            const int th = task / (G + 2), tt = task % (G + 2), thk = hp * HP + th;
+            const int hh = tt < G ? thk * G + tt : (tt == G ? H + thk : H + Hkv + thk);
             float y1, y2;
             rope_head(rope, row, hi, hh, H, Hkv, lane, y1, y2);
             fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
-            if (task >= G && split == 0 && hi >= 0 && hi < Tmax) {
-                bf16_t* dst = (task == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + hk) * 128;
+            if (tt >= G && split == 0 && hi >= 0 && hi < Tmax) {
+                bf16_t* dst = (tt == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + thk) * 128;
                 dst[lane] = f32_to_bf16(y1);
                 dst[lane + 64] = f32_to_bf16(y2);
             }
         }
         __syncthreads();
     }
+    const int fbase = (head_ok ? hsel : 0) * (G + 2);     // this lane's head inside fresh[]
 
     // q for the G heads of this kv head, pre-scaled by log2(e) / sqrt(128)
     const float qscale = 1.4426950408889634f * 0.08838834764831845f;
@@ -108,9 +122,9 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     for (int g = 0; g < G; g++) {
         if (FUSED) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) qf[g][e] = fresh[g][sub * 8 + e] * qscale;
+            for (int e = 0; e < 8; e++) qf[g][e] = fresh[fbase + g][sub * 8 + e] * qscale;
         } else {
-            const uint4 qv = *(const uint4*)(q + ((size_t)row * H + hk * G + g) * 128 + sub * 8);
+            const uint4 qv = *(const uint4*)(q + ((size_t)row * H + hk_addr * G + g) * 128 + sub * 8);
             const uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -127,22 +141,22 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         for (int d = 0; d < 8; d++) acc[g][d] = 0.f;
     }
     if (FUSED) {
-        // the row's own key: the first 16 lanes of wave 0 start their running softmax from it (weight exp2(0) = 1)
+        // the row's own key: the lanes of wave 0 that hold key slot 0 start their running softmax from it (weight exp2(0) = 1)
 #pragma unroll
         for (int g = 0; g < G; g++) {
             float d = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) d = fmaf(qf[g][e], fresh[G][sub * 8 + e], d);
+            for (int e = 0; e < 8; e++) d = fmaf(qf[g][e], fresh[fbase + G][sub * 8 + e], d);
             d = row16_sum(d);
-            if (split == 0 && wave == 0 && grp == 0) {
+            if (split == 0 && wave == 0 && ksel == 0 && head_ok) {
                 m[g] = d, l[g] = 1.f;
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[g][e] = fresh[G + 1][sub * 8 + e];
+                for (int e = 0; e < 8; e++) acc[g][e] = fresh[fbase + G + 1][sub * 8 + e];
             }
         }
     }
 
-    for (int kb0 = k_begin; kb0 < k_end; kb0 += 4 * UNROLL) {
+    for (int kb0 = k_begin; kb0 < k_end; kb0 += KPI * UNROLL) {
         if (kb0 != k_begin) fetch(kb0);
         float sc[G][UNROLL];
 #pragma unroll
@@ -188,46 +202,47 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         }
     }
 
-    // merge the four 16-lane groups of the wave
+    // merge the 16-lane groups of the wave that serve the same head (all four, or the two with the same hsel)
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        float mm = fmaxf(m[g], __shfl_xor(m[g], 16));
+        float mm = m[g];
+        if (HP == 1) mm = fmaxf(mm, __shfl_xor(mm, 16));
         mm = fmaxf(mm, __shfl_xor(mm, 32));
         const float w = exp2f(m[g] - mm);
         float lw = l[g] * w;
-        lw += __shfl_xor(lw, 16);
+        if (HP == 1) lw += __shfl_xor(lw, 16);
         lw += __shfl_xor(lw, 32);
 #pragma unroll
         for (int d = 0; d < 8; d++) {
             float a = acc[g][d] * w;
-            a += __shfl_xor(a, 16);
+            if (HP == 1) a += __shfl_xor(a, 16);
             a += __shfl_xor(a, 32);
             acc[g][d] = a;
         }
         m[g] = mm, l[g] = lw;
-        if (grp == 0) {
-            if (sub == 0) merge[wave][g][0] = mm, merge[wave][g][1] = lw;
+        if (ksel == 0) {
+            if (sub == 0) merge[wave][hsel * G + g][0] = mm, merge[wave][hsel * G + g][1] = lw;
 #pragma unroll
-            for (int d = 0; d < 8; d++) merge[wave][g][4 + sub * 8 + d] = acc[g][d];
+            for (int d = 0; d < 8; d++) merge[wave][hsel * G + g][4 + sub * 8 + d] = acc[g][d];
         }
     }
     __syncthreads();
 
-    // merge the four waves: thread (g, d) for d < 128
+    // merge the four waves: thread (head of the pair, g, d) for d < 128
     float am = 0.f;
-    for (int item = threadIdx.x; item < G * 128; item += 256) {
-        const int g = item >> 7, d = item & 127;
+    for (int item = threadIdx.x; item < n_heads_here * G * 128; item += 256) {
+        const int hg = item >> 7, d = item & 127;           // hg = (head of the pair) * G + g
         float mm = NEG_BIG;
 #pragma unroll
-        for (int w = 0; w < 4; w++) mm = fmaxf(mm, merge[w][g][0]);
+        for (int w = 0; w < 4; w++) mm = fmaxf(mm, merge[w][hg][0]);
         float ls = 0.f, a = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            const float sc = exp2f(merge[w][g][0] - mm);
-            ls += merge[w][g][1] * sc;
-            a += merge[w][g][4 + d] * sc;
+            const float sc = exp2f(merge[w][hg][0] - mm);
+            ls += merge[w][hg][1] * sc;
+            a += merge[w][hg][4 + d] * sc;
         }
-        const int head = hk * G + g;
+        const int head = (hp * HP + hg / G) * G + hg % G;
         if (nsplit == 1) {
             const bf16_t o = f32_to_bf16(a / ls);
             out[((size_t)row * H + head) * 128 + d] = o;
@@ -239,11 +254,11 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         }
     }
     if (nsplit > 1) {
-        // the split that arrives last at this (row, kv head) merges all of them, in split order
-        if (!arrive_and_check_last(&counters[row * Hkv + hk], (uint32_t)nsplit, &last_flag)) return;
-        for (int item = threadIdx.x; item < G * 128; item += 256) {
-            const int g = item >> 7, d = item & 127;
-            const int head = hk * G + g;
+        // the split that arrives last at this (row, head pair) merges all of them, in split order
+        if (!arrive_and_check_last(&counters[row * Hkv + hp * HP], (uint32_t)nsplit, &last_flag)) return;
+        for (int item = threadIdx.x; item < n_heads_here * G * 128; item += 256) {
+            const int hg = item >> 7, d = item & 127;
+            const int head = (hp * HP + hg / G) * G + hg % G;
             const float* p = partials + ((size_t)row * H + head) * nsplit * PART_STRIDE;
             float mm = NEG_BIG;
             for (int sidx = 0; sidx < nsplit; sidx++) mm = fmaxf(mm, coherent_load_f1(p + sidx * PART_STRIDE));
@@ -257,10 +272,10 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             out[((size_t)row * H + head) * 128 + d] = o;
             am = fmaxf(am, fabsf(bf16_to_f32(o)));
         }
-        if (threadIdx.x == 0) __hip_atomic_store(&counters[row * Hkv + hk], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) __hip_atomic_store(&counters[row * Hkv + hp * HP], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (amax_ws) {
-        // one publication per workgroup (only the first G*128 threads hold output values)
+        // one publication per workgroup (only the first threads hold output values)
         am = wave_max(am);
         __syncthreads();
         if (lane == 0) merge[wave][0][0] = am;
@@ -270,10 +285,16 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
 }
 
 // ------------------------------------------------------------------------------------------------
+// Two kv heads per workgroup when the head pairs alone still give the chip ~6 waves per CU (512-byte runs stream faster
+// than 256-byte ones only if enough workgroups remain).
+static int pick_heads_per_wg(int B, int T, int Hkv) { return (Hkv >= 2 && (long)B * T * ((Hkv + 1) / 2) * 4 >= 1536) ? 2 : 1; }
+
 static int pick_splits(int B, int T, int Hkv, int max_keys) {
-    // One split whenever the (row, kv head) pairs alone give every CU ~8 waves: measured at batch 64 x 13 heads,
+    // One split whenever the (row, kv head or head pair) workgroups alone give every CU ~6-8 waves: measured at batch 64 x 13 heads,
     // one split streams 513 keys at 5.9 TB/s and 2048 keys at 5.6 TB/s, and every extra split only adds merge work.
     // Small batches need the splits to fill the machine; keep at least 64 keys per wave.
+    const int hp = pick_heads_per_wg(B, T, Hkv);
+    if (hp == 2) return 1;
     const long base_waves = (long)B * T * Hkv * 4;
     int s = 1;
     while (s < 16 && base_waves * s < 2048 && max_keys / (4 * s * 2) >= 64) s *= 2;
@@ -324,22 +345,29 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t*
     }
     NcProfScope prof(0, 0.0, s);
     float* parts = (float*)partials;
-    dim3 grid(nsplit, Hkv, B * T), block(256);
+    const int hp = (force_splits > 0 || nsplit > 1) ? 1 : pick_heads_per_wg(B, T, Hkv);
+    dim3 grid(nsplit, hp == 2 ? (Hkv + 1) / 2 : Hkv, B * T), block(256);
     const NcRopeSrc none{};
-#define LAUNCH_G(GG)                                                                                                         \
-    do {                                                                                                                     \
-        if (rope)                                                                                                            \
-            hipLaunchKernelGGL((attn_partial_kernel<GG, true>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,          \
-                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, *rope); \
-        else                                                                                                                 \
-            hipLaunchKernelGGL((attn_partial_kernel<GG, false>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,         \
-                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, none);  \
+#define LAUNCH_GH(GG, HH)                                                                                                       \
+    do {                                                                                                                        \
+        if (rope)                                                                                                               \
+            hipLaunchKernelGGL((attn_partial_kernel<GG, true, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,         \
+                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, *rope);    \
+        else                                                                                                                    \
+            hipLaunchKernelGGL((attn_partial_kernel<GG, false, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,        \
+                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, none);     \
+    } while (0)
+#define LAUNCH_G(GG)                 \
+    do {                             \
+        if (hp == 2) LAUNCH_GH(GG, 2); \
+        else LAUNCH_GH(GG, 1);       \
     } while (0)
     if (G == 1) LAUNCH_G(1);
     else if (G == 2) LAUNCH_G(2);
     else if (G == 4) LAUNCH_G(4);
     else LAUNCH_G(8);
 #undef LAUNCH_G
+#undef LAUNCH_GH
     NC_CHECK_LAUNCH("decode_attention");
     return 0;
 }
