@@ -93,22 +93,39 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             vr[i] = ok[i] ? nt_load16(vbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
         }
     };
-    // the first batch of keys is on its way before anything that needs q
+    // Loads return in issue order, so the few KB that the head tasks of this wave need go out first and the first batch of keys
+    // right behind them: the rotary/norm arithmetic then runs while the keys are still on their way.
+    // Wave w finishes head task w, w+4, ...: per head of the pair, tasks 0..G-1 are the query heads, G the key head, G+1 the
+    // value head.
+    constexpr int TASKS_PER_WAVE = (TASKS + 3) / 4;
+    RopeRaw<4> raw[FUSED ? TASKS_PER_WAVE : 1];
+    auto task_head = [&](int task) {
+        const int th = task / (G + 2), tt = task % (G + 2), thk = hp * HP + th;
+        return tt < G ? thk * G + tt : (tt == G ? H + thk : H + Hkv + thk);
+    };
+    if (FUSED) {
+#pragma unroll
+        for (int i = 0; i < TASKS_PER_WAVE; i++) {
+            const int task = wave + 4 * i;
+            if (task < (G + 2) * n_heads_here) rope_head_load(rope, row, hi, task_head(task), H, Hkv, lane, raw[i]);
+        }
+    }
     if (k_begin < k_end) fetch(k_begin);
 
     if (FUSED) {
-        // wave w finishes head task w, w+4, ...: per head of the pair, tasks 0..G-1 are the query heads, G the key head,
-        // G+1 the value head
-        for (int task = wave; task < (G + 2) * n_heads_here; task += 4) {
-            const int th = task / (G + 2), tt = task % (G + 2), thk = hp * HP + th;
-            const int hh = tt < G ? thk * G + tt : (tt == G ? H + thk : H + Hkv + thk);
-            float y1, y2;
-            rope_head(rope, row, hi, hh, H, Hkv, lane, y1, y2);
-            fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
-            if (tt >= G && split == 0 && hi >= 0 && hi < Tmax) {
-                bf16_t* dst = (tt == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + thk) * 128;
-                dst[lane] = f32_to_bf16(y1);
-                dst[lane + 64] = f32_to_bf16(y2);
+#pragma unroll
+        for (int i = 0; i < TASKS_PER_WAVE; i++) {
+            const int task = wave + 4 * i;
+            if (task < (G + 2) * n_heads_here) {
+                const int tt = task % (G + 2), thk = hp * HP + task / (G + 2);
+                float y1, y2;
+                rope_head_finish(rope, row, task_head(task), H, Hkv, lane, raw[i], y1, y2);
+                fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
+                if (tt >= G && split == 0 && hi >= 0 && hi < Tmax) {
+                    bf16_t* dst = (tt == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + thk) * 128;
+                    dst[lane] = f32_to_bf16(y1);
+                    dst[lane + 64] = f32_to_bf16(y2);
+                }
             }
         }
         __syncthreads();

@@ -27,16 +27,59 @@ struct NcRopeSrc {
     int vocab_rows;
 };
 
-// hh in [0, H): query head; [H, H+Hkv): key head; [H+Hkv, H+2Hkv): value head.  Returns the finished pair.
-__device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos, int hh, int H, int Hkv, int lane, float& o1, float& o2) {
+// The loads of one head, issued in one go so that their latency is paid once and a caller can put other loads behind them:
+// the first PRE split partials (or the bf16 value), the rotary pair or the value-embedding pair, and for a value head the
+// twelve gate inputs (lane c < 12 holds channel c).
+template <int PRE>
+struct RopeRaw {
+    float t1[PRE], t2[PRE];
+    float e1, e2;             // q, k heads: cos, sin;  v heads with a value embedding: ve[lane], ve[lane + 64]
+    float xg;                 // v heads: xn[lane] for lane < 12
+};
+
+// hh in [0, H): query head; [H, H+Hkv): key head; [H+Hkv, H+2Hkv): value head.
+template <int PRE>
+__device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, int pos, int hh, int H, int Hkv, int lane, RopeRaw<PRE>& w) {
+    if (r.pq.parts) {
+        const float* pp = r.pq.parts + (size_t)token * r.pq.ld + hh * 128 + lane;
+#pragma unroll
+        for (int u = 0; u < PRE; u++) {
+            const size_t o = (size_t)(u < r.pq.nsplit ? u : 0) * r.pq.split_stride;
+            w.t1[u] = pp[o], w.t2[u] = pp[o + 64];
+        }
+    } else {
+        const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128;
+        w.t1[0] = bf16_to_f32(src[lane]), w.t2[0] = bf16_to_f32(src[lane + 64]);
+    }
+    w.e1 = w.e2 = w.xg = 0.f;
+    if (hh < H + Hkv) {
+        const int rp = pos < r.rope_len ? (pos < 0 ? 0 : pos) : r.rope_len - 1;
+        w.e1 = bf16_to_f32(r.cos_t[(size_t)rp * 64 + lane]), w.e2 = bf16_to_f32(r.sin_t[(size_t)rp * 64 + lane]);
+    } else if (r.ve_table) {
+        const int hv = hh - H - Hkv;
+        int64_t tok = r.idx[token];
+        if (tok < 0 || tok >= r.vocab_rows) tok = 0;
+        const bf16_t* ve = r.ve_table + ((size_t)tok * Hkv + hv) * 128;
+        w.e1 = bf16_to_f32(ve[lane]), w.e2 = bf16_to_f32(ve[lane + 64]);
+        w.xg = bf16_to_f32(r.xn[(size_t)token * r.ld_xn + (lane < 12 ? lane : 0)]);
+    }
+}
+
+// Returns the finished pair.
+template <int PRE>
+__device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, int hh, int H, int Hkv, int lane, const RopeRaw<PRE>& w, float& o1,
+                                                 float& o2) {
     float x1, x2;
     if (r.pq.parts) {
-        // the linear's output still sits in split partials: add them up, scale, round to bf16
+        // the linear's output still sits in split partials: add them up in split order, scale, round to bf16
         const int col = hh * 128 + lane;
-        const float* pp = r.pq.parts + (size_t)token * r.pq.ld + col;
         float a1 = 0.f, a2 = 0.f;
-        // eight splits at a time, loads first, sums after in split order (see mix_norm_vec_kernel)
-        for (int sp0 = 0; sp0 < r.pq.nsplit; sp0 += 8) {
+#pragma unroll
+        for (int u = 0; u < PRE; u++)
+            if (u < r.pq.nsplit) a1 += w.t1[u], a2 += w.t2[u];
+        // splits beyond the first PRE, eight at a time, loads first, sums after (see mix_norm_vec_kernel)
+        const float* pp = r.pq.parts + (size_t)token * r.pq.ld + col;
+        for (int sp0 = PRE; sp0 < r.pq.nsplit; sp0 += 8) {
             float t1[8], t2[8];
 #pragma unroll
             for (int u = 0; u < 8; u++) {
@@ -52,12 +95,10 @@ __device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos
         x1 = rbf((a1 * inv_a) * inv_b);
         x2 = rbf((a2 * inv_a) * inv_b);
     } else {
-        const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128;
-        x1 = bf16_to_f32(src[lane]), x2 = bf16_to_f32(src[lane + 64]);
+        x1 = w.t1[0], x2 = w.t2[0];
     }
     if (hh < H + Hkv) {
-        const int rp = pos < r.rope_len ? (pos < 0 ? 0 : pos) : r.rope_len - 1;
-        const float c = bf16_to_f32(r.cos_t[(size_t)rp * 64 + lane]), s = bf16_to_f32(r.sin_t[(size_t)rp * 64 + lane]);
+        const float c = w.e1, s = w.e2;
         float y1 = rbf(rbf(x1 * c) + rbf(x2 * s));
         float y2 = rbf(rbf(x1 * (-s)) + rbf(x2 * c));
         const float ss = wave_sum(y1 * y1 + y2 * y2);
@@ -68,16 +109,19 @@ __device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos
         const int hv = hh - H - Hkv;
         if (r.ve_table) {
             float dot = 0.f;
-            const bf16_t* xr = r.xn + (size_t)token * r.ld_xn;
 #pragma unroll
-            for (int cidx = 0; cidx < 12; cidx++) dot += bf16_to_f32(xr[cidx]) * rbf(r.ve_gate_w[hv * 12 + cidx]);
+            for (int cidx = 0; cidx < 12; cidx++)
+                dot += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w.xg), cidx)) * rbf(r.ve_gate_w[hv * 12 + cidx]);
             const float gate = rbf(3.0f * rbf(sigmoidf_(rbf(dot))));
-            int64_t tok = r.idx[token];
-            if (tok < 0 || tok >= r.vocab_rows) tok = 0;
-            const bf16_t* ve = r.ve_table + ((size_t)tok * Hkv + hv) * 128;
-            x1 = rbf(x1 + rbf(gate * bf16_to_f32(ve[lane])));
-            x2 = rbf(x2 + rbf(gate * bf16_to_f32(ve[lane + 64])));
+            x1 = rbf(x1 + rbf(gate * w.e1));
+            x2 = rbf(x2 + rbf(gate * w.e2));
         }
         o1 = x1, o2 = x2;
     }
+}
+
+__device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos, int hh, int H, int Hkv, int lane, float& o1, float& o2) {
+    RopeRaw<8> w;
+    rope_head_load(r, token, pos, hh, H, Hkv, lane, w);
+    rope_head_finish(r, token, hh, H, Hkv, lane, w, o1, o2);
 }
