@@ -201,6 +201,11 @@ __device__ __forceinline__ bool arrive_and_check_last(uint32_t* counter, uint32_
     return last;
 }
 
+// A kernel argument named here is fetched in the entry block.  The compiler otherwise fetches arguments where they are first used,
+// behind whatever branch that is, and a kernel whose body is a few microseconds long then makes several dependent trips to the
+// argument segment before its first data load.
+#define NC_ARG_NOW(a) asm volatile("" ::"s"(a))
+
 // ---------------------------------------------------------------- amax words
 // The tensorwise amax of an activation is max-reduced by its producer kernel into a device word (fp32 bit patterns
 // of non-negative values order like integers) and read by the FP8 linear that quantizes the activation.  Atomics on
@@ -225,13 +230,32 @@ __device__ __forceinline__ float amax_read(const uint32_t* h) {
     }
     return __uint_as_float(m);
 }
+// The same read split in two, for kernels that put all their loads ahead of their first wait: every lane issues one load (lane i < 8
+// takes slot i of a slotted site, every other lane the first word), no branch in between; the value is the maximum over lanes 0..7.
+__device__ __forceinline__ uint32_t amax_load_lane(const uint32_t* h) {
+    const uint32_t* p = (const uint32_t*)((uintptr_t)h & ~(uintptr_t)3);
+    const int lane = threadIdx.x & 63;
+    return p[(((uintptr_t)h & 1u) && lane < NC_AMAX_SLOTS) ? lane * NC_AMAX_STRIDE : 0];
+}
+// (lane reads that do not depend on which lanes are active, so this may sit inside divergent code as long as the load did not)
+__device__ __forceinline__ float amax_from_lanes(uint32_t loaded) {
+    uint32_t m = 0u;
+#pragma unroll
+    for (int i = 0; i < NC_AMAX_SLOTS; i++) {
+        const uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)loaded, i);
+        m = v > m ? v : m;
+    }
+    return __uint_as_float(m);
+}
 // One call per workgroup.  The atomic is skipped when the word already holds at least the value.
 __device__ __forceinline__ void amax_publish(uint32_t* h, float am) {
     const uint32_t bits = __float_as_uint(am);
     if (bits == 0u || (bits >> 31)) return;
     uint32_t* p = (uint32_t*)((uintptr_t)h & ~(uintptr_t)3);
     if ((uintptr_t)h & 1u) p += ((blockIdx.x + 3u * blockIdx.y + 5u * blockIdx.z) % NC_AMAX_SLOTS) * NC_AMAX_STRIDE;
-    if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
+    // with hundreds of workgroups per slot the atomics queue up behind each other and a look first pays; with a few, the look is
+    // a round trip to memory in front of an atomic that nobody waits for
+    if (gridDim.x * gridDim.y * gridDim.z > 64 * NC_AMAX_SLOTS && __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
     atomicMax(p, bits);
 }
 

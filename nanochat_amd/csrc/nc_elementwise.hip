@@ -120,30 +120,57 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
                                                            const float* __restrict__ x0_lambda, const float* __restrict__ backout_lambda,
                                                            const bf16_t* __restrict__ backout_src, bf16_t* __restrict__ backout_save,
                                                            bf16_t* __restrict__ xn_out, int cols, uint32_t* __restrict__ amax_ws) {
+    NC_ARG_NOW(x), NC_ARG_NOW(add), NC_ARG_NOW(padd.parts), NC_ARG_NOW(padd.nsplit), NC_ARG_NOW(padd.ld), NC_ARG_NOW(padd.split_stride);
+    NC_ARG_NOW(padd.a_amax), NC_ARG_NOW(padd.inv_b), NC_ARG_NOW(x0), NC_ARG_NOW(resid_lambda), NC_ARG_NOW(x0_lambda);
+    NC_ARG_NOW(backout_lambda), NC_ARG_NOW(backout_src), NC_ARG_NOW(backout_save), NC_ARG_NOW(xn_out), NC_ARG_NOW(cols), NC_ARG_NOW(amax_ws);
     __shared__ float red[8];
     const size_t base = (size_t)blockIdx.x * cols;
-    const float rl = resid_lambda ? rbf(*resid_lambda) : 0.f;
-    const float xl = x0_lambda ? rbf(*x0_lambda) : 0.f;
-    const float bl = backout_lambda ? rbf(*backout_lambda) : 0.f;
     const bool writes_x = add || padd.parts || resid_lambda || backout_lambda;
-    float p_inv_a = 0.f, p_inv_b = 0.f;
-    if (padd.parts) {
-        p_inv_a = 1.0f / scale_from_amax(amax_read(padd.a_amax));
-        p_inv_b = padd.inv_b[0];
+    const bf16_t* zsrc = resid_lambda ? x0 : (backout_lambda ? backout_src : nullptr);
+
+    // ---- every load the row needs is issued before anything waits for one: the kernel then costs one trip to memory, not one
+    // per operand (the operands are a few KB, so the trips, not the bytes, are its whole duration)
+    const float rl_raw = resid_lambda ? *resid_lambda : 0.f;
+    const float xl_raw = x0_lambda ? *x0_lambda : 0.f;
+    const float bl_raw = backout_lambda ? *backout_lambda : 0.f;
+    const float p_inv_b = padd.parts ? padd.inv_b[0] : 0.f;
+    const uint32_t p_amax_lane = padd.parts ? amax_load_lane(padd.a_amax) : 0u;
+    uint4 xv[NV], av[NV], zv[NV];
+    float4 a0[NV][8], a1[NV][8];
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int c = (threadIdx.x + it * 256) * 8;
+        if (c < cols) {
+            xv[it] = *(const uint4*)(x + base + c);
+            if (add) av[it] = *(const uint4*)(add + base + c);
+            if (zsrc) zv[it] = *(const uint4*)(zsrc + base + c);
+            if (padd.parts) {
+                const float* pp = padd.parts + (size_t)blockIdx.x * padd.ld + c;
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    const float* q = pp + (size_t)(u < padd.nsplit ? u : 0) * padd.split_stride;
+                    a0[it][u] = *(const float4*)q;
+                    a1[it][u] = *(const float4*)(q + 4);
+                }
+            }
+        }
     }
+    const float p_amax = amax_from_lanes(p_amax_lane);
+
+    // ---- arithmetic
+    const float rl = rbf(rl_raw), xl = rbf(xl_raw), bl = rbf(bl_raw);
+    const float p_inv_a = padd.parts ? 1.0f / scale_from_amax(p_amax) : 0.f;
     float v[NV][8];
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < NV; it++) {
         const int c = (threadIdx.x + it * 256) * 8;
         if (c < cols) {
-            const uint4 xv = *(const uint4*)(x + base + c);
-            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+            const uint32_t xw[4] = {xv[it].x, xv[it].y, xv[it].z, xv[it].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) v[it][2 * j] = bf16_lo(xw[j]), v[it][2 * j + 1] = bf16_hi(xw[j]);
             if (add) {
-                const uint4 av = *(const uint4*)(add + base + c);
-                const uint32_t aw[4] = {av.x, av.y, av.z, av.w};
+                const uint32_t aw[4] = {av[it].x, av[it].y, av[it].z, av[it].w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     v[it][2 * j] = rbf(v[it][2 * j] + bf16_lo(aw[j]));
@@ -152,23 +179,29 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
             }
             if (padd.parts) {
                 float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                // the sums keep the split order
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    if (u < padd.nsplit) {
+                        acc8[0] += a0[it][u].x, acc8[1] += a0[it][u].y, acc8[2] += a0[it][u].z, acc8[3] += a0[it][u].w;
+                        acc8[4] += a1[it][u].x, acc8[5] += a1[it][u].y, acc8[6] += a1[it][u].z, acc8[7] += a1[it][u].w;
+                    }
+                }
+                // splits beyond the first eight: again eight at a time, loads first
                 const float* pp = padd.parts + (size_t)blockIdx.x * padd.ld + c;
-                // eight splits at a time: all their loads are issued before the first sum (a loop with a run-time trip count
-                // makes one round trip to memory per split); the sums keep the split order
-                for (int sp0 = 0; sp0 < padd.nsplit; sp0 += 8) {
-                    float4 a0[8], a1[8];
+                for (int sp0 = 8; sp0 < padd.nsplit; sp0 += 8) {
+                    float4 b0[8], b1[8];
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
-                        const bool on = sp0 + u < padd.nsplit;
-                        const float* q = pp + (size_t)(on ? sp0 + u : sp0) * padd.split_stride;
-                        a0[u] = *(const float4*)q;
-                        a1[u] = *(const float4*)(q + 4);
+                        const float* q = pp + (size_t)(sp0 + u < padd.nsplit ? sp0 + u : sp0) * padd.split_stride;
+                        b0[u] = *(const float4*)q;
+                        b1[u] = *(const float4*)(q + 4);
                     }
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
                         if (sp0 + u < padd.nsplit) {
-                            acc8[0] += a0[u].x, acc8[1] += a0[u].y, acc8[2] += a0[u].z, acc8[3] += a0[u].w;
-                            acc8[4] += a1[u].x, acc8[5] += a1[u].y, acc8[6] += a1[u].z, acc8[7] += a1[u].w;
+                            acc8[0] += b0[u].x, acc8[1] += b0[u].y, acc8[2] += b0[u].z, acc8[3] += b0[u].w;
+                            acc8[4] += b1[u].x, acc8[5] += b1[u].y, acc8[6] += b1[u].z, acc8[7] += b1[u].w;
                         }
                     }
                 }
@@ -178,17 +211,14 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
             if (backout_save)
                 *(uint4*)(backout_save + base + c) = make_uint4(pack_bf16(v[it][0], v[it][1]), pack_bf16(v[it][2], v[it][3]),
                                                                 pack_bf16(v[it][4], v[it][5]), pack_bf16(v[it][6], v[it][7]));
+            const uint32_t zw[4] = {zv[it].x, zv[it].y, zv[it].z, zv[it].w};
             if (resid_lambda) {
-                const uint4 zv = *(const uint4*)(x0 + base + c);
-                const uint32_t zw[4] = {zv.x, zv.y, zv.z, zv.w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     v[it][2 * j] = rbf(rbf(rl * v[it][2 * j]) + rbf(xl * bf16_lo(zw[j])));
                     v[it][2 * j + 1] = rbf(rbf(rl * v[it][2 * j + 1]) + rbf(xl * bf16_hi(zw[j])));
                 }
             } else if (backout_lambda) {
-                const uint4 zv = *(const uint4*)(backout_src + base + c);
-                const uint32_t zw[4] = {zv.x, zv.y, zv.z, zv.w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     v[it][2 * j] = rbf(v[it][2 * j] - rbf(bl * bf16_lo(zw[j])));

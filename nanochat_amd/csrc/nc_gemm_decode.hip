@@ -55,6 +55,8 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
     __shared__ __align__(16) uint8_t lds[2][ROWS * 512];
     __shared__ float red[4];
 
+    NC_ARG_NOW(g.A), NC_ARG_NOW(g.a_amax), NC_ARG_NOW(g.inv_a), NC_ARG_NOW(g.B), NC_ARG_NOW(g.partial_out), NC_ARG_NOW(g.ksplits);
+    NC_ARG_NOW(g.ksteps_per_split), NC_ARG_NOW(g.M), NC_ARG_NOW(g.N), NC_ARG_NOW(g.K);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int frow = lane & 15, kb = lane >> 4;
     const int nblk = blockIdx.x, split = blockIdx.y;
@@ -70,13 +72,9 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
     if (ks_end > nksteps) ks_end = nksteps;
     const int k_hi = (ks_end << 7) < K ? (ks_end << 7) : K;       // exclusive K bound of this split
 
-    float scale = 1.f, inv_a;
-    if (A_BF16) {
-        scale = scale_from_amax(amax_read(g.a_amax));
-        inv_a = 1.0f / scale;
-    } else {
-        inv_a = *g.inv_a;
-    }
+    // the activation scale is asked for here and looked at only after the first operand loads are on their way
+    const uint32_t amax_lane = A_BF16 ? amax_load_lane(g.a_amax) : 0u;
+    float scale = 1.f, inv_a = A_BF16 ? 0.f : *g.inv_a;
 
     v4f acc[MB];
 #pragma unroll
@@ -159,8 +157,12 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
         if (nsub > 0) {
             load_b(kbase, 0);
             load_a(kbase);
-            store_a(0);
         }
+        if (A_BF16) {
+            scale = scale_from_amax(amax_from_lanes(amax_lane));
+            inv_a = 1.0f / scale;
+        }
+        if (nsub > 0) store_a(0);
         __syncthreads();
 #pragma unroll 1
         for (int sc = 0; sc < nsub; sc += 2) {
@@ -242,8 +244,13 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
                                                               const float* __restrict__ inv_b,
                                                               NcGemmSegs segs, void* __restrict__ out, int out_kind, float softcap,
                                                               uint32_t* __restrict__ out_amax, int M, int N, int ldc) {
+    NC_ARG_NOW(parts), NC_ARG_NOW(nsplit), NC_ARG_NOW(split_stride), NC_ARG_NOW(a_amax), NC_ARG_NOW(inv_a_ptr), NC_ARG_NOW(inv_b);
+    NC_ARG_NOW(out), NC_ARG_NOW(out_kind), NC_ARG_NOW(out_amax), NC_ARG_NOW(M), NC_ARG_NOW(N), NC_ARG_NOW(ldc);
     __shared__ float red[4];
-    const float inv_a = a_amax ? 1.0f / scale_from_amax(amax_read(a_amax)) : *inv_a_ptr;
+    // asked for now, looked at after the first batch of partial sums has been requested
+    const uint32_t amax_lane = a_amax ? amax_load_lane(a_amax) : 0u;
+    float inv_a = a_amax ? 0.f : *inv_a_ptr;
+    bool have_inv_a = a_amax == nullptr;
     const int n4 = N / 4;
     float am = 0.f;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)M * n4; i += (size_t)gridDim.x * 256) {
@@ -255,6 +262,7 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
             float4 p[8];
 #pragma unroll
             for (int u = 0; u < 8; u++) p[u] = *(const float4*)(pp + (size_t)(s0 + u < nsplit ? s0 + u : s0) * split_stride);
+            if (!have_inv_a) inv_a = 1.0f / scale_from_amax(amax_from_lanes(amax_lane)), have_inv_a = true;
 #pragma unroll
             for (int u = 0; u < 8; u++)
                 if (s0 + u < nsplit) a.x += p[u].x, a.y += p[u].y, a.z += p[u].z, a.w += p[u].w;

@@ -35,6 +35,8 @@ struct RopeRaw {
     float t1[PRE], t2[PRE];
     float e1, e2;             // q, k heads: cos, sin;  v heads with a value embedding: ve[lane], ve[lane + 64]
     float xg;                 // v heads: xn[lane] for lane < 12
+    float inv_b;              // partials: inverse weight scale of the head's segment
+    uint32_t amax_lane;       // partials: this lane's word of the activation amax (amax_load_lane)
 };
 
 // hh in [0, H): query head; [H, H+Hkv): key head; [H+Hkv, H+2Hkv): value head.
@@ -47,6 +49,9 @@ __device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, in
             const size_t o = (size_t)(u < r.pq.nsplit ? u : 0) * r.pq.split_stride;
             w.t1[u] = pp[o], w.t2[u] = pp[o + 64];
         }
+        // q | k | v segments end on head boundaries, so the head decides the segment
+        w.inv_b = r.pq.inv_b[hh * 128 >= r.pq.seg_end1 ? 2 : (hh * 128 >= r.pq.seg_end0 ? 1 : 0)];
+        w.amax_lane = amax_load_lane(r.pq.a_amax);
     } else {
         const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128;
         w.t1[0] = bf16_to_f32(src[lane]), w.t2[0] = bf16_to_f32(src[lane + 64]);
@@ -90,10 +95,9 @@ __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, 
             for (int u = 0; u < 8; u++)
                 if (sp0 + u < r.pq.nsplit) a1 += t1[u], a2 += t2[u];
         }
-        const float inv_a = 1.0f / scale_from_amax(amax_read(r.pq.a_amax));
-        const float inv_b = r.pq.inv_b[col >= r.pq.seg_end1 ? 2 : (col >= r.pq.seg_end0 ? 1 : 0)];
-        x1 = rbf((a1 * inv_a) * inv_b);
-        x2 = rbf((a2 * inv_a) * inv_b);
+        const float inv_a = 1.0f / scale_from_amax(amax_from_lanes(w.amax_lane));
+        x1 = rbf((a1 * inv_a) * w.inv_b);
+        x2 = rbf((a2 * inv_a) * w.inv_b);
     } else {
         x1 = w.t1[0], x2 = w.t2[0];
     }
