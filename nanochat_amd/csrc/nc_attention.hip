@@ -103,7 +103,9 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         const int th = task / (G + 2), tt = task % (G + 2), thk = hp * HP + th;
         return tt < G ? thk * G + tt : (tt == G ? H + thk : H + Hkv + thk);
     };
+    uint32_t amax_lane = 0u;
     if (FUSED) {
+        if (rope.pq.parts) amax_lane = amax_load_lane(rope.pq.a_amax);
 #pragma unroll
         for (int i = 0; i < TASKS_PER_WAVE; i++) {
             const int task = wave + 4 * i;
@@ -113,13 +115,14 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     if (k_begin < k_end) fetch(k_begin);
 
     if (FUSED) {
+        const float a_amax = amax_from_lanes(amax_lane);
 #pragma unroll
         for (int i = 0; i < TASKS_PER_WAVE; i++) {
             const int task = wave + 4 * i;
             if (task < (G + 2) * n_heads_here) {
                 const int tt = task % (G + 2), thk = hp * HP + task / (G + 2);
                 float y1, y2;
-                rope_head_finish(rope, row, task_head(task), H, Hkv, lane, raw[i], y1, y2);
+                rope_head_finish(rope, row, task_head(task), H, Hkv, lane, raw[i], a_amax, y1, y2);
                 fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
                 if (tt >= G && split == 0 && hi >= 0 && hi < Tmax) {
                     bf16_t* dst = (tt == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + thk) * 128;

@@ -255,7 +255,7 @@ __device__ __forceinline__ void amax_publish(uint32_t* h, float am) {
     if ((uintptr_t)h & 1u) p += ((blockIdx.x + 3u * blockIdx.y + 5u * blockIdx.z) % NC_AMAX_SLOTS) * NC_AMAX_STRIDE;
     // with hundreds of workgroups per slot the atomics queue up behind each other and a look first pays; with a few, the look is
     // a round trip to memory in front of an atomic that nobody waits for
-    if (gridDim.x * gridDim.y * gridDim.z > 64 * NC_AMAX_SLOTS && __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
+    if (gridDim.x * gridDim.y * gridDim.z > 16 * NC_AMAX_SLOTS && __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= bits) return;
     atomicMax(p, bits);
 }
 

@@ -120,9 +120,9 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
                                                            const float* __restrict__ x0_lambda, const float* __restrict__ backout_lambda,
                                                            const bf16_t* __restrict__ backout_src, bf16_t* __restrict__ backout_save,
                                                            bf16_t* __restrict__ xn_out, int cols, uint32_t* __restrict__ amax_ws) {
-    NC_ARG_NOW(x), NC_ARG_NOW(add), NC_ARG_NOW(padd.parts), NC_ARG_NOW(padd.nsplit), NC_ARG_NOW(padd.ld), NC_ARG_NOW(padd.split_stride);
-    NC_ARG_NOW(padd.a_amax), NC_ARG_NOW(padd.inv_b), NC_ARG_NOW(x0), NC_ARG_NOW(resid_lambda), NC_ARG_NOW(x0_lambda);
-    NC_ARG_NOW(backout_lambda), NC_ARG_NOW(backout_src), NC_ARG_NOW(backout_save), NC_ARG_NOW(xn_out), NC_ARG_NOW(cols), NC_ARG_NOW(amax_ws);
+    NC_ARG_NOW(x); NC_ARG_NOW(add); NC_ARG_NOW(padd.parts); NC_ARG_NOW(padd.nsplit); NC_ARG_NOW(padd.ld); NC_ARG_NOW(padd.split_stride);
+    NC_ARG_NOW(padd.a_amax); NC_ARG_NOW(padd.inv_b); NC_ARG_NOW(x0); NC_ARG_NOW(resid_lambda); NC_ARG_NOW(x0_lambda);
+    NC_ARG_NOW(backout_lambda); NC_ARG_NOW(backout_src); NC_ARG_NOW(backout_save); NC_ARG_NOW(xn_out); NC_ARG_NOW(cols); NC_ARG_NOW(amax_ws);
     __shared__ float red[8];
     const size_t base = (size_t)blockIdx.x * cols;
     const bool writes_x = add || padd.parts || resid_lambda || backout_lambda;

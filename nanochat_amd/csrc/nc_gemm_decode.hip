@@ -55,8 +55,8 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
     __shared__ __align__(16) uint8_t lds[2][ROWS * 512];
     __shared__ float red[4];
 
-    NC_ARG_NOW(g.A), NC_ARG_NOW(g.a_amax), NC_ARG_NOW(g.inv_a), NC_ARG_NOW(g.B), NC_ARG_NOW(g.partial_out), NC_ARG_NOW(g.ksplits);
-    NC_ARG_NOW(g.ksteps_per_split), NC_ARG_NOW(g.M), NC_ARG_NOW(g.N), NC_ARG_NOW(g.K);
+    NC_ARG_NOW(g.A); NC_ARG_NOW(g.a_amax); NC_ARG_NOW(g.inv_a); NC_ARG_NOW(g.B); NC_ARG_NOW(g.partial_out); NC_ARG_NOW(g.ksplits);
+    NC_ARG_NOW(g.ksteps_per_split); NC_ARG_NOW(g.M); NC_ARG_NOW(g.N); NC_ARG_NOW(g.K);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int frow = lane & 15, kb = lane >> 4;
     const int nblk = blockIdx.x, split = blockIdx.y;
@@ -244,8 +244,8 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
                                                               const float* __restrict__ inv_b,
                                                               NcGemmSegs segs, void* __restrict__ out, int out_kind, float softcap,
                                                               uint32_t* __restrict__ out_amax, int M, int N, int ldc) {
-    NC_ARG_NOW(parts), NC_ARG_NOW(nsplit), NC_ARG_NOW(split_stride), NC_ARG_NOW(a_amax), NC_ARG_NOW(inv_a_ptr), NC_ARG_NOW(inv_b);
-    NC_ARG_NOW(out), NC_ARG_NOW(out_kind), NC_ARG_NOW(out_amax), NC_ARG_NOW(M), NC_ARG_NOW(N), NC_ARG_NOW(ldc);
+    NC_ARG_NOW(parts); NC_ARG_NOW(nsplit); NC_ARG_NOW(split_stride); NC_ARG_NOW(a_amax); NC_ARG_NOW(inv_a_ptr); NC_ARG_NOW(inv_b);
+    NC_ARG_NOW(out); NC_ARG_NOW(out_kind); NC_ARG_NOW(out_amax); NC_ARG_NOW(M); NC_ARG_NOW(N); NC_ARG_NOW(ldc);
     __shared__ float red[4];
     // asked for now, looked at after the first batch of partial sums has been requested
     const uint32_t amax_lane = a_amax ? amax_load_lane(a_amax) : 0u;

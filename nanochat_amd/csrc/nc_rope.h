@@ -36,7 +36,6 @@ struct RopeRaw {
     float e1, e2;             // q, k heads: cos, sin;  v heads with a value embedding: ve[lane], ve[lane + 64]
     float xg;                 // v heads: xn[lane] for lane < 12
     float inv_b;              // partials: inverse weight scale of the head's segment
-    uint32_t amax_lane;       // partials: this lane's word of the activation amax (amax_load_lane)
 };
 
 // hh in [0, H): query head; [H, H+Hkv): key head; [H+Hkv, H+2Hkv): value head.
@@ -51,8 +50,8 @@ __device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, in
         }
         // q | k | v segments end on head boundaries, so the head decides the segment
         w.inv_b = r.pq.inv_b[hh * 128 >= r.pq.seg_end1 ? 2 : (hh * 128 >= r.pq.seg_end0 ? 1 : 0)];
-        w.amax_lane = amax_load_lane(r.pq.a_amax);
     } else {
+        w.inv_b = 0.f;
         const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128;
         w.t1[0] = bf16_to_f32(src[lane]), w.t2[0] = bf16_to_f32(src[lane + 64]);
     }
@@ -72,7 +71,8 @@ __device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, in
 
 // Returns the finished pair.
 template <int PRE>
-__device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, int hh, int H, int Hkv, int lane, const RopeRaw<PRE>& w, float& o1,
+__device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, int hh, int H, int Hkv, int lane, const RopeRaw<PRE>& w,
+                                                 float a_amax /* amax_from_lanes(amax_load_lane(r.pq.a_amax)) when r.pq.parts */, float& o1,
                                                  float& o2) {
     float x1, x2;
     if (r.pq.parts) {
@@ -95,7 +95,7 @@ __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, 
             for (int u = 0; u < 8; u++)
                 if (sp0 + u < r.pq.nsplit) a1 += t1[u], a2 += t2[u];
         }
-        const float inv_a = 1.0f / scale_from_amax(amax_from_lanes(w.amax_lane));
+        const float inv_a = 1.0f / scale_from_amax(a_amax);
         x1 = rbf((a1 * inv_a) * w.inv_b);
         x2 = rbf((a2 * inv_a) * w.inv_b);
     } else {
@@ -126,6 +126,7 @@ __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, 
 
 __device__ __forceinline__ void rope_head(const NcRopeSrc& r, int token, int pos, int hh, int H, int Hkv, int lane, float& o1, float& o2) {
     RopeRaw<8> w;
+    const uint32_t amax_lane = r.pq.parts ? amax_load_lane(r.pq.a_amax) : 0u;
     rope_head_load(r, token, pos, hh, H, Hkv, lane, w);
-    rope_head_finish(r, token, hh, H, Hkv, lane, w, o1, o2);
+    rope_head_finish(r, token, hh, H, Hkv, lane, w, amax_from_lanes(amax_lane), o1, o2);
 }

@@ -40,3 +40,39 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.LayerDesc) == 10 * 8 + 2 * 4
     assert ctypes.sizeof(_lib.ModelDesc) == 8 * 4 + 2 * 4 + 11 * 8
     assert ctypes.sizeof(_lib.CacheDesc) == 5 * 8 + 2 * 4
+
+
+def test_library_is_not_older_than_its_sources():
+    """A failed rebuild leaves the previous library in place; tests must not pass against a stale one."""
+    csrc = os.path.join(ROOT, "nanochat_amd", "csrc")
+    newest = max(os.path.getmtime(os.path.join(csrc, f)) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    newest = max(newest, os.path.getmtime(os.path.join(ROOT, "include", "nanochat_amd.h")))
+    assert os.path.getmtime(_lib.LIB_PATH) >= newest, "nanochat_amd/libnanochat_amd.so predates its sources: run python -m nanochat_amd.build"
+
+
+def test_hot_kernels_use_no_scratch_memory():
+    """The streaming kernels keep their state in registers: a private-memory spill costs the decode attention 15 %.
+    Compiles the sources that hold them with the resource-usage remarks on and reads the figures."""
+    import subprocess
+    from nanochat_amd import build as nb
+    # bytes of scratch per lane allowed: the persistent GEMM keeps a few tile-level addresses there (outside its K loop)
+    hot = {"nc_attention.hip": {"attn_partial_kernel": 0},
+           "nc_gemm_decode.hip": {"gemm_decode_kernel": 0, "finish_partials_kernel": 0},
+           "nc_elementwise.hip": {"mix_norm_vec_kernel": 0, "kv_prefill_copy_kernel": 0, "qkv_rope_append_kernel": 0},
+           "nc_gemm.hip": {"gemm_dl_kernel": 0, "gemm_dlp_kernel": 64}}
+    for src, kernels in hot.items():
+        cmd = ["hipcc", *nb.FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(nb.CSRC, src), "-o", os.devnull]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        name, seen = None, set()
+        for line in r.stderr.splitlines():
+            m = re.search(r"Function Name: (\S+)", line)
+            if m:
+                name = m.group(1)
+            m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+            if m and name:
+                for k in kernels:
+                    if k in name:
+                        seen.add(k)
+                        assert int(m.group(1)) <= kernels[k], f"{name} in {src} uses {m.group(1)} bytes of scratch per lane"
+        assert seen == set(kernels), f"{src}: kernels not found in the compiler's report: {set(kernels) - seen}"
