@@ -46,7 +46,8 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     __shared__ int last_flag;
     const int split = blockIdx.x, hp = blockIdx.y, row = blockIdx.z;
     const int b = row / T, t = row % T;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave index as a scalar: everything derived from it (the head tasks of this wave) then branches instead of predicating
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int grp = lane >> 4, sub = lane & 15;
     const int hsel = grp & (HP - 1), ksel = grp / HP;    // which head of the pair, which key of the instruction
     const int hk = hp * HP + hsel;                       // this lane's kv head
@@ -80,17 +81,22 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     constexpr int UNROLL = 8;     // 8 loads of 1 KB each for K and for V in flight per wave (32 keys of one head, or 16 keys of two)
     uint4 kr[UNROLL], vr[UNROLL];
     bool ok[UNROLL];
+    // Unconditional loads: a slot past the end of the run re-reads the run's last key (a valid address with finite values) and gets
+    // weight zero below, so no lane is masked off and no register is cleared around a load.  The first batch is asked for even by a
+    // wave whose run is empty (it reads row 0 and never looks at it): were the fetch behind a branch, the compiler could no longer
+    // count the loads in flight and the head tasks below would wait for the keys as well.
+    const int k_last = k_end - 1 > 0 ? k_end - 1 : 0;
     auto fetch = [&](int kb0) {
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
             const int j = kb0 + KPI * i + ksel;
             ok[i] = j < k_end && head_ok;
-            kr[i] = ok[i] ? nt_load16(kbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
+            kr[i] = nt_load16(kbase + (size_t)(j < k_end ? j : k_last) * key_stride);
         }
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
             const int j = kb0 + KPI * i + ksel;
-            vr[i] = ok[i] ? nt_load16(vbase + (size_t)j * key_stride) : make_uint4(0, 0, 0, 0);
+            vr[i] = nt_load16(vbase + (size_t)(j < k_end ? j : k_last) * key_stride);
         }
     };
     // Loads return in issue order, so the few KB that the head tasks of this wave need go out first and the first batch of keys
@@ -103,19 +109,19 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         const int th = task / (G + 2), tt = task % (G + 2), thk = hp * HP + th;
         return tt < G ? thk * G + tt : (tt == G ? H + thk : H + Hkv + thk);
     };
-    uint32_t amax_lane = 0u;
+    AmaxWords amax_words = {};
     if (FUSED) {
-        if (rope.pq.parts) amax_lane = amax_load_lane(rope.pq.a_amax);
+        if (rope.pq.parts) amax_words = amax_load_scalar(rope.pq.a_amax);
 #pragma unroll
         for (int i = 0; i < TASKS_PER_WAVE; i++) {
             const int task = wave + 4 * i;
             if (task < (G + 2) * n_heads_here) rope_head_load(rope, row, hi, task_head(task), H, Hkv, lane, raw[i]);
         }
     }
-    if (k_begin < k_end) fetch(k_begin);
+    fetch(k_begin < k_end ? k_begin : 0);
 
     if (FUSED) {
-        const float a_amax = amax_from_lanes(amax_lane);
+        const float a_amax = amax_from_words(amax_words);
 #pragma unroll
         for (int i = 0; i < TASKS_PER_WAVE; i++) {
             const int task = wave + 4 * i;

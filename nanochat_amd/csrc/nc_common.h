@@ -247,6 +247,25 @@ __device__ __forceinline__ float amax_from_lanes(uint32_t loaded) {
     }
     return __uint_as_float(m);
 }
+// And through the scalar cache, for a kernel whose vector loads must not queue behind it: scalar loads have a counter of their own,
+// so the words can be asked for first and looked at last without the compiler having to count vector loads in between.
+struct AmaxWords { uint32_t w[NC_AMAX_SLOTS]; };
+__device__ __forceinline__ AmaxWords amax_load_scalar(const uint32_t* h) {
+    const uint32_t* p = (const uint32_t*)((uintptr_t)h & ~(uintptr_t)3);
+    const int stride = ((uintptr_t)h & 1u) ? NC_AMAX_STRIDE : 0;
+    AmaxWords a;
+#pragma unroll
+    for (int i = 0; i < NC_AMAX_SLOTS; i++) a.w[i] = p[i * stride];
+    return a;
+}
+__device__ __forceinline__ float amax_from_words(AmaxWords a) {
+    uint32_t m = 0u;
+#pragma unroll
+    for (int i = 0; i < NC_AMAX_SLOTS; i++) {
+        m = a.w[i] > m ? a.w[i] : m;
+    }
+    return __uint_as_float(m);
+}
 // One call per workgroup.  The atomic is skipped when the word already holds at least the value.
 __device__ __forceinline__ void amax_publish(uint32_t* h, float am) {
     const uint32_t bits = __float_as_uint(am);

@@ -32,15 +32,22 @@ struct NcRopeSrc {
 // twelve gate inputs (lane c < 12 holds channel c).
 template <int PRE>
 struct RopeRaw {
-    float t1[PRE], t2[PRE];
-    float e1, e2;             // q, k heads: cos, sin;  v heads with a value embedding: ve[lane], ve[lane + 64]
-    float xg;                 // v heads: xn[lane] for lane < 12
+    // exactly what the loads returned: a conversion at load time would make the loading code wait for the value
+    float t1[PRE], t2[PRE];   // partial sums; without partials t1[0], t2[0] hold the two bf16 values as loaded (bits in the low half)
+    uint32_t e1, e2;          // q, k heads: cos, sin;  v heads with a value embedding: ve[lane], ve[lane + 64]   (bf16 bits)
+    uint32_t xg;              // v heads: xn[lane] for lane < 12   (bf16 bits)
     float inv_b;              // partials: inverse weight scale of the head's segment
 };
 
 // hh in [0, H): query head; [H, H+Hkv): key head; [H+Hkv, H+2Hkv): value head.
 template <int PRE>
 __device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, int pos, int hh, int H, int Hkv, int lane, RopeRaw<PRE>& w) {
+    // every field gets a value before the first load is issued (a store to a register that may hold a pending load makes the
+    // compiler wait for the load; an unset field sends the whole struct to scratch memory)
+    w.e1 = w.e2 = w.xg = 0u;
+    w.inv_b = 0.f;
+#pragma unroll
+    for (int u = 0; u < PRE; u++) w.t1[u] = w.t2[u] = 0.f;
     if (r.pq.parts) {
         const float* pp = r.pq.parts + (size_t)token * r.pq.ld + hh * 128 + lane;
 #pragma unroll
@@ -51,21 +58,20 @@ __device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, in
         // q | k | v segments end on head boundaries, so the head decides the segment
         w.inv_b = r.pq.inv_b[hh * 128 >= r.pq.seg_end1 ? 2 : (hh * 128 >= r.pq.seg_end0 ? 1 : 0)];
     } else {
-        w.inv_b = 0.f;
         const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128;
-        w.t1[0] = bf16_to_f32(src[lane]), w.t2[0] = bf16_to_f32(src[lane + 64]);
+        w.t1[0] = __uint_as_float((uint32_t)src[lane]), w.t2[0] = __uint_as_float((uint32_t)src[lane + 64]);
     }
-    w.e1 = w.e2 = w.xg = 0.f;
     if (hh < H + Hkv) {
         const int rp = pos < r.rope_len ? (pos < 0 ? 0 : pos) : r.rope_len - 1;
-        w.e1 = bf16_to_f32(r.cos_t[(size_t)rp * 64 + lane]), w.e2 = bf16_to_f32(r.sin_t[(size_t)rp * 64 + lane]);
+        w.e1 = r.cos_t[(size_t)rp * 64 + lane], w.e2 = r.sin_t[(size_t)rp * 64 + lane];
+        w.xg = r.cos_t[lane];      // never read for a q or k head; loaded so that xg is the result of a load on every path (see above)
     } else if (r.ve_table) {
         const int hv = hh - H - Hkv;
         int64_t tok = r.idx[token];
         if (tok < 0 || tok >= r.vocab_rows) tok = 0;
         const bf16_t* ve = r.ve_table + ((size_t)tok * Hkv + hv) * 128;
-        w.e1 = bf16_to_f32(ve[lane]), w.e2 = bf16_to_f32(ve[lane + 64]);
-        w.xg = bf16_to_f32(r.xn[(size_t)token * r.ld_xn + (lane < 12 ? lane : 0)]);
+        w.e1 = ve[lane], w.e2 = ve[lane + 64];
+        w.xg = r.xn[(size_t)token * r.ld_xn + (lane < 12 ? lane : 0)];
     }
 }
 
@@ -74,6 +80,11 @@ template <int PRE>
 __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, int hh, int H, int Hkv, int lane, const RopeRaw<PRE>& w,
                                                  float a_amax /* amax_from_lanes(amax_load_lane(r.pq.a_amax)) when r.pq.parts */, float& o1,
                                                  float& o2) {
+    // The conversions below must stay here: moved up to the loads (the compiler does that when it merges the branches of the load
+    // step) they would make the loading code wait.  An empty asm that "rewrites" the raw values pins their first use to this point.
+    uint32_t e1 = w.e1, e2 = w.e2, xg = w.xg;
+    float t10 = w.t1[0], t20 = w.t2[0];
+    asm volatile("" : "+v"(e1), "+v"(e2), "+v"(xg), "+v"(t10), "+v"(t20)::"memory");
     float x1, x2;
     if (r.pq.parts) {
         // the linear's output still sits in split partials: add them up in split order, scale, round to bf16
@@ -81,7 +92,7 @@ __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, 
         float a1 = 0.f, a2 = 0.f;
 #pragma unroll
         for (int u = 0; u < PRE; u++)
-            if (u < r.pq.nsplit) a1 += w.t1[u], a2 += w.t2[u];
+            if (u < r.pq.nsplit) a1 += u ? w.t1[u] : t10, a2 += u ? w.t2[u] : t20;
         // splits beyond the first PRE, eight at a time, loads first, sums after (see mix_norm_vec_kernel)
         const float* pp = r.pq.parts + (size_t)token * r.pq.ld + col;
         for (int sp0 = PRE; sp0 < r.pq.nsplit; sp0 += 8) {
@@ -99,10 +110,10 @@ __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, 
         x1 = rbf((a1 * inv_a) * w.inv_b);
         x2 = rbf((a2 * inv_a) * w.inv_b);
     } else {
-        x1 = w.t1[0], x2 = w.t2[0];
+        x1 = bf16_to_f32((bf16_t)__float_as_uint(t10)), x2 = bf16_to_f32((bf16_t)__float_as_uint(t20));
     }
     if (hh < H + Hkv) {
-        const float c = w.e1, s = w.e2;
+        const float c = bf16_to_f32((bf16_t)e1), s = bf16_to_f32((bf16_t)e2);
         float y1 = rbf(rbf(x1 * c) + rbf(x2 * s));
         float y2 = rbf(rbf(x1 * (-s)) + rbf(x2 * c));
         const float ss = wave_sum(y1 * y1 + y2 * y2);
@@ -115,10 +126,10 @@ __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, 
             float dot = 0.f;
 #pragma unroll
             for (int cidx = 0; cidx < 12; cidx++)
-                dot += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w.xg), cidx)) * rbf(r.ve_gate_w[hv * 12 + cidx]);
+                dot += bf16_to_f32((bf16_t)__builtin_amdgcn_readlane((int)xg, cidx)) * rbf(r.ve_gate_w[hv * 12 + cidx]);
             const float gate = rbf(3.0f * rbf(sigmoidf_(rbf(dot))));
-            x1 = rbf(x1 + rbf(gate * w.e1));
-            x2 = rbf(x2 + rbf(gate * w.e2));
+            x1 = rbf(x1 + rbf(gate * bf16_to_f32((bf16_t)e1)));
+            x2 = rbf(x2 + rbf(gate * bf16_to_f32((bf16_t)e2)));
         }
         o1 = x1, o2 = x2;
     }
