@@ -256,6 +256,12 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)M * n4; i += (size_t)gridDim.x * 256) {
         const int m = (int)(i / n4), n = (int)(i % n4) * 4;
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        // the weight scale of the column's segment is asked for together with the partial sums, not after them
+        int sg = 0;
+#pragma unroll
+        for (int k = 0; k < 3; k++)
+            if (k + 1 < segs.nseg && n >= segs.end[k]) sg = k + 1;
+        const float ib = inv_b[sg];
         // eight splits at a time: loads first, sums after in split order (one round trip to memory, not one per split)
         const float* pp = parts + (size_t)m * N + n;
         for (int s0 = 0; s0 < nsplit; s0 += 8) {
@@ -267,11 +273,6 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
             for (int u = 0; u < 8; u++)
                 if (s0 + u < nsplit) a.x += p[u].x, a.y += p[u].y, a.z += p[u].z, a.w += p[u].w;
         }
-        int sg = 0;
-#pragma unroll
-        for (int k = 0; k < 3; k++)
-            if (k + 1 < segs.nseg && n >= segs.end[k]) sg = k + 1;
-        const float ib = inv_b[sg];
         float v[4] = {(a.x * inv_a) * ib, (a.y * inv_a) * ib, (a.z * inv_a) * ib, (a.w * inv_a) * ib};
         if (out_kind == 1) {
             float* o = (float*)out + (size_t)m * ldc + n;
