@@ -86,6 +86,11 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m nanochat_amd.build` "
                                "(there is no non-HIP fallback)")
+        # a rebuild that failed leaves the previous library in place: refuse one whose build stamp names other sources
+        from . import build as _build
+        if os.path.exists(_build.STAMP_PATH) and open(_build.STAMP_PATH).read().strip() != _build.sources_digest():
+            raise RuntimeError(f"{LIB_PATH} was built from other sources than this tree holds: rebuild it with "
+                               "`python -m nanochat_amd.build`")
         _lib = _bind(C.CDLL(LIB_PATH))
     return _lib
 

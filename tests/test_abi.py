@@ -42,12 +42,13 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.CacheDesc) == 5 * 8 + 2 * 4
 
 
-def test_library_is_not_older_than_its_sources():
-    """A failed rebuild leaves the previous library in place; tests must not pass against a stale one."""
-    csrc = os.path.join(ROOT, "nanochat_amd", "csrc")
-    newest = max(os.path.getmtime(os.path.join(csrc, f)) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
-    newest = max(newest, os.path.getmtime(os.path.join(ROOT, "include", "nanochat_amd.h")))
-    assert os.path.getmtime(_lib.LIB_PATH) >= newest, "nanochat_amd/libnanochat_amd.so predates its sources: run python -m nanochat_amd.build"
+def test_library_was_built_from_these_sources():
+    """A failed rebuild leaves the previous library in place; tests must not pass against a stale one.  The build writes the
+    digest of its inputs next to the library."""
+    from nanochat_amd import build as nb
+    assert os.path.exists(nb.STAMP_PATH), "no build stamp next to the library: run python -m nanochat_amd.build"
+    assert open(nb.STAMP_PATH).read().strip() == nb.sources_digest(), \
+        "nanochat_amd/libnanochat_amd.so was built from other sources than the tree holds: run python -m nanochat_amd.build"
 
 
 def test_hot_kernels_use_no_scratch_memory():
