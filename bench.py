@@ -73,7 +73,7 @@ def read_profile(lib, cls):
 
 
 def gemm_rates(device, library_gemm=False):
-    """FP8 GEMM TFLOP/s at the isolated Float8Linear shapes (M=8192), kernel time by HIP events.  With library_gemm, the
+    """FP8 GEMM TFLOP/s at the isolated Float8Linear shapes (M=8192), HIP events around 100 back-to-back launches.  With library_gemm, the
     ROCm library GEMM behind torch._scaled_mm (the reference's own call, nanochat/fp8.py:143-153) is timed on the same operands
     beside it, torch events around the same 60 + 100 launches."""
     from nanochat_amd import _lib, ops
@@ -82,36 +82,15 @@ def gemm_rates(device, library_gemm=False):
     g = torch.Generator(device=device).manual_seed(0)
     for K, N in [(1664, 4992), (1664, 1664), (1664, 6656), (6656, 1664)]:
         M = 8192
-        a = torch.randn(M, K, device=device, generator=g).bfloat16()
+        a = torch.randn(M, K, device=device, generator=g)
+        a = (a * torch.where(torch.rand(M, K, device=device, generator=g) < 1e-3, 20.0, 1.0)).bfloat16()   # 0.1 % of the entries x 20
         w = ((torch.rand(N, K, device=device, generator=g) * 2 - 1) * (3.0 / K) ** 0.5).bfloat16()
         a8, ia, _ = ops.fp8_quantize(a)
         w8, iw, _ = ops.fp8_quantize(w)
         iw = iw.reshape(1)
         res = torch.empty(M, N, dtype=torch.bfloat16, device=device)
-        for _ in range(60):                    # enough back-to-back work for the clocks to settle
-            ops.fp8_gemm(a8, w8, ia, iw, out=res)
-        torch.cuda.synchronize()
-        lib.nc_profile_enable(1)
-        for _ in range(100):
-            ops.fp8_gemm(a8, w8, ia, iw, out=res)
-        torch.cuda.synchronize()
-        ms, flops, n = read_profile(lib, 1)
-        lib.nc_profile_enable(0)
-        # quantize (amax + convert) of the activation, 3 bytes per element algorithmic
-        lib.nc_profile_enable(1)
-        for _ in range(20):
-            ops.fp8_quantize(a)
-        torch.cuda.synchronize()
-        qms, qbytes, qn = read_profile(lib, 2)
-        lib.nc_profile_enable(0)
-        tf = flops / (ms * 1e-3) / 1e12
-        out[f"K{K}_N{N}"] = {"us": round(ms / n * 1e3, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
-                             "quantize_us": round(qms / qn * 1e3, 2),
-                             "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1)}
-        # the two backward GEMMs of the same layer (nanochat/fp8.py:156-192): e5m2 gradient x e4m3 saved operands
-        go = (torch.randn(M, N, device=device, generator=g) * 1e-3).bfloat16()
-
         def timed(fn, warm=30, n=50):
+            # one event pair around n back-to-back launches: the per-launch figure carries the launch gaps, not the events
             for _ in range(warm):
                 fn()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -121,6 +100,23 @@ def gemm_rates(device, library_gemm=False):
             e1.record()
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) * 1e3 / n
+        # 60 untimed launches first: enough back-to-back work for the clocks to settle
+        fwd_us = timed(lambda: ops.fp8_gemm(a8, w8, ia, iw, out=res), warm=60, n=100)
+        flops = 2.0 * M * N * K
+        # quantize (amax + convert) of the activation, 3 bytes per element algorithmic
+        lib.nc_profile_enable(1)
+        for _ in range(20):
+            ops.fp8_quantize(a)
+        torch.cuda.synchronize()
+        qms, qbytes, qn = read_profile(lib, 2)
+        lib.nc_profile_enable(0)
+        tf = flops / (fwd_us * 1e-6) / 1e12
+        out[f"K{K}_N{N}"] = {"us": round(fwd_us, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
+                             "quantize_us": round(qms / qn * 1e3, 2),
+                             "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1)}
+        # the two backward GEMMs of the same layer (nanochat/fp8.py:156-192): e5m2 gradient x e4m3 saved operands
+        go = (torch.randn(M, N, device=device, generator=g) * 1e-3).bfloat16()
+
         go8, igo, _ = ops.fp8_quantize(go, fp8_dtype=torch.float8_e5m2)
         wT, goT, xT = ops.fp8_transpose(w8), ops.fp8_transpose(go8), ops.fp8_transpose(a8)
         gi = torch.empty(M, K, dtype=torch.bfloat16, device=device)
@@ -234,6 +230,8 @@ def main():
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--library-gemm", action="store_true", help="also time torch._scaled_mm on the M=8192 GEMM operands")
     ap.add_argument("--profile-steps", type=int, default=16)
+    ap.add_argument("--window-pattern", default="SSSL",
+                    help="sliding-window pattern of the layers (the headline number is SSSL; L makes every layer read the whole context)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="after the decode steps, run an elementwise pass that reads and writes this many MiB "
                          "(a kernel of known traffic to scale hardware byte counters with)")
@@ -249,6 +247,7 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    D26["window_pattern"] = args.window_pattern
     K, W, P = args.steps, args.warmup, max(1, args.profile_steps)
     total_new = W + K + P
     prompt_len = CONTEXT - (W + K)            # the last timed step brings the context to 2048
@@ -320,14 +319,15 @@ def main():
         "vs_baseline": None,
         "dtype": "fp8_e4m3 x fp8_e4m3 -> fp32 acc (linears), bf16 (KV cache, activations)",
         "data": "synthetic: random token ids, random-init weights of the d26 architecture (seed 2)",
-        "config": {"workload": "nanochat d26 decode, batch 64, context 1792->2048, greedy, window pattern SSSL, "
+        "config": {"workload": f"nanochat d26 decode, batch 64, context 1792->2048, greedy, window pattern {args.window_pattern}, "
                                "Engine.generate loop (sample + GPT.forward with KV cache per step)",
                    "batch": BATCH, "context_end": CONTEXT, "prompt_tokens": prompt_len},
         "tpot_ms_median": round(sorted(step_times)[len(step_times) // 2] * 1e3, 4),
         "ttft_s": round(ttft, 3),
         "roofline": {"bound": "hbm", "kernel": "attn_partial_kernel (+combine) per layer launch",
                      "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4), "traffic": measured_traffic(),
+                     "frac": round(achieved / HBM_PEAK, 4),
+                     "traffic": measured_traffic() if args.window_pattern == "SSSL" else None,
                      "bytes_per_launch": int(att_bytes_launch), "avg_launch_us": round(att_avg_s * 1e6, 2),
                      "launches_timed": att_n},
         "kernel_ms_per_step": per_step_ms,
