@@ -78,7 +78,7 @@ __device__ __forceinline__ void rope_head_load(const NcRopeSrc& r, int token, in
 // Returns the finished pair.
 template <int PRE>
 __device__ __forceinline__ void rope_head_finish(const NcRopeSrc& r, int token, int hh, int H, int Hkv, int lane, const RopeRaw<PRE>& w,
-                                                 float a_amax /* amax_from_lanes(amax_load_lane(r.pq.a_amax)) when r.pq.parts */, float& o1,
+                                                 float a_amax /* amax of the linear's input (the word(s) r.pq.a_amax names), read by the caller; used with partials only */, float& o1,
                                                  float& o2) {
     // The conversions below must stay here: moved up to the loads (the compiler does that when it merges the branches of the load
     // step) they would make the loading code wait.  An empty asm that "rewrites" the raw values pins their first use to this point.
