@@ -287,6 +287,34 @@ def test_cached_decode_equals_cache_free_forward(d4_pair):
     assert (stepped.argmax(-1) == full[:, 15:].argmax(-1)).float().mean().item() > 0.5
 
 
+@pytest.mark.parametrize("cfg_kwargs,B", [(SMALL_MHA, 3), (SMALL_GQA, 70)])
+def test_decode_from_an_empty_cache(cfg_kwargs, B):
+    """One token per row per call from position 0: the first step's attention sees no cached key at all (every wave's run of
+    keys is empty and the row attends to itself only), the next ones see 1, 2, ... keys."""
+    say(f"decode from an empty cache {cfg_kwargs['n_embd']}/{cfg_kwargs['n_head']}q{cfg_kwargs['n_kv_head']}kv B={B}")
+    rt, model = build_pair(cfg_kwargs, seed=11)
+    from nanochat_amd.engine import KVCache
+    cfg = rt.cfg
+    g = torch.Generator().manual_seed(12)
+    steps = 6
+    ref = decode_ref.new_cache(cfg, B, steps, torch.bfloat16)
+    rt_def = gpt_ref.Runtime(cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+    ref_def = decode_ref.new_cache(cfg, B, steps, torch.bfloat16)
+    dec = KVCache(B, cfg.n_kv_head, steps, 128, cfg.n_layer, DEV, torch.bfloat16)
+    # whatever the cache memory holds must not matter before it is written
+    dec.k_cache.fill_(float("nan"))
+    dec.v_cache.fill_(float("nan"))
+    S, Dd, G = [], [], []
+    for s in range(steps):
+        nxt = torch.randint(0, cfg.vocab_size, (B, 1), generator=g)
+        S.append(gpt_ref.forward(rt, nxt, ref)[:, -1])
+        Dd.append(gpt_ref.forward(rt_def, nxt, ref_def)[:, -1])
+        G.append(model.forward_last(nxt.to(DEV), kv_cache=dec).cpu())
+    S, Dd, G = torch.stack(S), torch.stack(Dd), torch.stack(G)
+    assert torch.isfinite(G).all()
+    assert_within_floor(G, S, Dd, rel_l2(Dd, S), (S - Dd).abs().max().item(), "decode from an empty cache")
+
+
 @pytest.mark.parametrize("cfg_kwargs,B,P,steps", [(SMALL_GQA, 8, 40, 12), (SMALL_MHA, 5, 70, 10), (WIDE_GQA, 128, 90, 5),
                                                   (WIDE_MHA, 128, 3, 6)])
 def test_small_models_batched_decode(cfg_kwargs, B, P, steps):
@@ -305,6 +333,9 @@ def test_small_models_batched_decode(cfg_kwargs, B, P, steps):
     got = model.forward_last(prompt.to(DEV), kv_cache=pre).expand(B, -1).cpu()
     dec = KVCache(B, cfg.n_kv_head, P + steps, 128, cfg.n_layer, DEV, torch.bfloat16)
     dec.prefill(pre)
+    # positions that have not been written yet must never reach a result
+    dec.k_cache[:, :, P:] = float("nan")
+    dec.v_cache[:, :, P:] = float("nan")
     rt_def = gpt_ref.Runtime(cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
     def_pre = decode_ref.new_cache(cfg, 1, P, torch.bfloat16)
     wdef = gpt_ref.forward(rt_def, prompt, def_pre)[:, -1].expand(B, -1)
