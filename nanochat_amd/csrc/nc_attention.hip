@@ -16,6 +16,7 @@
 // query heads that share the kv head are processed by the same wave so K and V are read exactly once.
 //
 // HBM traffic per (row, kv head): 2 * n_keys * 256 bytes, the algorithmic minimum.
+#include <type_traits>
 #include "nc_common.h"
 #include "nc_kernels.h"
 #include "nc_rope.h"
@@ -80,19 +81,19 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
 
     constexpr int UNROLL = 8;     // 8 loads of 1 KB each for K and for V in flight per wave (32 keys of one head, or 16 keys of two)
     uint4 kr[UNROLL], vr[UNROLL];
-    bool ok[UNROLL];
     // Unconditional loads: a slot past the end of the run re-reads the run's last key (a valid address with finite values) and gets
     // weight zero below, so no lane is masked off and no register is cleared around a load.  The first batch is asked for even by a
     // wave whose run is empty (it reads row 0 and never looks at it): were the fetch behind a branch, the compiler could no longer
     // count the loads in flight and the head tasks below would wait for the keys as well.
     const int k_last = k_end - 1 > 0 ? k_end - 1 : 0;
-    auto fetch = [&](int kb0) {
+    auto fetch_k = [&](int kb0) {
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
             const int j = kb0 + KPI * i + ksel;
-            ok[i] = j < k_end && head_ok;
             kr[i] = nt_load16(kbase + (size_t)(j < k_end ? j : k_last) * key_stride);
         }
+    };
+    auto fetch_v = [&](int kb0) {
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
             const int j = kb0 + KPI * i + ksel;
@@ -118,7 +119,8 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             if (task < (G + 2) * n_heads_here) rope_head_load(rope, row, hi, task_head(task), H, Hkv, lane, raw[i]);
         }
     }
-    fetch(k_begin < k_end ? k_begin : 0);
+    fetch_k(k_begin < k_end ? k_begin : 0);
+    fetch_v(k_begin < k_end ? k_begin : 0);
 
     if (FUSED) {
         const float a_amax = amax_from_words(amax_words);
@@ -182,11 +184,15 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         }
     }
 
-    for (int kb0 = k_begin; kb0 < k_end; kb0 += KPI * UNROLL) {
-        if (kb0 != k_begin) fetch(kb0);
+    // One batch of keys: scores from kr, then (all but the last batch) the next batch's keys are asked for while the softmax and
+    // the value sums of this one run, and the next values once vr is free.  The last batch is a copy of the body without the
+    // prefetch, not a branch inside it: behind a branch the compiler could not count the loads in flight.
+    auto batch = [&](int kb0, auto prefetch) {
+        bool ok[UNROLL];
         float sc[G][UNROLL];
 #pragma unroll
         for (int i = 0; i < UNROLL; i++) {
+            ok[i] = kb0 + KPI * i + ksel < k_end && head_ok;
             const uint32_t w[4] = {kr[i].x, kr[i].y, kr[i].z, kr[i].w};
             float kf[8];
 #pragma unroll
@@ -200,6 +206,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
                 sc[g][i] = ok[i] ? d : NEG_BIG;
             }
         }
+        if (decltype(prefetch)::value) fetch_k(kb0 + KPI * UNROLL);
 #pragma unroll
         for (int g = 0; g < G; g++) {
             float mn = m[g];
@@ -226,6 +233,12 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
                 for (int d = 0; d < 8; d++) acc[g][d] = fmaf(sc[g][i], vf[d], acc[g][d]);
             }
         }
+        if (decltype(prefetch)::value) fetch_v(kb0 + KPI * UNROLL);
+    };
+    if (k_begin < k_end) {
+        int kb0 = k_begin;
+        for (; kb0 + KPI * UNROLL < k_end; kb0 += KPI * UNROLL) batch(kb0, std::true_type{});
+        batch(kb0, std::false_type{});
     }
 
     // merge the 16-lane groups of the wave that serve the same head (all four, or the two with the same hsel)
