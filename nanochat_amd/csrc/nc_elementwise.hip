@@ -114,7 +114,9 @@ __global__ __launch_bounds__(256) void mix_norm_kernel(bf16_t* __restrict__ x, c
 
 // Same contract as mix_norm_kernel for cols % 8 == 0 and cols <= 2048 * NV: the row stays in registers,
 // eight bf16 per 16-byte access, one reduction, one pass over memory.
-template <int NV>
+// PARTS: the addend arrives as split partial sums (decode).  Without them the kernel needs a third of the registers, and the
+// thousands of one-row workgroups of a prefill fit the chip in one round instead of two.
+template <int NV, bool PARTS>
 __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ add, NcPartialSrc padd,
                                                            const bf16_t* __restrict__ x0, const float* __restrict__ resid_lambda,
                                                            const float* __restrict__ x0_lambda, const float* __restrict__ backout_lambda,
@@ -125,7 +127,8 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
     NC_ARG_NOW(backout_lambda); NC_ARG_NOW(backout_src); NC_ARG_NOW(backout_save); NC_ARG_NOW(xn_out); NC_ARG_NOW(cols); NC_ARG_NOW(amax_ws);
     __shared__ float red[8];
     const size_t base = (size_t)blockIdx.x * cols;
-    const bool writes_x = add || padd.parts || resid_lambda || backout_lambda;
+    const bool has_parts = PARTS && padd.parts != nullptr;
+    const bool writes_x = add || has_parts || resid_lambda || backout_lambda;
     const bf16_t* zsrc = resid_lambda ? x0 : (backout_lambda ? backout_src : nullptr);
 
     // ---- every load the row needs is issued before anything waits for one: the kernel then costs one trip to memory, not one
@@ -133,10 +136,10 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
     const float rl_raw = resid_lambda ? *resid_lambda : 0.f;
     const float xl_raw = x0_lambda ? *x0_lambda : 0.f;
     const float bl_raw = backout_lambda ? *backout_lambda : 0.f;
-    const float p_inv_b = padd.parts ? padd.inv_b[0] : 0.f;
-    const uint32_t p_amax_lane = padd.parts ? amax_load_lane(padd.a_amax) : 0u;
+    const float p_inv_b = has_parts ? padd.inv_b[0] : 0.f;
+    const uint32_t p_amax_lane = has_parts ? amax_load_lane(padd.a_amax) : 0u;
     uint4 xv[NV], av[NV], zv[NV];
-    float4 a0[NV][8], a1[NV][8];
+    float4 a0[PARTS ? NV : 1][8], a1[PARTS ? NV : 1][8];
 #pragma unroll
     for (int it = 0; it < NV; it++) {
         const int c = (threadIdx.x + it * 256) * 8;
@@ -144,13 +147,13 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
             xv[it] = *(const uint4*)(x + base + c);
             if (add) av[it] = *(const uint4*)(add + base + c);
             if (zsrc) zv[it] = *(const uint4*)(zsrc + base + c);
-            if (padd.parts) {
+            if (has_parts) {
                 const float* pp = padd.parts + (size_t)blockIdx.x * padd.ld + c;
 #pragma unroll
                 for (int u = 0; u < 8; u++) {
                     const float* q = pp + (size_t)(u < padd.nsplit ? u : 0) * padd.split_stride;
-                    a0[it][u] = *(const float4*)q;
-                    a1[it][u] = *(const float4*)(q + 4);
+                    a0[PARTS ? it : 0][u] = *(const float4*)q;
+                    a1[PARTS ? it : 0][u] = *(const float4*)(q + 4);
                 }
             }
         }
@@ -159,7 +162,7 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
 
     // ---- arithmetic
     const float rl = rbf(rl_raw), xl = rbf(xl_raw), bl = rbf(bl_raw);
-    const float p_inv_a = padd.parts ? 1.0f / scale_from_amax(p_amax) : 0.f;
+    const float p_inv_a = has_parts ? 1.0f / scale_from_amax(p_amax) : 0.f;
     float v[NV][8];
     float ss = 0.f;
 #pragma unroll
@@ -177,14 +180,14 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
                     v[it][2 * j + 1] = rbf(v[it][2 * j + 1] + bf16_hi(aw[j]));
                 }
             }
-            if (padd.parts) {
+            if (has_parts) {
                 float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 // the sums keep the split order
 #pragma unroll
                 for (int u = 0; u < 8; u++) {
                     if (u < padd.nsplit) {
-                        acc8[0] += a0[it][u].x, acc8[1] += a0[it][u].y, acc8[2] += a0[it][u].z, acc8[3] += a0[it][u].w;
-                        acc8[4] += a1[it][u].x, acc8[5] += a1[it][u].y, acc8[6] += a1[it][u].z, acc8[7] += a1[it][u].w;
+                        acc8[0] += a0[PARTS ? it : 0][u].x, acc8[1] += a0[PARTS ? it : 0][u].y, acc8[2] += a0[PARTS ? it : 0][u].z, acc8[3] += a0[PARTS ? it : 0][u].w;
+                        acc8[4] += a1[PARTS ? it : 0][u].x, acc8[5] += a1[PARTS ? it : 0][u].y, acc8[6] += a1[PARTS ? it : 0][u].z, acc8[7] += a1[PARTS ? it : 0][u].w;
                     }
                 }
                 // splits beyond the first eight: again eight at a time, loads first
@@ -390,14 +393,20 @@ static int launch_mix_norm_impl(bf16_t* x, const bf16_t* add, NcPartialSrc padd,
                                             (uintptr_t)backout_save | (uintptr_t)padd.parts) & 15) == 0 && padd.ld % 4 == 0 &&
                          padd.split_stride % 4 == 0;
 #define MIX_ARGS x, add, padd, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws
-    if (aligned && cols <= 2048) hipLaunchKernelGGL(mix_norm_vec_kernel<1>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
-    else if (aligned && cols <= 4096) hipLaunchKernelGGL(mix_norm_vec_kernel<2>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
-    else if (aligned && cols <= 8192) hipLaunchKernelGGL(mix_norm_vec_kernel<4>, dim3(rows), dim3(256), 0, s, MIX_ARGS);
+#define MIX_LAUNCH(NVV)                                                                                                  \
+    do {                                                                                                                 \
+        if (padd.parts) hipLaunchKernelGGL((mix_norm_vec_kernel<NVV, true>), dim3(rows), dim3(256), 0, s, MIX_ARGS);      \
+        else hipLaunchKernelGGL((mix_norm_vec_kernel<NVV, false>), dim3(rows), dim3(256), 0, s, MIX_ARGS);                \
+    } while (0)
+    if (aligned && cols <= 2048) MIX_LAUNCH(1);
+    else if (aligned && cols <= 4096) MIX_LAUNCH(2);
+    else if (aligned && cols <= 8192) MIX_LAUNCH(4);
     else {
         NC_CHECK_ARG(!padd.parts, "mix_norm: partial-sum input needs cols %% 8 == 0, cols <= 8192 and 16-byte alignment");
         hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, add, x0, resid_lambda, x0_lambda,
                            backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws);
     }
+#undef MIX_LAUNCH
 #undef MIX_ARGS
     NC_CHECK_LAUNCH("mix_norm");
     return 0;
