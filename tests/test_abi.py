@@ -62,7 +62,10 @@ def test_hot_kernels_use_no_scratch_memory():
     hot = {"nc_attention.hip": {"attn_partial_kernel": 32},
            "nc_gemm_decode.hip": {"gemm_decode_kernel": 0, "finish_partials_kernel": 0},
            "nc_elementwise.hip": {"mix_norm_vec_kernel": 0, "kv_prefill_copy_kernel": 0, "qkv_rope_append_kernel": 0},
-           "nc_gemm.hip": {"gemm_dl_kernel": 0, "gemm_dlp_kernel": 64}}
+           "nc_gemm.hip": {"gemm_dl_kernel": 0, "gemm_dlp_kernel": 64},
+           "nc_attention_prefill.hip": {"attn_prefill_kernel": 0},
+           "nc_quantize.hip": {"amax_kernel": 0, "convert_kernel": 0, "transpose_u8_kernel": 0},
+           "nc_sample.hip": {"sample_kernel": 0}}
     for src, kernels in hot.items():
         cmd = ["hipcc", *nb.FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(nb.CSRC, src), "-o", os.devnull]
         r = subprocess.run(cmd, capture_output=True, text=True)
