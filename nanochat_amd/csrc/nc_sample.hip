@@ -45,19 +45,21 @@ __device__ __forceinline__ void block_argmax(float& v, int& i, float* sval, int*
         if (sval[k] > v || (sval[k] == v && sidx[k] < i)) v = sval[k], i = sidx[k];
 }
 
-// f(value, index) over one row of logits, 16-byte loads with four in flight per thread when the row is aligned
-template <typename F>
+// f(value, index) over one row of logits, 16-byte loads with NF in flight per thread when the row is aligned (a row of 32768
+// logits is 32 such loads per thread: with four in flight the scan is eight trips to memory, with sixteen it is two)
+template <int NF = 4, typename F>
 __device__ __forceinline__ void scan_row(const float* __restrict__ lr, int V, int tid, F f) {
     int done = 0;
     if (((uintptr_t)lr & 15) == 0) {
         const int nv = V >> 2;
         const float4* p = (const float4*)lr;
         int i = tid;
-        for (; i + 3 * SAMPLE_THREADS < nv; i += 4 * SAMPLE_THREADS) {
-            const float4 r0 = p[i], r1 = p[i + SAMPLE_THREADS], r2 = p[i + 2 * SAMPLE_THREADS], r3 = p[i + 3 * SAMPLE_THREADS];
-            const float4 r[4] = {r0, r1, r2, r3};
+        for (; i + (NF - 1) * SAMPLE_THREADS < nv; i += NF * SAMPLE_THREADS) {
+            float4 r[NF];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < NF; u++) r[u] = p[i + u * SAMPLE_THREADS];
+#pragma unroll
+            for (int u = 0; u < NF; u++) {
                 const int b = 4 * (i + u * SAMPLE_THREADS);
                 f(r[u].x, b), f(r[u].y, b + 1), f(r[u].z, b + 2), f(r[u].w, b + 3);
             }
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     if (temperature == 0.0f) {
         float bv = -INFINITY;
         int bi = 0x7fffffff;
-        scan_row(lr, V, tid, [&](float v, int i) {
+        scan_row<16>(lr, V, tid, [&](float v, int i) {
             if (v > bv || (v == bv && i < bi)) bv = v, bi = i;      // NaN never wins; an all-NaN row yields index 0 below
         });
         block_argmax(bv, bi, sval, sidx);
