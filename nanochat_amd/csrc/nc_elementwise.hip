@@ -76,6 +76,66 @@ __global__ __launch_bounds__(256) void embed_norm_smear_kernel(const int64_t* __
     }
 }
 
+// The same for one token per row (decode) with E % 8 == 0 and E <= 2048: thread c owns eight consecutive channels, the row and the
+// previous token's row are one 16-byte load each, asked for together with the gate weights, and the normalised row stays in
+// registers except for the 24 channels the gate reads.
+__global__ __launch_bounds__(256) void embed_norm_smear_decode_kernel(const int64_t* __restrict__ idx, const bf16_t* __restrict__ wte,
+                                                                      const float* __restrict__ smear_w,
+                                                                      const float* __restrict__ smear_lambda,
+                                                                      const bf16_t* __restrict__ prev_in, bf16_t* __restrict__ prev_out,
+                                                                      bf16_t* __restrict__ x_out, bf16_t* __restrict__ x0_out, int E,
+                                                                      int vocab_rows, uint32_t* __restrict__ clear_words, int n_clear) {
+    __shared__ float red[8];
+    __shared__ float head[24];
+    const int b = blockIdx.x, c0 = threadIdx.x * 8;
+    const bool mine = c0 < E;
+    int64_t tok = idx[b];
+    if (tok < 0 || tok >= vocab_rows) tok = 0;       // host validates; never read out of bounds
+    uint4 ev = make_uint4(0, 0, 0, 0), pv = make_uint4(0, 0, 0, 0);
+    if (mine) {
+        ev = *(const uint4*)(wte + (size_t)tok * E + c0);
+        if (prev_in) pv = *(const uint4*)(prev_in + (size_t)b * E + c0);
+    }
+    const float sw = (threadIdx.x & 63) < 24 ? smear_w[threadIdx.x & 63] : 0.f;      // lane c of every wave holds gate weight c
+    const float lam = *smear_lambda;
+    // first kernel of a forward pass: it also zeroes the pass's amax slots and arrival counters
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n_clear; i += gridDim.x * 256) clear_words[i] = 0u;
+
+    const uint32_t ew[4] = {ev.x, ev.y, ev.z, ev.w};
+    float v[8], ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[2 * j] = bf16_lo(ew[j]), v[2 * j + 1] = bf16_hi(ew[j]);
+#pragma unroll
+    for (int j = 0; j < 8; j++) ss += v[j] * v[j];
+    ss = block_sum<4>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)E + RMS_EPS);
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = rbf(v[j] * rstd);
+    if (mine) *(uint4*)(prev_out + (size_t)b * E + c0) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+    if (prev_in) {
+        if (threadIdx.x < 3) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) head[c0 + j] = v[j];
+        }
+        __syncthreads();
+        // gate = bf16(lambda) * sigmoid(W_s . x[:24]); every product of the chain is a bf16 tensor in eager mode
+        float dot = 0.f;
+        for (int c = 0; c < 24; c++) dot += head[c] * rbf(__shfl(sw, c));
+        const float gate = rbf(rbf(lam) * rbf(sigmoidf_(rbf(dot))));
+        const uint32_t pw[4] = {pv.x, pv.y, pv.z, pv.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[2 * j] = rbf(v[2 * j] + rbf(gate * bf16_lo(pw[j])));
+            v[2 * j + 1] = rbf(v[2 * j + 1] + rbf(gate * bf16_hi(pw[j])));
+        }
+    }
+    if (mine) {
+        const uint4 o = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+        *(uint4*)(x_out + (size_t)b * E + c0) = o;
+        if (x0_out) *(uint4*)(x0_out + (size_t)b * E + c0) = o;      // the copy the per-layer residual mix reads (gpt.py:495)
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // x1 = x (+ add);  [backout_save = x1];  x2 = rl*x1 + xl*x0  |  x1 - bl*backout_src  |  x1;
 // x = x2;  xn = rms_norm(x2);  amax(xn).                                    (gpt.py:500, 151-152, 503-508)
@@ -372,8 +432,14 @@ int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const floa
     NC_CHECK_ARG(idx && wte && smear_w && smear_lambda && prev_out && x_out, "embed_norm_smear: null pointer");
     NC_CHECK_ARG(B > 0 && T > 0 && E >= 24 && E <= 8192, "embed_norm_smear: bad shape B=%d T=%d E=%d", B, T, E);
     NcProfScope prof(3, 4.0 * B * T * E, s);
-    hipLaunchKernelGGL(embed_norm_smear_kernel, dim3(B * T), dim3(256), 2 * E * sizeof(float), s, idx, wte, smear_w, smear_lambda,
-                       prev_in, prev_out, x_out, x0_out, T, E, vocab_rows, clear_words, clear_words ? n_clear : 0);
+    const bool vec = T == 1 && E % 8 == 0 && E <= 2048 &&
+                     (((uintptr_t)wte | (uintptr_t)prev_in | (uintptr_t)prev_out | (uintptr_t)x_out | (uintptr_t)x0_out) & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL(embed_norm_smear_decode_kernel, dim3(B), dim3(256), 0, s, idx, wte, smear_w, smear_lambda, prev_in, prev_out,
+                           x_out, x0_out, E, vocab_rows, clear_words, clear_words ? n_clear : 0);
+    else
+        hipLaunchKernelGGL(embed_norm_smear_kernel, dim3(B * T), dim3(256), 2 * E * sizeof(float), s, idx, wte, smear_w, smear_lambda,
+                           prev_in, prev_out, x_out, x0_out, T, E, vocab_rows, clear_words, clear_words ? n_clear : 0);
     NC_CHECK_LAUNCH("embed_norm_smear");
     return 0;
 }

@@ -516,11 +516,13 @@ def test_mix_norm_variants(ops):
     ulp_close(xn.cpu(), F.rms_norm(x3, (cols,)))
 
 
-@pytest.mark.parametrize("B,T,with_prev", [(4, 1, True), (4, 1, False), (2, 9, False)])
-def test_embed_norm_smear(ops, B, T, with_prev):
-    say(f"embed_norm_smear B={B} T={T} prev={with_prev}")
+@pytest.mark.parametrize("B,T,with_prev,E", [(4, 1, True, 256), (4, 1, False, 256), (2, 9, False, 256), (5, 1, True, 1664),
+                                             (3, 1, True, 2048), (3, 1, True, 4096), (2, 1, True, 260), (2, 3, False, 1664)])
+def test_embed_norm_smear(ops, B, T, with_prev, E):
+    """E = 1664 / 2048: the one-token kernel with all four waves at work; 4096 and 260 (not a multiple of 8): the general one."""
+    say(f"embed_norm_smear B={B} T={T} prev={with_prev} E={E}")
     g = torch.Generator().manual_seed(1)
-    V, E = 512, 256
+    V = 512
     wte = torch.randn(V, E, generator=g).bfloat16()
     sw = (torch.rand(1, 24, generator=g) - 0.5)
     lam = torch.tensor([0.35])
