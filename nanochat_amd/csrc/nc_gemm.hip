@@ -633,6 +633,7 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
                                              const DlGeom& g, int m0, int n0, int M, int N) {
     constexpr int WTN = HALF ? 4 : 8, WCOLS = WTN * 16, ROWB = WCOLS * 2, LPR = ROWB / 16, RPI = 64 / LPR;
     const bool vec16 = (ep.ldc % 8 == 0) && (((uintptr_t)ep.out & 15) == 0);
+    const uint32_t reg_off = (uint32_t)(uintptr_t)(lds_ptr_t)reg;       // the region's byte offset in LDS
     constexpr bool relu2 = RELU2;
     float am = 0.f;
     const int lrow_e = g.lane / LPR, c = g.lane % LPR;
@@ -658,18 +659,28 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
                 o4[r] = (a4[r] * inv_a) * inv_b[j];
                 if (relu2) o4[r] = relu2_of(o4[r]);
             }
-            const uint2 pk = make_uint2(pack_bf16_hw(o4[0], o4[1]), pack_bf16_hw(o4[2], o4[3]));
-            *(uint2*)(reg + g.frow * ROWB + ((chunk ^ (g.frow & 7)) << 4) + (g.kb & 1) * 8) = pk;
+            const v2i pk = {(int)pack_bf16_hw(o4[0], o4[1]), (int)pack_bf16_hw(o4[2], o4[3])};
+            // written and read back with explicit instructions: an LDS access the compiler generates here waits for the next
+            // tile's operand loads (vmcnt(0)), because it cannot tell this region from the stages they are landing in
+            asm volatile("ds_write_b64 %0, %1" ::"v"(reg_off + g.frow * ROWB + ((chunk ^ (g.frow & 7)) << 4) + (g.kb & 1) * 8), "v"(pk) : "memory");
         }
         // the region is private to the wave: its own LDS writes only have to land before its reads
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_s_waitcnt(0xc07f);                    // lgkmcnt(0)
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        v4i rd[16 / RPI];
+#pragma unroll
+        for (int it = 0; it < 16 / RPI; it++) {
+            const int row = it * RPI + lrow_e;
+            asm volatile("ds_read_b128 %0, %1" : "=v"(rd[it]) : "v"(reg_off + row * ROWB + ((c ^ (row & 7)) << 4)) : "memory");
+        }
+        if (16 / RPI == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rd[0]), "+v"(rd[1]), "+v"(rd[2 % (16 / RPI)]), "+v"(rd[3 % (16 / RPI)])::"memory");
+        else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rd[0]), "+v"(rd[1])::"memory");
 #pragma unroll
         for (int it = 0; it < 16 / RPI; it++) {
             const int row = it * RPI + lrow_e;
             const int m = m0 + g.wm * 64 + i * 16 + row;
-            const uint4 v = *(const uint4*)(reg + row * ROWB + ((c ^ (row & 7)) << 4));
+            const uint4 v = make_uint4((uint32_t)rd[it][0], (uint32_t)rd[it][1], (uint32_t)rd[it][2], (uint32_t)rd[it][3]);
             if (m >= M || n_st >= N) continue;
             if (relu2) am = fmaxf(am, max_bf16x8(v, N - n_st));
             bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n_st;
@@ -704,6 +715,7 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
     constexpr int STAGE = 512 * 128;
     extern __shared__ __align__(16) uint8_t lds[];
     const DlGeom g = dl_geom();
+    const int wave_s = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
     const int cols = 32 / rows_per_xcd;
     const int sc_c = slot % cols, sc_r = slot / cols;
@@ -732,10 +744,16 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
     auto set_fetch_item = [&](int q) {
         int n0;
         item(q, n0, f_half);
+        // The lane's row and chunk are worked out again here from the lane id rather than kept in registers across the K loop:
+        // the kernel has none to spare (kept live, the row offset was spilled, and its reload put a vmcnt(0) into the stream
+        // of operand loads once per tile).  The asm keeps the compiler from hoisting the computation back out.
+        int lane_id;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_id));
+        const int sub = lane_id >> 3, gch = (lane_id & 7) ^ sub ^ (wave_s & 1);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int rb = n0 + 8 * g.wave + 64 * i + g.sub;
-            vo_b[i] = rb < N ? (uint32_t)rb * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+            const int rb = n0 + 8 * wave_s + 64 * i + sub;
+            vo_b[i] = rb < N ? (uint32_t)rb * (uint32_t)K + gch * 16 : NC_BUF_OOB;
         }
     };
     auto fetch_next = [&]() {
@@ -756,11 +774,14 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
         }
     };
 
-    const float inv_a = *ep.inv_a;
+    // the scales live in scalar registers across the K loops (as vector registers they were spilled, and the reloads in the
+    // epilogue waited for the operand loads issued just before it)
+    auto uniform = [](float v) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(v))); };
+    const float inv_a = uniform(*ep.inv_a);
     float sc[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
-    uint8_t* epi = lds + 2 * STAGE + g.wave * 4096;
+    for (int i = 0; i < 4; i++) sc[i] = uniform(ep.inv_b[i < ep.segs.nseg ? i : 0]);
+    uint8_t* epi = lds + 2 * STAGE + wave_s * 4096;
 
     // Invariant at the top of every K-step: its own operands have landed (the barrier before it) and the loads of the step
     // after it are already in flight.  After the barrier that ends a step, its buffer is free and takes the loads of
@@ -791,7 +812,14 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
             for (int j = 0; j < (HALF ? 4 : 8); j++) asm volatile("" : "+a"(acc[i][j]));
         int m0_here = m0;
         asm volatile("" : "+s"(m0_here));          // keeps the store addresses of all tiles from being precomputed (and spilled)
-        dlp_epilogue<HALF, RELU2>(acc, epi, ep, inv_a, sc, g, m0_here, n0, M, N);
+        // the epilogue's lane geometry is worked out afresh (see set_fetch_item): values kept for it across the K loop were
+        // spilled, and their reloads at this point waited for the next tile's operand loads that had just been issued
+        int lane_e;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+        DlGeom ge;
+        ge.lane = lane_e, ge.wave = wave_s, ge.wm = wave_s / 2, ge.wn = wave_s % 2, ge.frow = lane_e & 15, ge.kb = lane_e >> 4;
+        ge.sub = ge.gch = ge.rd_lo = ge.rd_hi = 0;
+        dlp_epilogue<HALF, RELU2>(acc, epi, ep, inv_a, sc, ge, m0_here, n0, M, N);
     };
     for (int q = 0; q < nitems; q++) {
         int n0;
