@@ -529,8 +529,13 @@ __device__ __forceinline__ void mfma_f8_first_ordered(v4f& acc, const v8i& b, co
     else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 blgp:1" : "=a"(acc) : "v"(b), "v"(a) : "memory");
 }
 // One K-step of a wave: 64 rows x (128 or, for a half-width tile, 64) columns from the stage at `st`.
-template <bool HALF, bool FIRST = false, int A_FMT = 0>
-__device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, const DlGeom& g) {
+// `behind_first_reads` runs once the step's first fragment reads are on their way: the place to issue the operand loads of a later
+// step, so that they do not stand between the barrier and the reads the first MFMA waits for.
+struct DlNothing {
+    __device__ void operator()() const {}
+};
+template <bool HALF, bool FIRST = false, int A_FMT = 0, typename F = DlNothing>
+__device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, const DlGeom& g, F&& behind_first_reads = F()) {
     constexpr int WTN = HALF ? 4 : 8;
     const uint8_t* a = st + g.wm * 64 * 128;
     const uint8_t* b = st + 256 * 128 + g.wn * (HALF ? 64 : 128) * 128;
@@ -538,6 +543,7 @@ __device__ __forceinline__ void dl_compute(v4f (&acc)[4][8], const uint8_t* st, 
     bf[0] = dl_frag(b, g);
 #pragma unroll
     for (int i = 0; i < 4; i++) af[i] = dl_frag(a + i * 2048, g);
+    behind_first_reads();
 #pragma unroll
     for (int j = 0; j < WTN; j++) {
         if (j + 1 < WTN) bf[(j + 1) & 1] = dl_frag(b + (j + 1) * 2048, g);    // one group ahead of its use
@@ -571,6 +577,7 @@ __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict_
     tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
     const int m0 = tm * 256, n0 = tn * 256;
     const DlGeom g = dl_geom();
+    const int wave_s = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, M * K, 0x00020000);
     const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, N * K, 0x00020000);
 
@@ -592,7 +599,7 @@ __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict_
 
     auto fetch = [&](int t, int buf) {
         if (t < ksteps) {
-            uint8_t* st = lds + buf * STAGE + g.wave * 1024;
+            uint8_t* st = lds + buf * STAGE + wave_s * 1024;      // uniform: the LDS address of a load goes through M0
 #pragma unroll
             for (int i = 0; i < 8; i++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 4 ? desc_a : desc_b, (lds_ptr_t)(st + i * 8192), 16, vo[i], t * 128, 0, 0);
@@ -604,11 +611,9 @@ __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict_
     dl_step_barrier();
     int kt = 0;
     for (; kt + 1 < ksteps; kt += 2) {
-        fetch(kt + 1, 1);
-        dl_compute<false, false, A_FMT>(acc, lds, g);
+        dl_compute<false, false, A_FMT>(acc, lds, g, [&] { fetch(kt + 1, 1); });
         dl_step_barrier();
-        fetch(kt + 2, 0);
-        dl_compute<false, false, A_FMT>(acc, lds + STAGE, g);
+        dl_compute<false, false, A_FMT>(acc, lds + STAGE, g, [&] { fetch(kt + 2, 0); });
         dl_step_barrier();
     }
     if (kt < ksteps) dl_compute<false, false, A_FMT>(acc, lds, g);
@@ -758,7 +763,7 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
     };
     auto fetch_next = [&]() {
         if (fq >= nitems) return;
-        uint8_t* st = lds + fbuf * STAGE + g.wave * 1024;
+        uint8_t* st = lds + fbuf * STAGE + wave_s * 1024;      // uniform: the LDS address of a load goes through M0
 #pragma unroll
         for (int i = 0; i < 4; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (lds_ptr_t)(st + i * 8192), 16, vo_a[i], fkt * 128, 0, 0);
 #pragma unroll
@@ -797,13 +802,13 @@ __global__ __launch_bounds__(512) void gemm_dlp_kernel(const uint8_t* __restrict
         dl_compute<HALF, true, A_FMT>(acc, lds + buf * STAGE, g);
         dl_step_barrier();
         buf ^= 1;
-        fetch_next();
         for (int kt = 1; kt < ksteps; kt++) {
-            dl_compute<HALF, false, A_FMT>(acc, lds + buf * STAGE, g);
+            // the loads into the buffer that the barrier has just freed go out behind this step's first fragment reads
+            dl_compute<HALF, false, A_FMT>(acc, lds + buf * STAGE, g, fetch_next);
             dl_step_barrier();
             buf ^= 1;
-            fetch_next();
         }
+        fetch_next();
         // the last MFMAs must have left the pipeline before the accumulators are read
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
