@@ -64,11 +64,6 @@ int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const
                    const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap, int M, int N,
                    int K, int ldc, int kernel, void* workspace, size_t workspace_bytes, nc_stream_t stream);
 
-/* (1)+(2) fused for decode, M <= 128: Float8Linear.forward (nanochat/fp8.py:202-213) in one launch.
- * a_bf16 [M,K] is quantized inside the kernel with the tensorwise scale derived from *a_amax (fp32
- * bits of max|a|, e.g. produced by nc_rmsnorm / nc_mix_norm / nc_decode_attention), bit-identical to
- * nc_fp8_quantize_tensorwise followed by nc_fp8_gemm_tn.  out_kind 0/1 as above; out_kind 2 writes
- * bf16 relu(bf16(v))^2 (nanochat/gpt.py:139) and max-reduces it into *out_amax.  ksplits 0 = choose. */
 /* The backward GEMMs of nanochat/fp8.py:166-190 (torch._scaled_mm with an e5m2 first operand):
  * out[M,N] = bf16((a[M,K] . b[N,K]^T, fp32 accumulate) * *inv_a * *inv_b), a in e5m2 (the quantized output gradient or
  * its transpose), b in e4m3fn (the transposed weight or input payload saved by the forward), K contiguous in both.
@@ -84,6 +79,11 @@ int nc_fp8_gemm_tn_grad(const uint8_t* a_e5m2, const uint8_t* b, const float* in
 int nc_fp8_gemm_tn_relu2(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, void* out,
                          uint32_t* out_amax, int M, int N, int K, int ldc, int kernel, nc_stream_t stream);
 
+/* (1)+(2) fused for decode, M <= 128: Float8Linear.forward (nanochat/fp8.py:202-213) in one launch.
+ * a_bf16 [M,K] is quantized inside the kernel with the tensorwise scale derived from *a_amax (fp32
+ * bits of max|a|, e.g. produced by nc_rmsnorm / nc_mix_norm / nc_decode_attention), bit-identical to
+ * nc_fp8_quantize_tensorwise followed by nc_fp8_gemm_tn.  out_kind 0/1 as above; out_kind 2 writes
+ * bf16 relu(bf16(v))^2 (nanochat/gpt.py:139) and max-reduces it into *out_amax.  ksplits 0 = choose. */
 size_t nc_fp8_small_m_workspace_bytes(int M, int N, int K);
 int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const uint8_t* b, const float* inv_b,
                           const int32_t* seg_ends, int nseg, void* out, int out_kind, float softcap,
@@ -137,6 +137,33 @@ int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16
                         const int32_t* cache_seqlens, int window_left, uint16_t* out, int B, int T, int H, int Hkv,
                         int Tmax, int seqlens_include_new, void* workspace, size_t workspace_bytes,
                         uint32_t* amax_ws, int splits, nc_stream_t stream);
+
+/* The same call with the new keys and values handed over, as the reference hands them: flash_attn_with_kvcache(q, k_cache,
+ * v_cache, k=k_new, v=v_new, cache_seqlens=..., causal=True, window_size=(w, 0)) at nanochat/gpt.py:113-120, whose in-place
+ * insert is nanochat/flash_attention.py:167-170.  k_new, v_new bf16 [B*T,Hkv,128] go to slots cache_seqlens[b] .. +T-1 of the
+ * caches (slots outside [0,Tmax) are skipped), then the T queries of every row attend as above; cache_seqlens counts the
+ * tokens BEFORE this call and is not advanced (the caller does that, nanochat/gpt.py:122-123).  With T = 1 the attention
+ * workgroups append their own heads and take the new key and value from on-chip memory. */
+int nc_decode_attention_append(const uint16_t* q, const uint16_t* k_new, const uint16_t* v_new, uint16_t* k_cache,
+                               uint16_t* v_cache, const int32_t* cache_seqlens, int window_left, uint16_t* out, int B, int T,
+                               int H, int Hkv, int Tmax, void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits,
+                               nc_stream_t stream);
+
+/* (4d)+(3) in one launch for decode (one new token per row): nc_qkv_rope_append followed by nc_decode_attention, i.e.
+ * nanochat/gpt.py:89-120 from the q|k|v linear's output to the attention output: rotary, QK-norm and gain on q and k, the
+ * value-embedding gate on v, the in-place append at cache_seqlens[b], attention over [max(0,p-window_left), p].  Arguments
+ * as for the two calls; out bf16 [B,H,128].  This is the kernel the whole-model forward uses at decode. */
+int nc_qkv_rope_append_attention(const uint16_t* qkv, int ld_qkv, const uint16_t* xn, int ld_xn, const int64_t* idx,
+                                 const uint16_t* ve_table, const float* ve_gate_w, const uint16_t* cos, const uint16_t* sin,
+                                 int rope_len, const int32_t* cache_seqlens, uint16_t* k_cache, uint16_t* v_cache,
+                                 int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax, int vocab_rows,
+                                 void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits, nc_stream_t stream);
+
+/* How a decode-attention launch of this shape is laid out (no counterpart in the reference; for tests and tuning):
+ * *splits_out = workgroups that share the keys of one (row, kv head); *heads_per_workgroup_out = 1, or 2 when a workgroup
+ * streams two neighbouring kv heads.  splits: the caller's request (0 = choose), as passed to the attention calls. */
+int nc_decode_attention_plan(int B, int T, int Hkv, int window_left, int Tmax, int splits, int* splits_out /*host*/,
+                             int* heads_per_workgroup_out /*host*/);
 
 /* KVCache.prefill: nanochat/engine.py:123-137.  Copies the first n_tokens positions of every (layer, row) of one
  * cache tensor (keys or values), laid out [layers, src_rows, src_tmax, token_bytes], into every row of
@@ -207,6 +234,15 @@ size_t nc_gpt_workspace_bytes(const nc_model_desc* model /*host*/, int B, int T)
 int nc_gpt_forward(const nc_model_desc* model /*host*/, const nc_cache_desc* cache /*host*/, const int64_t* idx,
                    int B, int T, float* logits_out, int last_only, void* workspace, size_t workspace_bytes,
                    nc_stream_t stream);
+
+/* The same forward with its intermediate activations copied out, for layer-by-layer comparison with another implementation
+ * (no counterpart in the reference; tests only).  tap_x (or NULL): bf16 [n_layer+1, B*T, E]; slot i is the residual stream as
+ * layer i reads it, i.e. after `x = resid_lambdas[i]*x + x0_lambdas[i]*x0` (nanochat/gpt.py:500), slot n_layer the final
+ * normalised rows that lm_head reads (gpt.py:508).  tap_y (or NULL): bf16 [n_layer, B*T, H*128], the attention outputs
+ * before c_proj (gpt.py:113-124). */
+int nc_gpt_forward_tapped(const nc_model_desc* model /*host*/, const nc_cache_desc* cache /*host*/, const int64_t* idx,
+                          int B, int T, float* logits_out, int last_only, void* workspace, size_t workspace_bytes,
+                          uint16_t* tap_x, uint16_t* tap_y, nc_stream_t stream);
 
 /* ---- measurement aid (no counterpart in the reference) --------------------------------------
  * While enabled, every launch made by this library is bracketed by a HIP event pair on its stream.

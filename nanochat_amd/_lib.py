@@ -15,6 +15,7 @@ EXPORTS = [
     "nc_rmsnorm", "nc_embed_norm_smear", "nc_mix_norm", "nc_relu2", "nc_qkv_rope_append",
     "nc_attention_workspace_bytes", "nc_decode_attention", "nc_kv_cache_prefill", "nc_softcap", "nc_sample",
     "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read",
+    "nc_decode_attention_append", "nc_qkv_rope_append_attention", "nc_decode_attention_plan", "nc_gpt_forward_tapped",
 ]
 
 
@@ -64,11 +65,15 @@ def _bind(lib):
         "nc_qkv_rope_append": (i, [p, i, p, i, p, p, p, p, p, i, p, p, p, p, i, i, i, i, i, i, p]),
         "nc_attention_workspace_bytes": (sz, [i, i, i, i]),
         "nc_decode_attention": (i, [p, p, p, p, i, p, i, i, i, i, i, i, p, sz, p, i, p]),
+        "nc_decode_attention_append": (i, [p, p, p, p, p, p, i, p, i, i, i, i, i, p, sz, p, i, p]),
+        "nc_qkv_rope_append_attention": (i, [p, i, p, i, p, p, p, p, p, i, p, p, p, i, p, i, i, i, i, i, p, sz, p, i, p]),
+        "nc_decode_attention_plan": (i, [i, i, i, i, i, i, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
         "nc_kv_cache_prefill": (i, [p, p, i, i, i, i, i, i, i, p]),
         "nc_softcap": (i, [p, p, i64, f, p]),
         "nc_sample": (i, [p, i, i, i, f, i, p, p, p]),
         "nc_gpt_workspace_bytes": (sz, [C.POINTER(ModelDesc), i, i]),
         "nc_gpt_forward": (i, [C.POINTER(ModelDesc), C.POINTER(CacheDesc), p, i, i, p, i, p, sz, p]),
+        "nc_gpt_forward_tapped": (i, [C.POINTER(ModelDesc), C.POINTER(CacheDesc), p, i, i, p, i, p, sz, p, p, p]),
         "nc_profile_enable": (i, [i]),
         "nc_profile_read": (i, [i, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     }

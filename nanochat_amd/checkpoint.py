@@ -37,7 +37,7 @@ def load_checkpoint(checkpoint_dir, step, device):
 
 
 def build_model(checkpoint_dir, step=None, device="cuda", fp8=True):
-    """GPT on `device` in bf16 with the checkpoint's weights, FP8 linears swapped in with the reference's filter
+    """GPT on `device` holding the checkpoint's tensors as saved, FP8 linears swapped in with the reference's filter
     (scripts/base_train.py:178-185) unless fp8=False is asked for.  Returns (model, meta)."""
     if step is None:
         step = find_last_step(checkpoint_dir)
@@ -54,18 +54,18 @@ def build_model(checkpoint_dir, step=None, device="cuda", fp8=True):
         model_data["x0_lambdas"] = torch.zeros(config.n_layer)
     with torch.device("meta"):
         model = GPT(config)
-    model.to_empty(device=device)
     own = model.state_dict()
     missing = sorted(set(own) - set(model_data))
     unexpected = sorted(set(model_data) - set(own))
     if missing or unexpected:
         raise RuntimeError(f"checkpoint does not match the model: missing {missing[:4]}, unexpected {unexpected[:4]}")
-    with torch.no_grad():
-        for k, v in model_data.items():
-            if own[k].shape != v.shape:
-                raise RuntimeError(f"{k}: checkpoint shape {tuple(v.shape)} != model shape {tuple(own[k].shape)}")
-            own[k].copy_(v.to(device=device, dtype=own[k].dtype))
-    model.to(torch.bfloat16)
+    for k, v in model_data.items():
+        if own[k].shape != v.shape:
+            raise RuntimeError(f"{k}: checkpoint shape {tuple(v.shape)} != model shape {tuple(own[k].shape)}")
+    # The checkpoint's tensors become the parameters, in the dtypes they were saved in (load_state_dict(strict=True,
+    # assign=True) at checkpoint_manager.py:104): fp32 master weights are quantized to e4m3 from fp32, as the reference's
+    # Float8Linear would do on every call.
+    model.load_state_dict({k: v.to(device) for k, v in model_data.items()}, strict=True, assign=True)
     model.eval()
     if fp8:
         convert_to_float8_training(model, module_filter_fn=fp8_module_filter)

@@ -5,6 +5,7 @@
 #include "../../include/nanochat_amd.h"
 #include "nc_common.h"
 #include "nc_kernels.h"
+#include "nc_rope.h"
 
 static thread_local char g_error[512] = "";
 
@@ -145,6 +146,47 @@ int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16
     void* parts = counters ? (uint8_t*)workspace + cb : nullptr;
     return nc_launch_attention(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new,
                                counters, parts, counters ? workspace_bytes - cb : 0, amax_ws, splits, 0, (hipStream_t)stream);
+}
+
+static void split_attention_workspace(void* workspace, size_t workspace_bytes, int B, int T, int H, uint32_t** counters, void** parts,
+                                      size_t* part_bytes) {
+    const size_t cb = nc_attn_counter_bytes(B > 0 ? B : 1, T > 0 ? T : 1, H > 0 ? H : 1);
+    *counters = (workspace && workspace_bytes > cb) ? (uint32_t*)workspace : nullptr;
+    *parts = *counters ? (uint8_t*)workspace + cb : nullptr;
+    *part_bytes = *counters ? workspace_bytes - cb : 0;
+}
+
+int nc_decode_attention_append(const uint16_t* q, const uint16_t* k_new, const uint16_t* v_new, uint16_t* k_cache, uint16_t* v_cache,
+                               const int32_t* cache_seqlens, int window_left, uint16_t* out, int B, int T, int H, int Hkv, int Tmax,
+                               void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits, nc_stream_t stream) {
+    uint32_t* counters;
+    void* parts;
+    size_t part_bytes;
+    split_attention_workspace(workspace, workspace_bytes, B, T, H, &counters, &parts, &part_bytes);
+    return nc_launch_attention_append(q, k_new, v_new, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, counters, parts,
+                                      part_bytes, amax_ws, splits, (hipStream_t)stream);
+}
+
+int nc_qkv_rope_append_attention(const uint16_t* qkv, int ld_qkv, const uint16_t* xn, int ld_xn, const int64_t* idx,
+                                 const uint16_t* ve_table, const float* ve_gate_w, const uint16_t* cos, const uint16_t* sin, int rope_len,
+                                 const int32_t* cache_seqlens, uint16_t* k_cache, uint16_t* v_cache, int window_left, uint16_t* out, int B,
+                                 int H, int Hkv, int Tmax, int vocab_rows, void* workspace, size_t workspace_bytes, uint32_t* amax_ws,
+                                 int splits, nc_stream_t stream) {
+    NC_CHECK_ARG(qkv && ld_qkv >= (H + 2 * Hkv) * 128, "qkv_rope_append_attention: qkv rows of %d elements needed", (H + 2 * Hkv) * 128);
+    uint32_t* counters;
+    void* parts;
+    size_t part_bytes;
+    split_attention_workspace(workspace, workspace_bytes, B, 1, H, &counters, &parts, &part_bytes);
+    NcRopeSrc rope{qkv, ld_qkv, NcPartialSrc{nullptr, 0, 0, 0, nullptr, nullptr, 0, 0}, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin,
+                   rope_len, vocab_rows, nullptr, nullptr};
+    return nc_launch_attention_fused(rope, k_cache, v_cache, cache_seqlens, window_left, out, B, H, Hkv, Tmax, counters, parts, part_bytes,
+                                     amax_ws, splits, 0, (hipStream_t)stream);
+}
+
+int nc_decode_attention_plan(int B, int T, int Hkv, int window_left, int Tmax, int splits, int* splits_out, int* heads_per_workgroup_out) {
+    NC_CHECK_ARG(B > 0 && T > 0 && Hkv > 0 && Tmax > 0, "decode_attention_plan: bad shape");
+    nc_attention_plan(B, T, Hkv, window_left, Tmax, splits, splits_out, heads_per_workgroup_out);
+    return 0;
 }
 
 int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_stream_t stream) {

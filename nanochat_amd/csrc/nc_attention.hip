@@ -33,13 +33,17 @@
 // both heads of one key (512 contiguous bytes) and a load instruction fetches two keys: the same bytes per instruction in
 // runs twice as long, which streams ~8 % faster when there are enough workgroups left.  A lane still serves one head
 // (hsel), so the register budget does not change; an odd head count leaves the second half of the last pair idle.
-template <int G, bool FUSED, int HP>
+// MODE 0: q is given, the new tokens are already in the cache.  MODE 1: FUSED as described above.  MODE 2: q and the new key and value
+// are given finished (flash_attn_with_kvcache(q, k_cache, v_cache, k=, v=), nanochat/flash_attention.py:139-185): the workgroup
+// copies its heads of them into LDS, appends key and value to the cache and attends like MODE 1.
+template <int G, int MODE, int HP>
 __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache,
                                                            bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
                                                            float* __restrict__ partials, uint32_t* __restrict__ counters,
                                                            uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, int nsplit,
                                                            NcRopeSrc rope) {
+    constexpr bool FUSED = MODE != 0;                    // the row's own token comes from LDS, not from the cache
     constexpr int KPI = 4 / HP;                          // keys per load instruction
     constexpr int TASKS = (G + 2) * HP;                  // FUSED: per head the G query heads, then the new key and value
     __shared__ float merge[4][HP * G][PART_STRIDE];
@@ -105,18 +109,32 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     // Wave w finishes head task w, w+4, ...: per head of the pair, tasks 0..G-1 are the query heads, G the key head, G+1 the
     // value head.
     constexpr int TASKS_PER_WAVE = (TASKS + 3) / 4;
-    RopeRaw<4> raw[FUSED ? TASKS_PER_WAVE : 1];
+    RopeRaw<4> raw[MODE == 1 ? TASKS_PER_WAVE : 1];
+    uint32_t plain1[MODE == 2 ? TASKS_PER_WAVE : 1], plain2[MODE == 2 ? TASKS_PER_WAVE : 1];
     auto task_head = [&](int task) {
         const int th = task / (G + 2), tt = task % (G + 2), thk = hp * HP + th;
         return tt < G ? thk * G + tt : (tt == G ? H + thk : H + Hkv + thk);
     };
     AmaxWords amax_words = {};
-    if (FUSED) {
+    if (MODE == 1) {
         if (rope.pq.parts) amax_words = amax_load_scalar(rope.pq.a_amax);
 #pragma unroll
         for (int i = 0; i < TASKS_PER_WAVE; i++) {
             const int task = wave + 4 * i;
             if (task < (G + 2) * n_heads_here) rope_head_load(rope, row, hi, task_head(task), H, Hkv, lane, raw[i]);
+        }
+    }
+    if (MODE == 2) {
+#pragma unroll
+        for (int i = 0; i < TASKS_PER_WAVE; i++) {
+            const int task = wave + 4 * i;
+            plain1[i] = plain2[i] = 0u;
+            if (task < (G + 2) * n_heads_here) {
+                const int tt = task % (G + 2), thk = hp * HP + task / (G + 2);
+                const bf16_t* src = tt < G ? q + ((size_t)row * H + thk * G + tt) * 128
+                                           : (tt == G ? rope.k_new : rope.v_new) + ((size_t)row * Hkv + thk) * 128;
+                plain1[i] = src[lane], plain2[i] = src[lane + 64];
+            }
         }
     }
     fetch_k(k_begin < k_end ? k_begin : 0);
@@ -130,7 +148,8 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             if (task < (G + 2) * n_heads_here) {
                 const int tt = task % (G + 2), thk = hp * HP + task / (G + 2);
                 float y1, y2;
-                rope_head_finish(rope, row, task_head(task), H, Hkv, lane, raw[i], a_amax, y1, y2);
+                if (MODE == 1) rope_head_finish(rope, row, task_head(task), H, Hkv, lane, raw[i], a_amax, y1, y2);
+                else y1 = bf16_to_f32((bf16_t)plain1[i]), y2 = bf16_to_f32((bf16_t)plain2[i]);
                 fresh[task][lane] = y1, fresh[task][lane + 64] = y2;
                 if (tt >= G && split == 0 && hi >= 0 && hi < Tmax) {
                     bf16_t* dst = (tt == G ? k_cache : v_cache) + (((size_t)b * Tmax + hi) * Hkv + thk) * 128;
@@ -349,14 +368,16 @@ int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax) {
     return pick_splits(B, T, Hkv, max_keys);
 }
 
-static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens,
-                        int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
-                        uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
-                        int counters_are_zero, hipStream_t s) {
-    NC_CHECK_ARG((q || rope) && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
+// mode 0: q given, new tokens already in the cache.  mode 1: *rope names the raw q|k|v rows (rotary, QK-norm, value embedding and the
+// append are done here).  mode 2: q given, rope->k_new / rope->v_new hold the finished new key and value, appended here.
+static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, int mode, bf16_t* k_cache, bf16_t* v_cache,
+                                 const int32_t* cache_seqlens, int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax,
+                                 int seqlens_include_new, uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws,
+                                 int force_splits, int counters_are_zero, hipStream_t s) {
+    NC_CHECK_ARG((q || mode == 1) && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
     // many queries per row: the matrix-core kernel (a workgroup there covers 128 queries; below 16 queries per row
     // the per-query streaming kernel wastes less)
-    if (!rope && T >= 16 && force_splits <= 0)
+    if (mode == 0 && T >= 16 && force_splits <= 0)
         return nc_launch_attention_prefill(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new,
                                            amax_ws, s);
     NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0, "decode_attention: bad shape");
@@ -369,12 +390,15 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t*
     int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
     int nsplit = force_splits > 0 ? force_splits : pick_splits(B, T, Hkv, max_keys);
     NC_CHECK_ARG(nsplit >= 1 && nsplit <= 16, "decode_attention: splits must be 1..16");
-    if (rope) {
-        NC_CHECK_ARG(T == 1 && !seqlens_include_new, "decode_attention: the fused q|k|v finish needs one new token per row, not yet counted");
+    if (mode != 0) {
+        NC_CHECK_ARG(rope && T == 1 && !seqlens_include_new, "decode_attention: the in-kernel append needs one new token per row, not yet counted");
+    }
+    if (mode == 1) {
         NC_CHECK_ARG((rope->qkv || rope->pq.parts) && rope->cos_t && rope->sin_t && rope->rope_len > 0, "decode_attention: rotary source missing");
         NC_CHECK_ARG(!rope->ve_table || (rope->ve_gate_w && rope->xn && rope->idx && rope->ld_xn >= 12),
                      "decode_attention: value embedding needs gate weights, xn and idx");
     }
+    if (mode == 2) NC_CHECK_ARG(rope->k_new && rope->v_new, "decode_attention: new key / value missing");
     if (nsplit > 1) {
         const size_t need = (size_t)B * T * H * nsplit * PART_STRIDE * sizeof(float);
         NC_CHECK_ARG(counters && partials && partial_bytes >= need, "decode_attention: %zu bytes of split workspace needed, %zu given",
@@ -387,19 +411,20 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t*
     const int hp = (force_splits > 0 || nsplit > 1) ? 1 : pick_heads_per_wg(B, T, Hkv);
     dim3 grid(nsplit, hp == 2 ? (Hkv + 1) / 2 : Hkv, B * T), block(256);
     const NcRopeSrc none{};
-#define LAUNCH_GH(GG, HH)                                                                                                       \
-    do {                                                                                                                        \
-        if (rope)                                                                                                               \
-            hipLaunchKernelGGL((attn_partial_kernel<GG, true, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,         \
-                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, *rope);    \
-        else                                                                                                                    \
-            hipLaunchKernelGGL((attn_partial_kernel<GG, false, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,        \
-                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, none);     \
+    const NcRopeSrc& rs = rope ? *rope : none;
+#define LAUNCH_GMH(GG, MM, HH)                                                                                                \
+    hipLaunchKernelGGL((attn_partial_kernel<GG, MM, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens, window_left, \
+                       seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, rs)
+#define LAUNCH_GH(GG, HH)                          \
+    do {                                           \
+        if (mode == 1) LAUNCH_GMH(GG, 1, HH);      \
+        else if (mode == 2) LAUNCH_GMH(GG, 2, HH); \
+        else LAUNCH_GMH(GG, 0, HH);                \
     } while (0)
-#define LAUNCH_G(GG)                 \
-    do {                             \
+#define LAUNCH_G(GG)                   \
+    do {                               \
         if (hp == 2) LAUNCH_GH(GG, 2); \
-        else LAUNCH_GH(GG, 1);       \
+        else LAUNCH_GH(GG, 1);         \
     } while (0)
     if (G == 1) LAUNCH_G(1);
     else if (G == 2) LAUNCH_G(2);
@@ -407,15 +432,25 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, bf16_t*
     else LAUNCH_G(8);
 #undef LAUNCH_G
 #undef LAUNCH_GH
+#undef LAUNCH_GMH
     NC_CHECK_LAUNCH("decode_attention");
     return 0;
+}
+
+// What a launch with these shapes does: the number of key splits and the kv heads per workgroup (1 or 2).  `in_kernel_append`:
+// the decode forms that finish / append the new token themselves (they never take the many-queries kernel).
+void nc_attention_plan(int B, int T, int Hkv, int window_left, int Tmax, int force_splits, int* splits_out, int* heads_per_wg_out) {
+    const int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
+    const int nsplit = force_splits > 0 ? force_splits : pick_splits(B, T, Hkv, max_keys);
+    if (splits_out) *splits_out = nsplit;
+    if (heads_per_wg_out) *heads_per_wg_out = (force_splits > 0 || nsplit > 1) ? 1 : pick_heads_per_wg(B, T, Hkv);
 }
 
 int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
                         int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                         uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
                         int counters_are_zero, hipStream_t s) {
-    return launch_attention_impl(q, nullptr, const_cast<bf16_t*>(k_cache), const_cast<bf16_t*>(v_cache), cache_seqlens, window_left, out,
+    return launch_attention_impl(q, nullptr, 0, const_cast<bf16_t*>(k_cache), const_cast<bf16_t*>(v_cache), cache_seqlens, window_left, out,
                                  B, T, H, Hkv, Tmax, seqlens_include_new, counters, partials, partial_bytes, amax_ws, force_splits,
                                  counters_are_zero, s);
 }
@@ -425,6 +460,43 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
 int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
                               bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* counters, void* partials, size_t partial_bytes,
                               uint32_t* amax_ws, int force_splits, int counters_are_zero, hipStream_t s) {
-    return launch_attention_impl(nullptr, &rope, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, counters,
+    return launch_attention_impl(nullptr, &rope, 1, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, counters,
                                  partials, partial_bytes, amax_ws, force_splits, counters_are_zero, s);
+}
+
+// cache[b, cache_seqlens[b] + t] = new[b, t] for keys and values (nanochat/flash_attention.py:167-170 with per-row positions);
+// positions outside [0, Tmax) are skipped.  token_elems = Hkv * 128.
+__global__ void kv_append_kernel(const bf16_t* __restrict__ k_new, const bf16_t* __restrict__ v_new, bf16_t* __restrict__ k_cache,
+                                 bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens, int T, int Tmax, int token_elems) {
+    const int b = blockIdx.y, t = blockIdx.x;
+    const int pos = cache_seqlens[b] + t;
+    if (pos < 0 || pos >= Tmax) return;
+    const uint4* ks = (const uint4*)(k_new + ((size_t)b * T + t) * token_elems);
+    const uint4* vs = (const uint4*)(v_new + ((size_t)b * T + t) * token_elems);
+    uint4* kd = (uint4*)(k_cache + ((size_t)b * Tmax + pos) * token_elems);
+    uint4* vd = (uint4*)(v_cache + ((size_t)b * Tmax + pos) * token_elems);
+    for (int i = threadIdx.x; i < token_elems / 8; i += blockDim.x) kd[i] = ks[i], vd[i] = vs[i];
+}
+
+// flash_attn_with_kvcache(q, k_cache, v_cache, k=k_new, v=v_new, cache_seqlens=...): append, then attend.  One new token per row
+// is appended by the attention workgroups themselves; several go through a copy kernel and the ordinary kernels.
+int nc_launch_attention_append(const bf16_t* q, const bf16_t* k_new, const bf16_t* v_new, bf16_t* k_cache, bf16_t* v_cache,
+                               const int32_t* cache_seqlens, int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax,
+                               uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
+                               hipStream_t s) {
+    NC_CHECK_ARG(q && k_new && v_new && k_cache && v_cache && cache_seqlens && out, "attention_append: null pointer");
+    NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0 && B <= 65535, "attention_append: bad shape");
+    NC_CHECK_ARG((((uintptr_t)k_new | (uintptr_t)v_new | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0,
+                 "attention_append: pointers must be 16-byte aligned");
+    if (T == 1) {
+        NcRopeSrc src{};
+        src.k_new = k_new, src.v_new = v_new;
+        return launch_attention_impl(q, &src, 2, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, counters, partials,
+                                     partial_bytes, amax_ws, force_splits, 0, s);
+    }
+    hipLaunchKernelGGL(kv_append_kernel, dim3(T, B), dim3(Hkv * 16 < 256 ? Hkv * 16 : 256), 0, s, k_new, v_new, k_cache, v_cache,
+                       cache_seqlens, T, Tmax, Hkv * 128);
+    NC_CHECK_LAUNCH("kv_append");
+    return launch_attention_impl(q, nullptr, 0, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, 0, counters, partials,
+                                 partial_bytes, amax_ws, force_splits, 0, s);
 }

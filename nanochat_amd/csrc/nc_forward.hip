@@ -87,7 +87,16 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     w.xl = c.take<bf16_t>((size_t)B * E);
     w.inv = c.take<float>(4 * (size_t)m->n_layer + 1);
     const size_t amax_words = (4 * (size_t)m->n_layer + 1) * NC_AMAX_SLOTS * NC_AMAX_STRIDE;     // one slotted site per FP8 linear input
-    const size_t attn_words = nc_attn_counter_bytes(B, T, m->n_head) / 4;
+    // attention split counters and partials only when some layer's launch really splits its keys over workgroups (never with 16 or
+    // more queries per row, which take the matrix-core kernel, and never once rows x kv heads fill the chip); the cache length is not
+    // known here, so each layer is sized for its whole window
+    int max_splits = 1;
+    if (T < 16)
+        for (int i = 0; i < m->n_layer; i++) {
+            const int sp = nc_attn_splits(B, T, m->n_kv_head, m->layers ? m->layers[i].window_left : -1, 1 << 30);
+            max_splits = sp > max_splits ? sp : max_splits;
+        }
+    const size_t attn_words = max_splits > 1 ? nc_attn_counter_bytes(B, T, m->n_head) / 4 : 0;
     uint32_t* zero = c.take<uint32_t>(amax_words + attn_words);
     w.amax = zero;
     w.attn_counters = zero ? zero + amax_words : nullptr;
@@ -103,7 +112,7 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     }
     w.gemm_part_bytes = gneed;
     w.gemm_parts = c.take<uint8_t>(gneed);
-    w.attn_part_bytes = nc_attn_partial_bytes(B, T, m->n_head);
+    w.attn_part_bytes = max_splits > 1 ? nc_attn_partial_bytes(B, T, m->n_head) / 16 * max_splits : 0;
     w.attn_parts = c.take<uint8_t>(w.attn_part_bytes);
     w.total = (c.off + 255) & ~(size_t)255;
     return w;
@@ -118,6 +127,12 @@ __global__ void gather_last_rows_kernel(const bf16_t* __restrict__ x, bf16_t* __
 }
 
 const NcPartialSrc NO_PARTIALS{nullptr, 0, 0, 0, nullptr, nullptr, 0, 0};
+
+int tap_copy(bf16_t* dst, const bf16_t* src, size_t elems, hipStream_t s) {
+    const hipError_t e = hipMemcpyAsync(dst, src, elems * sizeof(bf16_t), hipMemcpyDeviceToDevice, s);
+    if (e != hipSuccess) NC_FAIL(-2, "gpt_forward: tap copy failed: %s", hipGetErrorString(e));
+    return 0;
+}
 
 // One FP8 linear on `rows` rows of bf16 input whose amax sits in slot `site`.  Small M: the result is either
 // in `out` (single split: epilogue done in the GEMM) or described by *src (split partials for the consumer).
@@ -159,9 +174,10 @@ extern "C" size_t nc_gpt_workspace_bytes(const nc_model_desc* model, int B, int 
     return carve(model, B, T, nullptr).total;
 }
 
-extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, const int64_t* idx, int B, int T,
-                              float* logits_out, int last_only, void* workspace, size_t workspace_bytes, nc_stream_t stream) {
-    hipStream_t s = (hipStream_t)stream;
+// tap_x (or nullptr): bf16 [L+1, M, E], slot i = the residual stream as layer i reads it (after the lambda mix, gpt.py:500), slot L = the
+// final normalised rows (gpt.py:508).  tap_y (or nullptr): bf16 [L, M, H*128], the attention outputs before c_proj (gpt.py:113-124).
+static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, const int64_t* idx, int B, int T, float* logits_out,
+                            int last_only, void* workspace, size_t workspace_bytes, bf16_t* tap_x, bf16_t* tap_y, hipStream_t s) {
     NC_CHECK_ARG(m && kv && idx && logits_out && workspace, "gpt_forward: null pointer");
     NC_CHECK_ARG(B > 0 && T > 0, "gpt_forward: bad batch/time B=%d T=%d", B, T);
     NC_CHECK_ARG(m->n_embd == m->n_head * 128, "gpt_forward: head_dim must be 128 (n_embd=%d n_head=%d)", m->n_embd, m->n_head);
@@ -195,6 +211,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         // x += mlp_out(prev layer); [save backout]; x = rl*x + xl*x0; xn = norm(x)
         bf16_t* save = (i > 0 && (i - 1) == L / 2) ? w.xb : nullptr;
         TRY(mix(m->resid_lambdas + i, m->x0_lambdas + i, nullptr, nullptr, save, w.site(site)));
+        if (tap_x) TRY(tap_copy(tap_x + (size_t)i * M * E, w.x, (size_t)M * E, s));
         // q|k|v = FP8 linear(xn): one activation quantization, three weight scales
         NcGemmSegs qkv_segs{3, {H * 128, (H + Hkv) * 128, qkv_w, 0}};
         NcPartialSrc qsrc;
@@ -205,7 +222,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
         if (T == 1) {
             // decode: the attention workgroups finish their own q|k|v heads and append to the cache themselves
             const NcRopeSrc rope{qsrc.parts ? nullptr : w.qkv, qkv_w, qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin,
-                                 m->rope_len, m->padded_vocab};
+                                 m->rope_len, m->padded_vocab, nullptr, nullptr};
             TRY(nc_launch_attention_fused(rope, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, H, Hkv, kv->max_seq_len,
                                           w.attn_counters, w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s));
         } else {
@@ -218,6 +235,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
             TRY(nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
                                     w.attn_counters, w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s));
         }
+        if (tap_y) TRY(tap_copy(tap_y + (size_t)i * M * H * 128, w.y, (size_t)M * H * 128, s));
         TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E, &pending_parts));
         pending_add = pending_parts.parts ? nullptr : w.o;
         site++;
@@ -240,6 +258,7 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
             pending_parts = NO_PARTIALS;
         }
         TRY(mix(nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.site(site)));
+        if (tap_x) TRY(tap_copy(tap_x + (size_t)L * M * E, w.xn, (size_t)M * E, s));
     }
     // lm_head.  Its activation scale is tensorwise over all M rows (that is what the reference quantizes),
     // even when only the last position of every row is projected.
@@ -254,4 +273,15 @@ extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, c
     TRY(lin.run(head_in, head_rows, site, m->w_lm_head, m->inv_lm_head, one_seg(m->vocab_size), logits_out, 1, m->softcap, nullptr,
                 m->vocab_size, E, m->vocab_size, nullptr));
     return 0;
+}
+
+extern "C" int nc_gpt_forward(const nc_model_desc* m, const nc_cache_desc* kv, const int64_t* idx, int B, int T, float* logits_out,
+                              int last_only, void* workspace, size_t workspace_bytes, nc_stream_t stream) {
+    return gpt_forward_impl(m, kv, idx, B, T, logits_out, last_only, workspace, workspace_bytes, nullptr, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int nc_gpt_forward_tapped(const nc_model_desc* m, const nc_cache_desc* kv, const int64_t* idx, int B, int T, float* logits_out,
+                                     int last_only, void* workspace, size_t workspace_bytes, uint16_t* tap_x, uint16_t* tap_y,
+                                     nc_stream_t stream) {
+    return gpt_forward_impl(m, kv, idx, B, T, logits_out, last_only, workspace, workspace_bytes, tap_x, tap_y, (hipStream_t)stream);
 }

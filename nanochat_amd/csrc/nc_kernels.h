@@ -89,6 +89,11 @@ int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf
                                 int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                                 uint32_t* amax_ws, hipStream_t s);
 int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax);
+void nc_attention_plan(int B, int T, int Hkv, int window_left, int Tmax, int force_splits, int* splits_out, int* heads_per_wg_out);
+int nc_launch_attention_append(const bf16_t* q, const bf16_t* k_new, const bf16_t* v_new, bf16_t* k_cache, bf16_t* v_cache,
+                               const int32_t* cache_seqlens, int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax,
+                               uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
+                               hipStream_t s);
 struct NcRopeSrc;
 int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
                               bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* counters, void* partials, size_t partial_bytes,

@@ -25,6 +25,8 @@ struct NcRopeSrc {
     const bf16_t* sin_t;
     int rope_len;
     int vocab_rows;
+    const bf16_t* k_new;      // only for the attention kernel's plain-append form: finished new keys / values [tokens, Hkv, 128]
+    const bf16_t* v_new;
 };
 
 // The loads of one head, issued in one go so that their latency is paid once and a caller can put other loads behind them:

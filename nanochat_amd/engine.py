@@ -281,6 +281,10 @@ class Engine:
                 continue
             if run_ahead:
                 kv_decode.rewind(1, prev_before)
+            # forced tokens come from the tokenizer, not from the sampler: refuse what the embedding table does not hold
+            rows_in_table = getattr(self.model, "padded_vocab_size", None)
+            if rows_in_table is not None and not all(0 <= t < rows_in_table for t in column):
+                raise IndexError(f"token id out of range for an embedding table of {rows_in_table} rows: {column}")
             ids = torch.tensor(column, dtype=torch.long, device=device).unsqueeze(1)
             logits = self._last_logits(ids, kv_decode)
 

@@ -20,13 +20,10 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, cache_seqlens=N
                             window_size=(-1, -1)):
     assert cache_seqlens is not None, "cache_seqlens is required"
     assert causal, "only causal attention is implemented (nanochat always passes causal=True)"
-    B, T = q.shape[0], q.shape[1]
     if k is not None and v is not None:
-        # in-place insert at [pos_b, pos_b + T) per row (flash_attention.py:167-170)
-        rows = torch.arange(B, device=q.device)[:, None].expand(B, T)
-        cols = cache_seqlens.long()[:, None] + torch.arange(T, device=q.device)[None, :]
-        k_cache[rows, cols] = k.to(k_cache.dtype)
-        v_cache[rows, cols] = v.to(v_cache.dtype)
+        # in-place insert at [pos_b, pos_b + T) per row (flash_attention.py:167-170), done by the library
+        return ops.decode_attention_append(q, k.to(k_cache.dtype), v.to(v_cache.dtype), k_cache, v_cache, cache_seqlens,
+                                           window_left=window_size[0])
     return ops.decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=window_size[0])
 
 

@@ -14,6 +14,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib, ops
+from .common import COMPUTE_DTYPE
 from .fp8 import Float8Linear
 
 
@@ -108,6 +109,45 @@ class GPT(nn.Module):
         self._workspaces = {}
 
     # -------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def init_weights(self):
+        """The reference's initialisation, draw for draw (gpt.py:204-268): the random stream is consumed in the same
+        order by the same distributions, so a seeded CPU init gives the reference's weights bit for bit.
+
+        wte normal(0, 0.8); lm_head normal(0, 0.001); per block c_q, c_k, c_v uniform(+-s), attn.c_proj zero,
+        c_fc uniform(+-0.4 s), mlp.c_proj zero, with s = sqrt(3 / n_embd); resid / x0 lambdas on linear ramps;
+        smear_lambda 0, backout_lambda 0.2, smear_gate uniform(0, 0.02); value embeddings uniform(+-s); value-embedding
+        gates uniform(0, 0.02); finally the embedding tables go to the compute dtype (not for fp16)."""
+        cfg = self.config
+        nn.init.normal_(self.transformer.wte.weight, mean=0.0, std=0.8)
+        nn.init.normal_(self.lm_head.weight, mean=0.0, std=0.001)
+        s = 3 ** 0.5 * cfg.n_embd ** -0.5
+        for block in self.transformer.h:
+            nn.init.uniform_(block.attn.c_q.weight, -s, s)
+            nn.init.uniform_(block.attn.c_k.weight, -s, s)
+            nn.init.uniform_(block.attn.c_v.weight, -s, s)
+            nn.init.zeros_(block.attn.c_proj.weight)
+            nn.init.uniform_(block.mlp.c_fc.weight, -s * 0.4, s * 0.4)
+            nn.init.zeros_(block.mlp.c_proj.weight)
+        L = cfg.n_layer
+        for i in range(L):
+            self.resid_lambdas.data[i] = 1.15 - (0.10 * i / max(L - 1, 1))
+            self.x0_lambdas.data[i] = 0.20 - (0.15 * i / max(L - 1, 1))
+        nn.init.zeros_(self.smear_lambda)
+        nn.init.constant_(self.backout_lambda, 0.2)
+        nn.init.uniform_(self.smear_gate.weight, 0.0, 0.02)
+        for ve in self.value_embeds.values():
+            nn.init.uniform_(ve.weight, -s, s)
+        for block in self.transformer.h:
+            if block.attn.ve_gate is not None:
+                nn.init.uniform_(block.attn.ve_gate.weight, 0.0, 0.02)
+        # the rotary tables are rebuilt with the weight plan (rotary_tables), nothing to store here
+        if COMPUTE_DTYPE != torch.float16:
+            self.transformer.wte.to(dtype=COMPUTE_DTYPE)
+            for ve in self.value_embeds.values():
+                ve.to(dtype=COMPUTE_DTYPE)
+        self._plan = None
+
     def get_device(self):
         return self.transformer.wte.weight.device
 
@@ -247,13 +287,20 @@ class GPT(nn.Module):
 
     # -------------------------------------------------------------------------------------------
     @torch.no_grad()
-    def _run(self, idx, kv_cache, last_only):
+    def _run(self, idx, kv_cache, last_only, taps=None):
         from .engine import KVCache
         cfg = self.config
         if not idx.is_cuda:
             raise RuntimeError("GPT.forward runs on the GPU only; there is no CPU fallback")
         B, T = idx.shape
         assert idx.dtype == torch.long
+        if T > 1:
+            # a prompt: worth one read-back to refuse ids outside the embedding table, as the reference's nn.Embedding does
+            # (decode steps are fed by the sampler, or by the Engine's forced tokens, which it checks on the host; a direct
+            # one-token call with a bad id is not caught and reads row 0 of the table)
+            lo, hi = torch.aminmax(idx)
+            if int(lo) < 0 or int(hi) >= self.padded_vocab_size:
+                raise IndexError(f"token id out of range: [{int(lo)}, {int(hi)}] for an embedding table of {self.padded_vocab_size} rows")
         md = self._ensure_plan()
         if kv_cache is None:
             kv_cache = KVCache(B, cfg.n_kv_head, T, cfg.n_embd // cfg.n_head, cfg.n_layer, idx.device, torch.bfloat16)
@@ -278,8 +325,15 @@ class GPT(nn.Module):
         cd.prev_out = prev_out.data_ptr()
         cd.batch, cd.max_seq_len = B, kv_cache.max_seq_len
         ws_ptr, ws_bytes = self._workspace(md, B, T, idx.device)
-        rc = _lib.lib().nc_gpt_forward(C.byref(md), C.byref(cd), idx.data_ptr(), B, T, logits.data_ptr(), 1 if last_only else 0,
-                                       ws_ptr, ws_bytes, torch.cuda.current_stream().cuda_stream)
+        if taps is None:
+            rc = _lib.lib().nc_gpt_forward(C.byref(md), C.byref(cd), idx.data_ptr(), B, T, logits.data_ptr(), 1 if last_only else 0,
+                                           ws_ptr, ws_bytes, torch.cuda.current_stream().cuda_stream)
+        else:
+            taps["x"] = torch.empty(cfg.n_layer + 1, B, T, cfg.n_embd, dtype=torch.bfloat16, device=idx.device)
+            taps["y"] = torch.empty(cfg.n_layer, B, T, cfg.n_head, cfg.n_embd // cfg.n_head, dtype=torch.bfloat16, device=idx.device)
+            rc = _lib.lib().nc_gpt_forward_tapped(C.byref(md), C.byref(cd), idx.data_ptr(), B, T, logits.data_ptr(), 1 if last_only else 0,
+                                                  ws_ptr, ws_bytes, taps["x"].data_ptr(), taps["y"].data_ptr(),
+                                                  torch.cuda.current_stream().cuda_stream)
         _lib.check(rc)
         kv_cache.prev_embedding = prev_out
         kv_cache.advance(T)
@@ -294,6 +348,13 @@ class GPT(nn.Module):
     def forward_last(self, idx, kv_cache=None):
         """Logits of the last position only, [B,vocab]: what Engine.generate consumes."""
         return self._run(idx, kv_cache, last_only=True)
+
+    def forward_tapped(self, idx, kv_cache=None):
+        """(logits [B,T,vocab], taps) for layer-by-layer comparisons: taps["x"] [L+1,B,T,E] holds the residual stream as each
+        layer reads it (after the lambda mix, gpt.py:500) and, last, the final normalised rows (gpt.py:508); taps["y"]
+        [L,B,T,H,D] the attention outputs before c_proj."""
+        taps = {}
+        return self._run(idx, kv_cache, last_only=False, taps=taps), taps
 
     # -------------------------------------------------------------------------------------------
     @torch.no_grad()

@@ -287,13 +287,74 @@ def decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=-1, seqlens
     q = q.contiguous()
     out = torch.empty_like(q)
     lib = _lib.lib()
-    ws_bytes = lib.nc_attention_workspace_bytes(B, T, H, Tmax)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)      # the call clears its own counters
+    ws, ws_bytes = _attention_workspace(B, T, H, Tmax, q.device)
     rc = lib.nc_decode_attention(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cache_seqlens), int(window_left), _ptr(out), B, T, H,
                                  Hkv, Tmax, 1 if seqlens_include_new else 0, _ptr(ws), ws_bytes, C.c_void_p(0), splits,
                                  _stream())
     _lib.check(rc)
     return out
+
+
+def _attention_workspace(B, T, H, Tmax, device):
+    lib = _lib.lib()
+    ws_bytes = lib.nc_attention_workspace_bytes(B, T, H, Tmax)
+    return torch.empty(ws_bytes, dtype=torch.uint8, device=device), ws_bytes      # the call clears its own counters
+
+
+def decode_attention_append(q, k_new, v_new, k_cache, v_cache, cache_seqlens, window_left=-1, splits=0):
+    """flash_attn_with_kvcache(q, k_cache, v_cache, k=k_new, v=v_new, cache_seqlens=...) (nanochat/flash_attention.py:139-185):
+    the new keys and values go into the caches at cache_seqlens[b].. (in place), then q [B,T,H,128] attends."""
+    _need_cuda(q, k_new, v_new, k_cache, v_cache, cache_seqlens)
+    for t in (q, k_new, v_new, k_cache, v_cache):
+        if t.dtype != torch.bfloat16:
+            raise ValueError("decode_attention_append: bf16 only")
+    if cache_seqlens.dtype != torch.int32:
+        raise ValueError("decode_attention_append: cache_seqlens must be int32")
+    B, T, H, D = q.shape
+    Tmax, Hkv = k_cache.shape[1], k_cache.shape[2]
+    if D != 128 or k_cache.shape[-1] != 128 or tuple(k_new.shape) != (B, T, Hkv, 128) or tuple(v_new.shape) != (B, T, Hkv, 128):
+        raise ValueError("decode_attention_append: q [B,T,H,128], k/v [B,T,Hkv,128], caches [B,Tmax,Hkv,128] expected")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("decode_attention_append: caches must be contiguous (B,Tmax,Hkv,128)")
+    q, k_new, v_new = q.contiguous(), k_new.contiguous(), v_new.contiguous()
+    out = torch.empty_like(q)
+    ws, ws_bytes = _attention_workspace(B, T, H, Tmax, q.device)
+    rc = _lib.lib().nc_decode_attention_append(_ptr(q), _ptr(k_new), _ptr(v_new), _ptr(k_cache), _ptr(v_cache), _ptr(cache_seqlens),
+                                               int(window_left), _ptr(out), B, T, H, Hkv, Tmax, _ptr(ws), ws_bytes, C.c_void_p(0),
+                                               splits, _stream())
+    _lib.check(rc)
+    return out
+
+
+def qkv_rope_append_attention(qkv, xn, idx, ve_table, ve_gate_w, cos, sin, cache_seqlens, k_cache, v_cache, n_head, n_kv_head,
+                              window_left=-1, splits=0):
+    """Decode (one new token per row): qkv_rope_append and decode_attention in one launch (nanochat/gpt.py:89-120).
+    qkv [B,1,(H+2Hkv)*128] bf16.  Returns the attention output [B,1,H,128]; the caches get the new key and value."""
+    _need_cuda(qkv, k_cache, v_cache, cache_seqlens)
+    B = qkv.shape[0]
+    if qkv.numel() != B * (n_head + 2 * n_kv_head) * 128:
+        raise ValueError("qkv_rope_append_attention: one new token per row expected")
+    qkv = qkv.contiguous()
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    Tmax = k_cache.shape[1]
+    out = torch.empty(B, 1, n_head, 128, dtype=torch.bfloat16, device=qkv.device)
+    vocab_rows = ve_table.shape[0] if ve_table is not None else 0
+    xn_c = xn.contiguous() if xn is not None else None
+    ws, ws_bytes = _attention_workspace(B, 1, n_head, Tmax, qkv.device)
+    rc = _lib.lib().nc_qkv_rope_append_attention(
+        _ptr(qkv), qkv.shape[-1], _ptr(xn_c), xn_c.shape[-1] if xn_c is not None else 0, _ptr(idx.contiguous() if idx is not None else None),
+        _ptr(ve_table), _ptr(ve_gate_w.float().contiguous() if ve_gate_w is not None else None), _ptr(cos), _ptr(sin), cos.shape[0],
+        _ptr(cache_seqlens), _ptr(k_cache), _ptr(v_cache), int(window_left), _ptr(out), B, n_head, n_kv_head, Tmax, vocab_rows,
+        _ptr(ws), ws_bytes, C.c_void_p(0), splits, _stream())
+    _lib.check(rc)
+    return out
+
+
+def decode_attention_plan(B, T, n_kv_head, window_left, Tmax, splits=0):
+    """(key splits, kv heads per workgroup) a decode-attention launch of this shape uses."""
+    s, h = C.c_int(0), C.c_int(0)
+    _lib.check(_lib.lib().nc_decode_attention_plan(B, T, n_kv_head, int(window_left), Tmax, splits, C.byref(s), C.byref(h)))
+    return s.value, h.value
 
 
 def kv_cache_prefill(dst, src, n_tokens):

@@ -224,6 +224,7 @@ def forward(rt: Runtime, idx, kv_cache=None):
     for i in range(L):
         pre = f"transformer.h.{i}."
         x = p["resid_lambdas"][i] * x + p["x0_lambdas"][i] * x0
+        rt.tap(f"xmix{i}", x)
         ve_name = f"value_embeds.{i}.weight"
         ve = F.embedding(idx, p[ve_name]).to(x.dtype) if ve_name in p else None
         # --- attention

@@ -5,6 +5,7 @@ Run in the authoring container only (the reference tree is not shipped anywhere)
     python tests/golden/make_golden.py quantize
     python tests/golden/make_golden.py gpt_fp32
     NANOCHAT_DTYPE=bfloat16 python tests/golden/make_golden.py gpt_bf16_fp8
+    NANOCHAT_DTYPE=bfloat16 python tests/golden/make_golden.py cost
 
 What is imported from the reference: ``nanochat.fp8`` (``_to_fp8``, ``Float8Linear``,
 ``convert_to_float8_training``), ``nanochat.gpt`` (``GPT``, ``GPTConfig``) and,
@@ -168,6 +169,52 @@ def make_gpt(tag, fp8):
     print("wrote", tag)
 
 
+# ----------------------------------------------------------------------------------------
+COST_CONFIGS = {
+    "d4": dict(sequence_len=2048, vocab_size=32768, n_layer=4, n_head=2, n_kv_head=2, n_embd=256),
+    "d20": dict(sequence_len=2048, vocab_size=32768, n_layer=20, n_head=10, n_kv_head=10, n_embd=1280),
+    "d26": dict(sequence_len=2048, vocab_size=32768, n_layer=26, n_head=13, n_kv_head=13, n_embd=1664),
+    "d26_L": dict(sequence_len=2048, vocab_size=32768, n_layer=26, n_head=13, n_kv_head=13, n_embd=1664, window_pattern="L"),
+    "d32_gqa": dict(sequence_len=2048, vocab_size=32768, n_layer=32, n_head=16, n_kv_head=4, n_embd=2048),
+    "odd_vocab": dict(sequence_len=1024, vocab_size=50257, n_layer=5, n_head=3, n_kv_head=1, n_embd=384, window_pattern="SL"),
+}
+COST_CONTEXTS = (1, 512, 513, 1920, 2048)
+COST_PROMPTS = (1, 400, 512, 1792, 2048)
+
+
+def make_cost():
+    """The reference's own cost accounting (gpt.py:341-388, scripts/infer_bench.py:51-53,130-138) on models that
+    exist on the meta device only (no weights are materialised), before any FP8 conversion."""
+    from nanochat.common import COMPUTE_DTYPE
+    from nanochat.gpt import GPT, GPTConfig
+    assert COMPUTE_DTYPE == torch.bfloat16
+    out = {"compute_dtype": str(COMPUTE_DTYPE), "configs": {}}
+    for name, kw in COST_CONFIGS.items():
+        with torch.device("meta"):
+            model = GPT(GPTConfig(**kw))
+        # the dtypes a loaded checkpoint has in the reference: everything as built (fp32), embeddings in the compute dtype
+        # (gpt.py:264-267); element sizes follow from that without materialising a weight
+        emb = {id(model.transformer.wte.weight)} | {id(ve.weight) for ve in model.value_embeds.values()}
+        w_bytes = sum(p.numel() * (COMPUTE_DTYPE.itemsize if id(p) in emb else p.element_size()) for p in model.parameters())
+        rec = {
+            "config": kw,
+            "num_params": sum(p.numel() for p in model.parameters()),
+            "num_matmul_params": model.num_matmul_params(),
+            "weight_bytes_embeddings_in_compute_dtype": w_bytes,
+            "kv_bytes_per_token": model.kv_bytes_per_token(),
+            "window_sizes": [list(w) for w in model.window_sizes],
+            "value_embed_layers": sorted(int(k) for k in model.value_embeds.keys()),
+            "kv_read_bytes": {str(c): model.kv_read_bytes(c) for c in COST_CONTEXTS},
+            "estimate_decode_flops": {str(c): model.estimate_decode_flops(c) for c in COST_CONTEXTS},
+            "estimate_prefill_flops": {str(n): model.estimate_prefill_flops(n) for n in COST_PROMPTS},
+        }
+        out["configs"][name] = rec
+        print(name, rec["num_params"], rec["num_matmul_params"], rec["kv_bytes_per_token"])
+    with open(os.path.join(HERE, "cost_accounting.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print("wrote cost_accounting.json")
+
+
 if __name__ == "__main__":
     mode = sys.argv[1]
     if mode == "quantize":
@@ -178,5 +225,8 @@ if __name__ == "__main__":
     elif mode == "gpt_bf16_fp8":
         assert os.environ.get("NANOCHAT_DTYPE") == "bfloat16"
         make_gpt("gpt_d4_bf16_fp8", fp8=True)
+    elif mode == "cost":
+        assert os.environ.get("NANOCHAT_DTYPE") == "bfloat16"
+        make_cost()
     else:
         raise SystemExit(f"unknown mode {mode}")

@@ -58,7 +58,8 @@ def build_pair(cfg_kwargs, seed, trained_like=True):
 D4 = dict(sequence_len=2048, vocab_size=32768, n_layer=4, n_head=2, n_kv_head=2, n_embd=256)
 SMALL_GQA = dict(sequence_len=256, vocab_size=1024, n_layer=5, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
 SMALL_MHA = dict(sequence_len=512, vocab_size=2048, n_layer=6, n_head=3, n_kv_head=3, n_embd=384, window_pattern="SSSL")
-# batch x kv heads >= 512: attention runs one workgroup per (row, kv head) and finishes q|k|v (rotary, append) itself
+# batch x kv heads = 512: attention runs one workgroup per (row, kv head), unsplit, and finishes q|k|v (rotary, append) itself;
+# the variant with two kv heads per workgroup needs batch x ceil(kv heads / 2) >= 384 and is covered in test_gpu_variants.py
 WIDE_GQA = dict(sequence_len=128, vocab_size=1024, n_layer=3, n_head=8, n_kv_head=4, n_embd=1024, window_pattern="SL")
 WIDE_MHA = dict(sequence_len=128, vocab_size=1024, n_layer=2, n_head=4, n_kv_head=4, n_embd=512, window_pattern="SL")
 
@@ -160,10 +161,10 @@ def test_prefill_logits_match_oracle(d4_pair):
     assert torch.allclose(cache.prev_embedding.cpu().float(), ref_cache.prev_embedding.float(), atol=2e-2)
 
 
-def test_greedy_decode_64_tokens_through_engine(d4_pair, d4_repo_pair):
-    """Engine.generate on the GPU, greedy, 64 tokens.  Repo init: ids equal to the oracle's (margin aware).
-    Trained-like: the first divergence, if any, must sit where the oracle's top-2 margin is inside its own
-    sensitivity floor."""
+def test_greedy_decode_64_tokens_through_engine(d4_repo_pair):
+    """Engine.generate on the GPU, greedy, 64 tokens, repository init: ids equal to the oracle's; a difference is accepted only
+    where the oracle's own top-2 margin is within twice the stated logit tolerance (bf16 logits tie often at this init).
+    The trained-like counterpart, with a bound derived from the oracle's own sensitivity, is in test_gpu_variants.py."""
     from nanochat_amd.engine import Engine
     from test_engine_host import ByteTokenizer
 
@@ -176,22 +177,23 @@ def test_greedy_decode_64_tokens_through_engine(d4_pair, d4_repo_pair):
             return 32765
     g = torch.Generator().manual_seed(0)
     prompt = torch.randint(0, 32768, (32,), generator=g).tolist()
-    for name, (rt, model), slack in (("repo", d4_repo_pair, 2e-3), ("trained_like", d4_pair, 0.3)):
-        say(f"d4 {name}: greedy decode 64 tokens via Engine.generate")
-        want_cols, want_logits = decode_ref.generate(rt, prompt, 1, 64, temperature=0.0, collect_logits=True)
-        want_ids = [c[0] for c in want_cols]
-        got_ids = []
-        for column, masks in Engine(model, Tok()).generate(prompt, num_samples=1, max_tokens=64, temperature=0.0):
-            got_ids.append(column[0])
-            if column[0] in (32764, 32765):
-                break
-        first_div = next((i for i, (a, b) in enumerate(zip(got_ids, want_ids)) if a != b), len(got_ids))
-        print(f"{name}: greedy ids identical for the first {first_div} of {len(got_ids)} tokens")
-        if first_div < min(len(got_ids), len(want_ids)):
-            top2 = torch.topk(want_logits[first_div][0], 2).values
-            gap = (top2[0] - top2[1]).item()
-            assert gap <= slack, f"{name}: token {first_div} differs although the oracle margin is {gap}"
-        assert first_div >= 1
+    rt, model = d4_repo_pair
+    say("d4 repo: greedy decode 64 tokens via Engine.generate")
+    want_cols, want_logits = decode_ref.generate(rt, prompt, 1, 64, temperature=0.0, collect_logits=True)
+    want_ids = [c[0] for c in want_cols]
+    got_ids = []
+    for column, masks in Engine(model, Tok()).generate(prompt, num_samples=1, max_tokens=64, temperature=0.0):
+        got_ids.append(column[0])
+        if column[0] in (32764, 32765):
+            break
+    first_div = next((i for i, (a, b) in enumerate(zip(got_ids, want_ids)) if a != b), len(got_ids))
+    print(f"repo: greedy ids identical for the first {first_div} of {len(got_ids)} tokens")
+    if first_div < min(len(got_ids), len(want_ids)):
+        top2 = torch.topk(want_logits[first_div][0], 2).values
+        gap = (top2[0] - top2[1]).item()
+        assert gap <= 2 * LOGIT_TOL, f"token {first_div} differs although the oracle margin is {gap}"
+    else:
+        assert got_ids == want_ids[:len(got_ids)]
 
 
 def test_decode_logits_stepwise_teacher_forced(d4_pair):
@@ -245,23 +247,32 @@ def test_reference_written_goldens(d4_pair, d4_repo_pair):
         prompt = torch.tensor([gold["prompt"]])
         cache = KVCache(1, 2, 32 + 64, 128, 4, DEV, torch.bfloat16)
         logits = model.forward_last(prompt.to(DEV), kv_cache=cache).cpu()
-        worst, num, den = 0.0, 0.0, 0.0
+        # the floor: the oracle's fp32-definition variant (a form the reference treats as equal to its SDPA path, which wrote the
+        # goldens) on the same tokens, measured on the same samples of every logits row
+        rt_def = gpt_ref.Runtime(rt.cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+        c_def = decode_ref.new_cache(rt.cfg, 1, 32 + 64, torch.bfloat16)
+        other = gpt_ref.forward(rt_def, prompt, c_def)[:, -1]
+        worst, num, den, f_worst, f_num = 0.0, 0.0, 0.0, 0.0, 0.0
         for t in range(40):
             dig = run["steps"][t]["digest"]
-            row = logits[0]
-            for got, want in ((row[:32], dig["head"]), (row[::1021], dig["strided"]), (row[dig["top_idx"]], dig["top_val"])):
+            row, orow = logits[0], other[0]
+            for pick, want in ((slice(0, 32), dig["head"]), (slice(None, None, 1021), dig["strided"]), (dig["top_idx"], dig["top_val"])):
                 want = torch.tensor(want)
-                worst = max(worst, (got - want).abs().max().item())
-                num += (got - want).pow(2).sum().item()
+                worst = max(worst, (row[pick] - want).abs().max().item())
+                num += (row[pick] - want).pow(2).sum().item()
                 den += want.pow(2).sum().item()
+                f_worst = max(f_worst, (orow[pick] - want).abs().max().item())
+                f_num += (orow[pick] - want).pow(2).sum().item()
             nxt = torch.tensor([[run["greedy_ids"][t]]])          # teacher forcing with the reference's ids
             logits = model.forward_last(nxt.to(DEV), kv_cache=cache).cpu()
-        rel = (num / den) ** 0.5
-        print(f"{name} vs reference goldens: max |dlogit| = {worst:.5f}, rel_l2 = {rel:.4f}")
+            other = gpt_ref.forward(rt_def, nxt, c_def)[:, -1]
+        rel, f_rel = (num / den) ** 0.5, (f_num / den) ** 0.5
+        print(f"{name} vs reference goldens: max |dlogit| = {worst:.5f}, rel_l2 = {rel:.4f}; the oracle's other variant: "
+              f"max {f_worst:.5f}, rel_l2 {f_rel:.4f}")
         if name == "repo":
             assert worst <= LOGIT_TOL
         else:
-            assert rel <= 0.08 and worst <= 0.3       # 1.5x the oracle's own floor at this logit scale (see module doc)
+            assert rel <= 1.5 * f_rel + 1e-3 and worst <= 1.5 * f_worst + LOGIT_TOL
     if checked == 0:
         pytest.skip("golden weights not reproducible on this host")
 
@@ -280,11 +291,24 @@ def test_cached_decode_equals_cache_free_forward(d4_pair):
         rows.append(model(seq[:, t:t + 1], kv_cache=cache)[:, -1])
     stepped = torch.stack(rows, dim=1)                   # logits at positions 15..23
     # Not bit-equal: the activation scale of an FP8 linear is tensorwise over the rows of the call, so a
-    # 24-token call and a 1-token call quantize differently.  The fp8 noise bounds the gap.
+    # 24-token call and a 1-token call quantize differently.  The oracle does the same computation both ways; the gap it
+    # shows between its two ways is the yardstick, and each way is checked against the oracle's.
+    seq_c = seq.cpu()
+    full_o = gpt_ref.forward(rt, seq_c, None)
+    c = decode_ref.new_cache(rt.cfg, 2, 32, torch.bfloat16)
+    rows_o = [gpt_ref.forward(rt, seq_c[:, :16], c)[:, -1]]
+    for t in range(16, 24):
+        rows_o.append(gpt_ref.forward(rt, seq_c[:, t:t + 1], c)[:, -1])
+    stepped_o = torch.stack(rows_o, dim=1)
+    gap_o = (stepped_o - full_o[:, 15:]).abs().max().item()
     diff = (stepped - full[:, 15:]).abs().max().item()
-    print(f"cached vs cache-free max |dlogit| = {diff:.4f}")
-    assert diff < 0.5
-    assert (stepped.argmax(-1) == full[:, 15:].argmax(-1)).float().mean().item() > 0.5
+    print(f"cached vs cache-free max |dlogit| = {diff:.4f}; the oracle's own gap {gap_o:.4f}")
+    assert diff <= 1.5 * gap_o + LOGIT_TOL
+    agree_o = (stepped_o.argmax(-1) == full_o[:, 15:].argmax(-1)).float().mean().item()
+    assert (stepped.argmax(-1) == full[:, 15:].argmax(-1)).float().mean().item() >= agree_o - 0.25
+    # (the oracle's two attention forms only differ when there is a cache: a prefill into an empty cache is the same computation)
+    floor_rel, floor_max, a, b = oracle_floor(rt, lambda r: gpt_ref.forward(r, seq_c, decode_ref.new_cache(r.cfg, 2, 24, torch.bfloat16)))
+    assert_within_floor(full.cpu(), a, b, floor_rel, floor_max, "cache-free forward")
 
 
 @pytest.mark.parametrize("cfg_kwargs,B", [(SMALL_MHA, 3), (SMALL_GQA, 70)])

@@ -1,0 +1,475 @@
+"""GPU parity of the decode-attention kernel variants and of the configurations the headline numbers are quoted on.
+
+  * every form of the decode attention (keys already appended; new key/value handed over and appended by the kernel;
+    raw q|k|v finished by the kernel: rotary, QK-norm, value embedding, append) at shapes that select the variant with two
+    kv heads per workgroup -- the one the d26 / batch-64 step runs -- against the CPU oracle, with the selected variant
+    asserted through nc_decode_attention_plan;
+  * small trained-like models whose decode step takes that variant (odd and even kv-head counts, MHA and GQA), logits and
+    layer 0's appended cache rows against the oracle;
+  * one-layer models (no amplification through re-quantization) and layer-by-layer taps of a deeper model;
+  * the d20 shape of BASELINE config 3 through Engine.generate at T = 1.0 / top_k = 50, and the d32-GQA width of config 5
+    with ragged prompts and T = 0.8 / top_k = 50.
+"""
+import sys
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import decode_ref, gpt_ref
+from oracle.attention_ref import attention_with_kvcache
+from test_gpu_gpt import DEV, LOGIT_TOL, assert_within_floor, build_pair, oracle_floor, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(f"[gpu-case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from nanochat_amd import ops as _ops
+    return _ops
+
+
+def ulp_stats(got, want):
+    """(fraction of elements that differ, largest difference in bf16 ulps) of two bf16 tensors."""
+    gi, wi = got.view(torch.int16).int(), want.view(torch.int16).int()
+    # monotone integer image of the bf16 line
+    gi = torch.where(gi < 0, -(gi & 0x7fff), gi)
+    wi = torch.where(wi < 0, -(wi & 0x7fff), wi)
+    d = (gi - wi).abs()
+    return (d > 0).float().mean().item(), int(d.max().item())
+
+
+# ------------------------------------------------------------------------------------------------ kernel level
+# (B, H, Hkv, Tmax, window): B * ceil(Hkv / 2) >= 384 selects two kv heads per workgroup and one split
+HP2_SHAPES = [
+    (128, 6, 6, 80, -1),        # three full pairs
+    (96, 7, 7, 70, 16),         # odd head count: the last pair has an idle half
+    (128, 5, 5, 40, -1),        # odd, the 13-heads-in-7-pairs case in small
+    (128, 12, 6, 90, 32),       # two query heads per kv head
+    (100, 32, 8, 50, -1),       # four
+    (192, 32, 4, 33, 8),        # eight
+]
+
+
+def ragged_lengths(B, Tmax, g):
+    seq = torch.randint(0, Tmax, (B,), generator=g, dtype=torch.int32)
+    seq[0], seq[1], seq[-1] = 0, 1, Tmax - 1                       # an empty row, a one-key row, a row that fills the cache
+    return seq
+
+
+def rope_oracle(qkv, xn, idx, ve_table, gate_w, cos, sin, seq, H, Hkv):
+    """The eager op sequence of CausalSelfAttention.forward from the q|k|v linears' outputs to q, k, v (gpt.py:89-104)."""
+    B, T = qkv.shape[0], qkv.shape[1]
+    q = qkv[..., :H * 128].view(B, T, H, 128)
+    k = qkv[..., H * 128:(H + Hkv) * 128].view(B, T, Hkv, 128)
+    v = qkv[..., (H + Hkv) * 128:].view(B, T, Hkv, 128)
+    if ve_table is not None:
+        ve = F.embedding(idx, ve_table).view(B, T, Hkv, 128)
+        gt = 3 * torch.sigmoid(gpt_ref.small_linear(xn[..., :12], gate_w))
+        v = v + gt.unsqueeze(-1) * ve
+    posv = seq.long()[:, None] + torch.arange(T)[None, :]
+    c, s = cos[posv][:, :, None, :], sin[posv][:, :, None, :]
+    q, k = gpt_ref.rotate(q, c, s), gpt_ref.rotate(k, c, s)
+    return gpt_ref.rms_norm(q) * 1.2, gpt_ref.rms_norm(k) * 1.2, v
+
+
+@pytest.mark.parametrize("B,H,Hkv,Tmax,window", HP2_SHAPES)
+def test_decode_attention_two_heads_per_workgroup_all_forms(ops, B, H, Hkv, Tmax, window):
+    say(f"decode attention, head pairs: B={B} H={H} Hkv={Hkv} Tmax={Tmax} window={window}")
+    assert ops.decode_attention_plan(B, 1, Hkv, window, Tmax) == (1, 2), "this shape was meant to select two kv heads per workgroup"
+    g = torch.Generator().manual_seed(B + H + Tmax)
+    kc = torch.randn(B, Tmax, Hkv, 128, generator=g).bfloat16()
+    vc = torch.randn(B, Tmax, Hkv, 128, generator=g).bfloat16()
+    q = (torch.randn(B, 1, H, 128, generator=g) * 1.5).bfloat16()
+    k_new = torch.randn(B, 1, Hkv, 128, generator=g).bfloat16()
+    v_new = torch.randn(B, 1, Hkv, 128, generator=g).bfloat16()
+    seq = ragged_lengths(B, Tmax, g)
+    # (a) the new key and value are handed over: flash_attn_with_kvcache(q, k_cache, v_cache, k=, v=)
+    kc_want, vc_want = kc.clone(), vc.clone()
+    want = attention_with_kvcache(q, kc_want, vc_want, k_new, v_new, seq, (window, 0))
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    # slots that hold nothing yet must never reach a result
+    for b in range(B):
+        kd[b, seq[b] + 1:] = float("nan")
+        vd[b, seq[b] + 1:] = float("nan")
+    kd_nan, vd_nan = kd.clone(), vd.clone()
+    got = ops.decode_attention_append(q.to(DEV), k_new.to(DEV), v_new.to(DEV), kd, vd, seq.to(DEV), window_left=window).cpu()
+    assert torch.isfinite(got.float()).all()
+    assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2), (got.float() - want.float()).abs().max().item()
+    for b in range(0, B, 7):                                      # the append touched slot seq[b] only, with the exact bytes
+        assert torch.equal(kd[b, seq[b]].cpu(), k_new[b, 0]) and torch.equal(vd[b, seq[b]].cpu(), v_new[b, 0])
+        assert torch.equal(kd[b, :seq[b]].cpu(), kc[b, :seq[b]])
+        assert torch.equal(kd[b, seq[b] + 1:].view(torch.int16), kd_nan[b, seq[b] + 1:].view(torch.int16))
+    # (b) the same launch shape with the keys already in the cache (the kernel reads its own token from the cache)
+    got_b = ops.decode_attention(q.to(DEV), kd, vd, seq.to(DEV), window_left=window).cpu()
+    assert torch.allclose(got_b.float(), want.float(), atol=1e-2, rtol=1e-2)
+    # (c) raw q|k|v rows: rotary, QK-norm, gain, value-embedding gate and the append happen in the attention kernel
+    V = 300
+    qkv = torch.randn(B, 1, (H + 2 * Hkv) * 128, generator=g).bfloat16()
+    xn = torch.randn(B, 1, H * 128, generator=g).bfloat16()
+    idx = torch.randint(0, V, (B, 1), generator=g)
+    ve_table = (torch.randn(V, Hkv * 128, generator=g) * 0.5).bfloat16()
+    gate_w = torch.rand(Hkv, 12, generator=g) - 0.5
+    cos, sin = gpt_ref.rotary_tables(Tmax + 8, 128, torch.bfloat16)
+    for with_ve in (True, False):
+        q2, k2, v2 = rope_oracle(qkv, xn, idx, ve_table if with_ve else None, gate_w, cos, sin, seq, H, Hkv)
+        kc2, vc2 = kc.clone(), vc.clone()
+        want2 = attention_with_kvcache(q2, kc2, vc2, k2, v2, seq, (window, 0))
+        kd2, vd2 = kd_nan.clone(), vd_nan.clone()
+        got2 = ops.qkv_rope_append_attention(qkv.to(DEV), xn.to(DEV), idx.to(DEV), ve_table.to(DEV) if with_ve else None,
+                                             gate_w.to(DEV) if with_ve else None, cos.to(DEV), sin.to(DEV), seq.to(DEV), kd2, vd2, H, Hkv,
+                                             window_left=window).cpu()
+        assert torch.isfinite(got2.float()).all()
+        assert torch.allclose(got2.float(), want2.float(), atol=1e-2, rtol=1e-2), (got2.float() - want2.float()).abs().max().item()
+        rows = torch.arange(B)
+        frac_k, ulp_k = ulp_stats(kd2[rows, seq.long()].cpu(), k2[:, 0])
+        frac_v, ulp_v = ulp_stats(vd2[rows, seq.long()].cpu(), v2[:, 0])
+        assert ulp_k <= 1 and ulp_v <= 1 and frac_k < 0.01 and frac_v < 0.01, (frac_k, ulp_k, frac_v, ulp_v)
+
+
+@pytest.mark.parametrize("splits", [0, 1, 2, 4, 16])
+@pytest.mark.parametrize("H,Hkv", [(4, 2), (13, 13)])
+def test_decode_attention_in_kernel_append_with_key_splits(ops, splits, H, Hkv):
+    """Few rows: the keys of a head are split over workgroups; split 0 alone appends and counts the row's own key."""
+    say(f"decode attention with in-kernel append, splits={splits} H={H} Hkv={Hkv}")
+    B, Tmax, window = 3, 300, -1
+    g = torch.Generator().manual_seed(splits + H)
+    kc = torch.randn(B, Tmax, Hkv, 128, generator=g).bfloat16()
+    vc = torch.randn(B, Tmax, Hkv, 128, generator=g).bfloat16()
+    q = (torch.randn(B, 1, H, 128, generator=g) * 1.5).bfloat16()
+    k_new = torch.randn(B, 1, Hkv, 128, generator=g).bfloat16()
+    v_new = torch.randn(B, 1, Hkv, 128, generator=g).bfloat16()
+    seq = torch.tensor([0, 151, 299], dtype=torch.int32)
+    kc_want, vc_want = kc.clone(), vc.clone()
+    want = attention_with_kvcache(q, kc_want, vc_want, k_new, v_new, seq, (window, 0))
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    got = ops.decode_attention_append(q.to(DEV), k_new.to(DEV), v_new.to(DEV), kd, vd, seq.to(DEV), window_left=window, splits=splits).cpu()
+    assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2)
+    assert torch.equal(kd.cpu(), kc_want) and torch.equal(vd.cpu(), vc_want)
+    # several new tokens per row through the same entry (a copy kernel appends, then the ordinary kernels attend)
+    T = 5 if splits else 20
+    qT = (torch.randn(B, T, H, 128, generator=g) * 1.5).bfloat16()
+    kT = torch.randn(B, T, Hkv, 128, generator=g).bfloat16()
+    vT = torch.randn(B, T, Hkv, 128, generator=g).bfloat16()
+    seqT = torch.tensor([0, 100, Tmax - T], dtype=torch.int32)
+    kc_w, vc_w = kc.clone(), vc.clone()
+    wantT = attention_with_kvcache(qT, kc_w, vc_w, kT, vT, seqT, (64, 0))
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    gotT = ops.decode_attention_append(qT.to(DEV), kT.to(DEV), vT.to(DEV), kd, vd, seqT.to(DEV), window_left=64, splits=splits).cpu()
+    assert torch.allclose(gotT.float(), wantT.float(), atol=1e-2, rtol=1e-2)
+    assert torch.equal(kd.cpu(), kc_w) and torch.equal(vd.cpu(), vc_w)
+
+
+# ------------------------------------------------------------------------------------------------ model level
+# decode steps of these run attn_partial_kernel<G, fused, two heads>: batch x ceil(kv heads / 2) >= 384
+PAIR_MHA_ODD = dict(sequence_len=128, vocab_size=1024, n_layer=2, n_head=5, n_kv_head=5, n_embd=640, window_pattern="SL")
+PAIR_GQA = dict(sequence_len=128, vocab_size=1024, n_layer=2, n_head=12, n_kv_head=6, n_embd=1536, window_pattern="SL")
+PAIR_MHA_7 = dict(sequence_len=256, vocab_size=1024, n_layer=3, n_head=7, n_kv_head=7, n_embd=896, window_pattern="SSL")
+
+
+@pytest.mark.parametrize("cfg_kwargs,B,P,steps", [(PAIR_MHA_ODD, 128, 9, 6), (PAIR_GQA, 128, 40, 6), (PAIR_MHA_7, 96, 70, 5)])
+def test_models_whose_decode_takes_the_head_pair_kernel(ops, cfg_kwargs, B, P, steps):
+    say(f"head-pair decode in a model {cfg_kwargs['n_embd']}/{cfg_kwargs['n_head']}q{cfg_kwargs['n_kv_head']}kv B={B}")
+    rt, model = build_pair(cfg_kwargs, seed=13)
+    from nanochat_amd.engine import KVCache
+    cfg = rt.cfg
+    for w, _ in model.window_sizes:
+        assert ops.decode_attention_plan(B, 1, cfg.n_kv_head, w, P + steps) == (1, 2)
+    g = torch.Generator().manual_seed(14)
+    prompt = torch.randint(0, cfg.vocab_size, (1, P), generator=g)
+    rt_def = gpt_ref.Runtime(cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+    caches = {}
+    for name, r in (("sdpa", rt), ("def", rt_def)):
+        pre = decode_ref.new_cache(cfg, 1, P, torch.bfloat16)
+        first = gpt_ref.forward(r, prompt, pre)[:, -1].expand(B, -1)
+        dec = decode_ref.new_cache(cfg, B, P + steps, torch.bfloat16)
+        dec.prefill(pre)
+        caches[name] = (dec, [first])
+    pre = KVCache(1, cfg.n_kv_head, P, 128, cfg.n_layer, DEV, torch.bfloat16)
+    G = [model.forward_last(prompt.to(DEV), kv_cache=pre).expand(B, -1).cpu()]
+    dec = KVCache(B, cfg.n_kv_head, P + steps, 128, cfg.n_layer, DEV, torch.bfloat16)
+    dec.prefill(pre)
+    dec.k_cache[:, :, P:] = float("nan")
+    dec.v_cache[:, :, P:] = float("nan")
+    for s in range(steps):
+        nxt = torch.randint(0, cfg.vocab_size, (B, 1), generator=g)       # distinct tokens per row
+        for name, r in (("sdpa", rt), ("def", rt_def)):
+            caches[name][1].append(gpt_ref.forward(r, nxt, caches[name][0])[:, -1])
+        G.append(model.forward_last(nxt.to(DEV), kv_cache=dec).cpu())
+    S, Dd, G = torch.stack(caches["sdpa"][1]), torch.stack(caches["def"][1]), torch.stack(G)
+    assert torch.isfinite(G).all()
+    assert_within_floor(G, S, Dd, rel_l2(Dd, S), (S - Dd).abs().max().item(), "head-pair decode")
+    # layer 0 reads the embedding rows, identical on both sides: the rows it appended during decode agree to the last bf16 bit or so
+    ref = caches["sdpa"][0]
+    for got_c, want_c, what in ((dec.k_cache, ref.k_cache, "k"), (dec.v_cache, ref.v_cache, "v")):
+        frac, ulps = ulp_stats(got_c[0, :, P:P + steps].cpu(), want_c[0, :, P:P + steps])
+        print(f"layer-0 appended {what} rows: {frac:.4%} of the elements differ, by at most {ulps} bf16 ulp")
+        assert ulps <= 2 and frac < 0.02, (what, frac, ulps)
+
+
+ONE_LAYER = [
+    dict(sequence_len=128, vocab_size=1024, n_layer=1, n_head=5, n_kv_head=5, n_embd=640, window_pattern="L"),
+    dict(sequence_len=128, vocab_size=2048, n_layer=1, n_head=8, n_kv_head=2, n_embd=1024, window_pattern="L"),
+    dict(sequence_len=64, vocab_size=1024, n_layer=1, n_head=2, n_kv_head=2, n_embd=256, window_pattern="L"),
+]
+
+
+@pytest.mark.parametrize("cfg_kwargs,B", [(ONE_LAYER[0], 128), (ONE_LAYER[1], 8), (ONE_LAYER[2], 3)])
+def test_one_layer_models_stay_within_a_few_bf16_ulps(cfg_kwargs, B):
+    """One block on identical inputs: nothing re-quantizes a difference twice, so the logits stay within a few bf16 ulps of
+    the oracle's (the lm_head output is a bf16 number before the softcap: the ulp is taken at each logit's magnitude)."""
+    say(f"one-layer model {cfg_kwargs['n_embd']}/{cfg_kwargs['n_head']}q{cfg_kwargs['n_kv_head']}kv B={B}")
+    rt, model = build_pair(cfg_kwargs, seed=17)
+    from nanochat_amd.engine import KVCache
+    cfg = rt.cfg
+    g = torch.Generator().manual_seed(18)
+    P, steps = 11, 6
+    prompt = torch.randint(0, cfg.vocab_size, (B, P), generator=g)
+    ref = decode_ref.new_cache(cfg, B, P + steps, torch.bfloat16)
+    dec = KVCache(B, cfg.n_kv_head, P + steps, 128, 1, DEV, torch.bfloat16)
+    want = [gpt_ref.forward(rt, prompt, ref)[:, -1]]
+    got = [model.forward_last(prompt.to(DEV), kv_cache=dec).cpu()]
+    for _ in range(steps):
+        nxt = torch.randint(0, cfg.vocab_size, (B, 1), generator=g)
+        want.append(gpt_ref.forward(rt, nxt, ref)[:, -1])
+        got.append(model.forward_last(nxt.to(DEV), kv_cache=dec).cpu())
+    want, got = torch.stack(want), torch.stack(got)
+    # one bf16 ulp at the magnitude of each logit (never below the ulp of 1.0: the softcap's input was a bf16 number of that size)
+    ulp = torch.exp2(torch.floor(torch.log2(want.abs().clamp_min(1.0))) - 7)
+    in_ulps = ((got - want).abs() / ulp)
+    worst, rel = in_ulps.max().item(), rel_l2(got, want)
+    off = (in_ulps > 1.0).float().mean().item()
+    print(f"one layer: max |dlogit| {(got - want).abs().max().item():.5f} = {worst:.2f} bf16 ulp, rel-L2 {rel:.5f}, "
+          f"{off:.4%} of the logits off by more than one ulp; max |logit| {want.abs().max().item():.2f}")
+    assert worst <= 4.0 and rel <= 1e-2 and off < 0.02
+    frac, ulps = ulp_stats(dec.k_cache[0].cpu(), ref.k_cache[0])
+    assert ulps <= 2 and frac < 0.02, (frac, ulps)
+
+
+def test_layer_by_layer_taps_against_the_oracle():
+    """The residual stream as every layer reads it and every layer's attention output, HIP against the oracle, on a prefill
+    and on a decode step.  Layer 0 sees identical inputs and must agree to bf16 rounding; deeper layers may drift no more than
+    the two reference-equivalent oracle variants drift from each other at the same layer."""
+    say("layer-by-layer taps, 6 layers, trained-like")
+    cfg_kwargs = dict(sequence_len=256, vocab_size=2048, n_layer=6, n_head=3, n_kv_head=3, n_embd=384, window_pattern="SSL")
+    rt, model = build_pair(cfg_kwargs, seed=19)
+    from nanochat_amd.engine import KVCache
+    cfg = rt.cfg
+    L = cfg.n_layer
+    rt_def = gpt_ref.Runtime(cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+    g = torch.Generator().manual_seed(20)
+    B, P = 4, 23
+    prompt = torch.randint(0, cfg.vocab_size, (B, P), generator=g)
+    nxt = torch.randint(0, cfg.vocab_size, (B, 1), generator=g)
+    caches = {"sdpa": decode_ref.new_cache(cfg, B, P + 1, torch.bfloat16), "def": decode_ref.new_cache(cfg, B, P + 1, torch.bfloat16)}
+    dec = KVCache(B, cfg.n_kv_head, P + 1, 128, L, DEV, torch.bfloat16)
+    for phase, ids in (("prefill", prompt), ("decode", nxt)):
+        taps = {}
+        for name, r in (("sdpa", rt), ("def", rt_def)):
+            r.taps = {}
+            gpt_ref.forward(r, ids, caches[name])
+            taps[name], r.taps = r.taps, None
+        logits, got = model.forward_tapped(ids.to(DEV), kv_cache=dec)
+        gx, gy = got["x"].cpu(), got["y"].cpu()
+        assert gx.shape == (L + 1, B, ids.shape[1], cfg.n_embd) and gy.shape == (L, B, ids.shape[1], cfg.n_head, 128)
+        frac, ulps = ulp_stats(gx[0], taps["sdpa"]["xmix0"])
+        print(f"{phase}: layer-0 input: {frac:.4%} of the elements differ, at most {ulps} ulp")
+        assert ulps <= 1 and frac < 0.01
+        for i in range(L):
+            for key, mine in ((f"xmix{i}", gx[i]), (f"y{i}", gy[i])):
+                a, b = taps["sdpa"][key].float(), taps["def"][key].float()
+                floor = rel_l2(b, a)
+                dist = min(rel_l2(mine, a), rel_l2(mine, b))
+                print(f"{phase} {key}: HIP vs oracle rel-L2 {dist:.5f}; oracle vs oracle {floor:.5f}")
+                if i == 0:
+                    assert dist <= (5e-3 if key.startswith("y") else 1e-3), (phase, key, dist)      # bf16 rounding of identical inputs
+                else:
+                    assert dist <= 1.5 * floor + 5e-3, (phase, key, dist, floor)
+        fin = min(rel_l2(gx[L], taps["sdpa"]["xf"]), rel_l2(gx[L], taps["def"]["xf"]))
+        assert fin <= 1.5 * rel_l2(taps["def"]["xf"], taps["sdpa"]["xf"]) + 5e-3
+        assert torch.isfinite(logits).all()
+
+
+def test_greedy_prefix_matches_until_the_oracle_margin_is_inside_its_own_floor():
+    """Greedy ids through Engine.generate on a trained-like model must equal the oracle's for as long as the oracle's own
+    top-2 margin exceeds twice what the logits bar allows (1.5 x the distance between the two oracle variants at that step,
+    plus the stated 1e-2): before that point a different id cannot come from rounding."""
+    say("greedy prefix bound, d4 trained-like")
+    from nanochat_amd.engine import Engine
+    from test_engine_host import ByteTokenizer
+    D4 = dict(sequence_len=2048, vocab_size=32768, n_layer=4, n_head=2, n_kv_head=2, n_embd=256)
+    rt, model = build_pair(D4, seed=0, trained_like=True)
+    rt_def = gpt_ref.Runtime(rt.cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+
+    class Tok(ByteTokenizer):
+        def __init__(self):
+            self._special = {"<|python_start|>": 32760, "<|python_end|>": 32761, "<|output_start|>": 32762,
+                             "<|output_end|>": 32763, "<|assistant_end|>": 32764, "<|bos|>": 32765}
+
+        def get_bos_token_id(self):
+            return 32765
+    for seed in (0, 3):
+        g = torch.Generator().manual_seed(seed)
+        prompt = torch.randint(0, 32000, (32,), generator=g).tolist()
+        n = 64
+        want_cols, want_logits = decode_ref.generate(rt, prompt, 1, n, temperature=0.0, collect_logits=True)
+        want_ids = [c[0] for c in want_cols]
+        # the other oracle variant, fed the same tokens
+        c = decode_ref.new_cache(rt.cfg, 1, 32 + n, torch.bfloat16)
+        other = [gpt_ref.forward(rt_def, torch.tensor([prompt]), c)[:, -1]]
+        for t in range(n - 1):
+            other.append(gpt_ref.forward(rt_def, torch.tensor([[want_ids[t]]]), c)[:, -1])
+        floor_so_far, must_match = 0.0, n
+        for t in range(n):
+            floor_so_far = max(floor_so_far, (want_logits[t] - other[t]).abs().max().item())
+            top2 = torch.topk(want_logits[t][0], 2).values
+            if (top2[0] - top2[1]).item() <= 2 * (1.5 * floor_so_far + LOGIT_TOL):
+                must_match = t
+                break
+        got_ids = []
+        for column, masks in Engine(model, Tok()).generate(prompt, num_samples=1, max_tokens=n, temperature=0.0):
+            got_ids.append(column[0])
+            if column[0] in (32764, 32765):
+                break
+        first_div = next((i for i, (a, b) in enumerate(zip(got_ids, want_ids)) if a != b), len(got_ids))
+        print(f"seed {seed}: ids equal for {first_div} tokens; the oracle's margin first falls inside its floor at token {must_match}")
+        assert first_div >= min(must_match, len(got_ids)), (first_div, must_match)
+
+
+# ------------------------------------------------------------------------------------------------ BASELINE config 3
+class RecordingSampler:
+    """Stands in for nanochat_amd.engine.sample_next_token: draws the Exp(1) variates the way the Engine's sampler does, calls the
+    HIP sampler with them, and keeps (logits, noise, ids) of every step.  With same_noise_for_all_rows the variates of row 0
+    are used for every row."""
+
+    def __init__(self, ops, same_noise_for_all_rows=False):
+        self.ops, self.same, self.steps = ops, same_noise_for_all_rows, []
+
+    def __call__(self, logits, rng, temperature=1.0, top_k=None):
+        B, V = logits.shape
+        k = min(top_k, V) if (top_k is not None and top_k > 0) else V
+        noise = torch.empty(B, k, dtype=torch.float32, device=logits.device).exponential_(1.0, generator=rng)
+        if self.same:
+            noise = noise[:1].expand(B, k).contiguous()
+        ids = self.ops.sample(logits.float(), temperature, top_k, noise)
+        self.steps.append((logits.float().cpu(), noise.cpu(), ids.cpu()))
+        return ids
+
+
+def test_config3_d20_batch8_sampled_generation(ops, monkeypatch):
+    """d20 (n_embd 1280, 10 heads, 20 layers, vocabulary 32768), one 512-token prompt replicated to 8 rows, temperature 1.0,
+    top_k 50 through Engine.generate: reproducible per seed; rows identical when they draw identical variates; every sampled id
+    is the oracle sampler's id on the same logits and variates; the prefill and the first decode steps' logits against the
+    oracle model."""
+    say("config 3: d20 B=8 prompt 512, T=1.0 top_k=50")
+    import nanochat_amd.engine as engine_mod
+    from nanochat_amd.engine import Engine
+    from nanochat_amd.synthetic import SyntheticTokenizer
+    cfg_kwargs = dict(sequence_len=2048, vocab_size=32768, n_layer=20, n_head=10, n_kv_head=10, n_embd=1280)
+    rt, model = build_pair(cfg_kwargs, seed=1)
+    g = torch.Generator().manual_seed(1)
+    prompt = torch.randint(0, 32768, (512,), generator=g).tolist()
+    eng = Engine(model, SyntheticTokenizer())
+    kw = dict(num_samples=8, max_tokens=24, temperature=1.0, top_k=50)
+    a, _ = eng.generate_batch(prompt, seed=11, **kw)
+    b, _ = eng.generate_batch(prompt, seed=11, **kw)
+    c, _ = eng.generate_batch(prompt, seed=12, **kw)
+    assert a == b and a != c and len(a) == 8 and all(len(r) == 512 + 24 for r in a)
+    assert len({tuple(r[512:]) for r in a}) > 1                                 # rows sample independently
+    # every step's id against the oracle sampler on the same logits and variates
+    rec = RecordingSampler(ops)
+    monkeypatch.setattr(engine_mod, "sample_next_token", rec)
+    d, _ = eng.generate_batch(prompt, seed=11, **kw)
+    assert d == a                                                               # the stand-in draws what the Engine's sampler draws
+    assert len(rec.steps) == 24
+    for t, (logits, noise, ids) in enumerate(rec.steps):
+        want = decode_ref.sample_with_noise(logits, 1.0, 50, noise)
+        assert torch.equal(ids, want), f"step {t}"
+        assert [r[512 + t] for r in d] == ids[:, 0].tolist()
+    # identical variates for every row: the rows stay identical, bit for bit, logits included
+    same = RecordingSampler(ops, same_noise_for_all_rows=True)
+    monkeypatch.setattr(engine_mod, "sample_next_token", same)
+    e, _ = eng.generate_batch(prompt, seed=11, **kw)
+    assert all(r == e[0] for r in e)
+    for logits, _, ids in same.steps:
+        assert torch.equal(logits, logits[:1].expand_as(logits)) and (ids == ids[0]).all()
+    monkeypatch.undo()
+    # the model itself against the oracle: the 512-token prefill and three decode steps on the tokens row 0..7 sampled
+    steps = [torch.tensor([[r[512 + t]] for r in a]) for t in range(3)]
+
+    def run(r):
+        pre = decode_ref.new_cache(r.cfg, 1, 512, torch.bfloat16)
+        outs = [gpt_ref.forward(r, torch.tensor([prompt]), pre)[:, -1].expand(8, -1)]
+        dec = decode_ref.new_cache(r.cfg, 8, 512 + 3, torch.bfloat16)
+        dec.prefill(pre)
+        for nxt in steps:
+            outs.append(gpt_ref.forward(r, nxt, dec)[:, -1])
+        return torch.stack(outs)
+    floor_rel, floor_max, want, want_def = oracle_floor(rt, run)
+    got = torch.stack([lg for lg, _, _ in rec.steps[:4]])
+    assert_within_floor(got, want, want_def, floor_rel, floor_max, "d20 prefill + 3 sampled decode steps")
+
+
+# ------------------------------------------------------------------------------------------------ BASELINE config 5
+def test_config5_d32_gqa_width_ragged_prefill_and_sampled_decode(ops):
+    """The d32-GQA width (n_embd 2048, 16 query / 4 kv heads) with three layers, so that the CPU oracle can follow: rows with
+    ragged prompt lengths are prefilled one by one (the reference's forward takes one length per call), gathered into one
+    cache with per-row lengths, and decoded together at temperature 0.8 / top_k 50."""
+    say("config 5 width: ragged prefill + sampled decode, 3 layers")
+    from nanochat_amd.engine import KVCache
+    cfg_kwargs = dict(sequence_len=2048, vocab_size=32768, n_layer=3, n_head=16, n_kv_head=4, n_embd=2048)
+    rt, model = build_pair(cfg_kwargs, seed=3)
+    rt_def = gpt_ref.Runtime(rt.cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+    cfg = rt.cfg
+    g = torch.Generator().manual_seed(3)
+    lens = [64, 333, 1201, 2040]
+    B, Tmax, steps = len(lens), 2048, 3
+    prompts = [torch.randint(0, cfg.vocab_size, (1, n), generator=g) for n in lens]
+    big = KVCache(B, cfg.n_kv_head, Tmax, 128, cfg.n_layer, DEV, torch.bfloat16)
+    ref_big = decode_ref.new_cache(cfg, B, Tmax, torch.bfloat16)
+    def_big = decode_ref.new_cache(cfg, B, Tmax, torch.bfloat16)
+    prevs, rprevs, dprevs, first_got, first_want, first_def = [], [], [], [], [], []
+    for b, pr in enumerate(prompts):
+        one = KVCache(1, cfg.n_kv_head, lens[b], 128, cfg.n_layer, DEV, torch.bfloat16)
+        first_got.append(model.forward_last(pr.to(DEV), kv_cache=one).cpu())
+        big.k_cache[:, b, :lens[b]] = one.k_cache[:, 0]
+        big.v_cache[:, b, :lens[b]] = one.v_cache[:, 0]
+        prevs.append(one.prev_embedding)
+        for r, dst, keep, firsts in ((rt, ref_big, rprevs, first_want), (rt_def, def_big, dprevs, first_def)):
+            o = decode_ref.new_cache(cfg, 1, lens[b], torch.bfloat16)
+            firsts.append(gpt_ref.forward(r, pr, o)[:, -1])
+            dst.k_cache[:, b, :lens[b]] = o.k_cache[:, 0]
+            dst.v_cache[:, b, :lens[b]] = o.v_cache[:, 0]
+            keep.append(o.prev_embedding)
+    # the ragged prefill, row by row
+    fg, fw, fd = torch.cat(first_got), torch.cat(first_want), torch.cat(first_def)
+    assert_within_floor(fg, fw, fd, rel_l2(fd, fw), (fw - fd).abs().max().item(), "ragged prefill at d32-GQA width")
+    big.set_seqlens(lens)
+    big.prev_embedding = torch.cat(prevs, dim=0)
+    for c, keep in ((ref_big, rprevs), (def_big, dprevs)):
+        c.cache_seqlens.copy_(torch.tensor(lens, dtype=torch.int32))
+        c.prev_embedding = torch.cat(keep, dim=0)
+    # the oracle takes per-row positions only in its fp32-definition form; the second variant for the floor is the same
+    # form over the cache the SDPA oracle prefilled
+    rt_rag = gpt_ref.Runtime(cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+    rng = torch.Generator(device=DEV).manual_seed(5)
+    logits = fg.to(DEV)
+    S, Dd, G = [], [], []
+    for s in range(steps):
+        noise = torch.empty(B, 50, dtype=torch.float32, device=DEV).exponential_(1.0, generator=rng)
+        ids = ops.sample(logits, 0.8, 50, noise)
+        assert torch.equal(ids.cpu(), decode_ref.sample_with_noise(logits.cpu(), 0.8, 50, noise.cpu()))
+        if lens[-1] + s >= Tmax:
+            break
+        logits = model.forward_last(ids, kv_cache=big)
+        G.append(logits.cpu())
+        S.append(gpt_ref.forward(rt_rag, ids.cpu(), ref_big)[:, -1])
+        Dd.append(gpt_ref.forward(rt_def, ids.cpu(), def_big)[:, -1])
+    S, Dd, G = torch.stack(S), torch.stack(Dd), torch.stack(G)
+    assert big.cache_seqlens.tolist() == [n + len(G) for n in lens]
+    assert_within_floor(G, S, Dd, max(rel_l2(Dd, S), 0.03), (S - Dd).abs().max().item(), "ragged sampled decode at d32-GQA width")
