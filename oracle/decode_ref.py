@@ -50,12 +50,17 @@ def new_cache(cfg, batch, seq_len, dtype):
 def sample_with_noise(logits, temperature, top_k, noise):
     """engine.py:140-156 with torch.multinomial written out as its definition:
     multinomial(p, 1) == argmax(p / e), e ~ Exp(1) drawn from the generator.
-    ``noise`` holds those exponentials, shape [B, k] (or [B, V] without top-k)."""
+    ``noise`` holds those exponentials, shape [B, k] (or [B, V] without top-k).
+
+    torch.topk leaves the order of equal values unspecified (it differs between its CPU and GPU kernels), and bf16-rounded
+    logits tie often; equal values are taken lowest index first here (a stable descending sort), which is one of the
+    orders torch.topk may return and equals it whenever the k+1 largest values are distinct."""
     if temperature == 0.0:
         return torch.argmax(logits, dim=-1, keepdim=True)
     if top_k is not None and top_k > 0:
         k = min(top_k, logits.size(-1))
-        vals, idx = torch.topk(logits, k, dim=-1)
+        vals, idx = torch.sort(logits, dim=-1, descending=True, stable=True)
+        vals, idx = vals[:, :k], idx[:, :k]
         probs = F.softmax(vals / temperature, dim=-1)
         choice = torch.argmax(probs / noise, dim=-1, keepdim=True)
         return idx.gather(1, choice)

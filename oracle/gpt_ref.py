@@ -217,7 +217,7 @@ def forward(rt: Runtime, idx, kv_cache=None):
         elif prev is not None:
             gate = lam_s * torch.sigmoid(small_linear(x[:, :, :SMEAR_CHANNELS], gate_w))
             x = x + gate * prev
-    rt.tap("x0", x)
+    rt.tap("xemb", x)
 
     x0 = x
     x_backout = None
@@ -229,9 +229,12 @@ def forward(rt: Runtime, idx, kv_cache=None):
         ve = F.embedding(idx, p[ve_name]).to(x.dtype) if ve_name in p else None
         # --- attention
         xn = rms_norm(x)
+        rt.tap(f"xn{i}", xn)
         q = rt.linear(xn, pre + "attn.c_q.weight").view(B, T, H, D)
         k = rt.linear(xn, pre + "attn.c_k.weight").view(B, T, Hkv, D)
         v = rt.linear(xn, pre + "attn.c_v.weight").view(B, T, Hkv, D)
+        if rt.taps is not None:
+            rt.tap(f"qkv{i}", torch.cat([q.reshape(B, T, -1), k.reshape(B, T, -1), v.reshape(B, T, -1)], dim=-1))
         if ve is not None:
             ve = ve.view(B, T, Hkv, D)
             g = 3 * torch.sigmoid(small_linear(xn[..., :VE_GATE_CHANNELS], p[pre + "attn.ve_gate.weight"]))
@@ -257,11 +260,19 @@ def forward(rt: Runtime, idx, kv_cache=None):
                 kv_cache.advance(T)
         rt.tap(f"y{i}", y)
         y = y.contiguous().view(B, T, -1)
-        x = x + rt.linear(y, pre + "attn.c_proj.weight")
+        attn_out = rt.linear(y, pre + "attn.c_proj.weight")
+        rt.tap(f"attn_out{i}", attn_out)
+        x = x + attn_out
+        rt.tap(f"xmid{i}", x)
         # --- MLP
-        h = rt.linear(rms_norm(x), pre + "mlp.c_fc.weight")
+        xn2 = rms_norm(x)
+        rt.tap(f"xn2_{i}", xn2)
+        h = rt.linear(xn2, pre + "mlp.c_fc.weight")
         h = F.relu(h).square()
-        x = x + rt.linear(h, pre + "mlp.c_proj.weight")
+        rt.tap(f"h2_{i}", h)
+        mlp_out = rt.linear(h, pre + "mlp.c_proj.weight")
+        rt.tap(f"mlp_out{i}", mlp_out)
+        x = x + mlp_out
         rt.tap(f"x{i}", x)
         if i == L // 2:
             x_backout = x

@@ -118,7 +118,7 @@ def test_checkpoint_model_matches_the_oracle_on_the_same_file(tmp_path):
     from nanochat_amd import ops
     from oracle import fp8_ref
     for key, mod in (("lm_head.weight", model.lm_head), ("transformer.h.1.mlp.c_proj.weight", model.transformer.h[1].mlp.c_proj)):
-        w8, inv = fp8_ref.to_fp8(state[key])
+        w8, inv, _ = fp8_ref.to_fp8(state[key])
         payload, inv_gpu, _ = ops.fp8_quantize(mod.weight.detach())
         assert torch.equal(payload.cpu().view(torch.uint8), w8.view(torch.uint8)), key
         assert inv_gpu.cpu().view(torch.int32).item() == inv.reshape(()).view(torch.int32).item(), key
