@@ -159,6 +159,18 @@ int nc_qkv_rope_append_attention(const uint16_t* qkv, int ld_qkv, const uint16_t
                                  int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax, int vocab_rows,
                                  void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits, nc_stream_t stream);
 
+/* nc_decode_attention for callers that cannot allocate device memory and have no workspace to hand over: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid allocation.  It has no counterpart in the reference.  Same
+ * arguments and results as nc_decode_attention minus the workspace: the split counters and partial results live in a
+ * device array built into the library (8.65 MB, held by every GPU the library runs on until the process ends).  Limit:
+ * B * T * H <= nc_decode_attention_static_max_row_heads() (1024), larger calls are refused with an error.  The call
+ * allocates nothing and clears what it needs itself with a fill kernel.  All calls on one GPU share the array: calls that
+ * overlap on one GPU (two streams, two threads) race; serialise them. */
+size_t nc_decode_attention_static_max_row_heads(void);
+int nc_decode_attention_static(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                               const int32_t* cache_seqlens, int window_left, uint16_t* out, int B, int T, int H, int Hkv,
+                               int Tmax, int seqlens_include_new, uint32_t* amax_ws, int splits, nc_stream_t stream);
+
 /* How a decode-attention launch of this shape is laid out (no counterpart in the reference; for tests and tuning):
  * *splits_out = workgroups that share the keys of one (row, kv head); *heads_per_workgroup_out = 1, or 2 when a workgroup
  * streams two neighbouring kv heads.  splits: the caller's request (0 = choose), as passed to the attention calls. */

@@ -16,6 +16,7 @@ EXPORTS = [
     "nc_attention_workspace_bytes", "nc_decode_attention", "nc_kv_cache_prefill", "nc_softcap", "nc_sample",
     "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read",
     "nc_decode_attention_append", "nc_qkv_rope_append_attention", "nc_decode_attention_plan", "nc_gpt_forward_tapped",
+    "nc_decode_attention_static", "nc_decode_attention_static_max_row_heads",
 ]
 
 
@@ -67,6 +68,8 @@ def _bind(lib):
         "nc_decode_attention": (i, [p, p, p, p, i, p, i, i, i, i, i, i, p, sz, p, i, p]),
         "nc_decode_attention_append": (i, [p, p, p, p, p, p, i, p, i, i, i, i, i, p, sz, p, i, p]),
         "nc_qkv_rope_append_attention": (i, [p, i, p, i, p, p, p, p, p, i, p, p, p, i, p, i, i, i, i, i, p, sz, p, i, p]),
+        "nc_decode_attention_static": (i, [p, p, p, p, i, p, i, i, i, i, i, i, p, i, p]),
+        "nc_decode_attention_static_max_row_heads": (sz, []),
         "nc_decode_attention_plan": (i, [i, i, i, i, i, i, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
         "nc_kv_cache_prefill": (i, [p, p, i, i, i, i, i, i, i, p]),
         "nc_softcap": (i, [p, p, i64, f, p]),

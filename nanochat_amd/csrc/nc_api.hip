@@ -183,6 +183,15 @@ int nc_qkv_rope_append_attention(const uint16_t* qkv, int ld_qkv, const uint16_t
                                      amax_ws, splits, 0, (hipStream_t)stream);
 }
 
+size_t nc_decode_attention_static_max_row_heads(void) { return nc_attention_static_max_row_heads(); }
+
+int nc_decode_attention_static(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int32_t* cache_seqlens,
+                               int window_left, uint16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
+                               uint32_t* amax_ws, int splits, nc_stream_t stream) {
+    return nc_launch_attention_static(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new, amax_ws,
+                                      splits, (hipStream_t)stream);
+}
+
 int nc_decode_attention_plan(int B, int T, int Hkv, int window_left, int Tmax, int splits, int* splits_out, int* heads_per_workgroup_out) {
     NC_CHECK_ARG(B > 0 && T > 0 && Hkv > 0 && Tmax > 0, "decode_attention_plan: bad shape");
     nc_attention_plan(B, T, Hkv, window_left, Tmax, splits, splits_out, heads_per_workgroup_out);

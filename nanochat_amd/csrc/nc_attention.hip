@@ -500,3 +500,53 @@ int nc_launch_attention_append(const bf16_t* q, const bf16_t* k_new, const bf16_
     return launch_attention_impl(q, nullptr, 0, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, 0, counters, partials,
                                  partial_bytes, amax_ws, force_splits, 0, s);
 }
+
+// ------------------------------------------------------------------------------------------------
+// The same attention for callers that cannot allocate and have no workspace to bring (code under HIP graph capture, tight serving
+// loops): the split counters and partial results live in a file-scope device array instead of a caller's buffer.  Every GPU the
+// library runs on holds its own copy of the array, at its own address, until the process ends; the address is looked up once per
+// device, with that device current, and only that looked-up pointer is ever handed to a kernel (the array's name in host code is
+// a host-side stand-in, not a device address).  All calls on one GPU share the array: calls that overlap there race.
+#define NC_STATIC_ATTN_MAX_ROW_HEADS 1024     // B * T * H at most: 1024 * (16 splits * 132 floats + one counter)
+#define NC_STATIC_ATTN_COUNTER_BYTES ((size_t)NC_STATIC_ATTN_MAX_ROW_HEADS * sizeof(uint32_t))
+#define NC_STATIC_ATTN_PARTIAL_BYTES ((size_t)NC_STATIC_ATTN_MAX_ROW_HEADS * 16 * PART_STRIDE * sizeof(float))
+static __device__ __align__(256) unsigned char scratch[NC_STATIC_ATTN_COUNTER_BYTES + NC_STATIC_ATTN_PARTIAL_BYTES];
+
+#define NC_MAX_DEVICES 64
+static void* g_scratch_ptr[NC_MAX_DEVICES];      // per device: the address of that device's copy of scratch[]
+
+// The device-side address of scratch[] on the current device, or nullptr after nc_set_error().
+static void* static_scratch_for_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NC_MAX_DEVICES) {
+        nc_set_error("decode_attention_static: no current device (or more than %d devices)", NC_MAX_DEVICES);
+        return nullptr;
+    }
+    void* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            nc_set_error("decode_attention_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);    // two threads racing here look up the same address
+    }
+    return p;
+}
+
+size_t nc_attention_static_max_row_heads(void) { return NC_STATIC_ATTN_MAX_ROW_HEADS; }
+
+int nc_launch_attention_static(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
+                               bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new, uint32_t* amax_ws,
+                               int force_splits, hipStream_t s) {
+    NC_CHECK_ARG(B > 0 && T > 0 && H > 0, "decode_attention_static: bad shape");
+    NC_CHECK_ARG((long)B * T * H <= NC_STATIC_ATTN_MAX_ROW_HEADS,
+                 "decode_attention_static: %ld (row, head) pairs exceed the built-in scratch of %d; use nc_decode_attention with a workspace",
+                 (long)B * T * H, NC_STATIC_ATTN_MAX_ROW_HEADS);
+    unsigned char* base = (unsigned char*)static_scratch_for_current_device();
+    if (!base) return -2;
+    // the counters are cleared by a small fill kernel inside the launch (what the previous call left there is not trusted)
+    return launch_attention_impl(q, nullptr, 0, const_cast<bf16_t*>(k_cache), const_cast<bf16_t*>(v_cache), cache_seqlens, window_left, out, B,
+                                 T, H, Hkv, Tmax, seqlens_include_new, (uint32_t*)base, base + NC_STATIC_ATTN_COUNTER_BYTES,
+                                 NC_STATIC_ATTN_PARTIAL_BYTES, amax_ws, force_splits, 0, s);
+}

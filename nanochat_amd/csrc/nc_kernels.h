@@ -94,6 +94,10 @@ int nc_launch_attention_append(const bf16_t* q, const bf16_t* k_new, const bf16_
                                const int32_t* cache_seqlens, int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax,
                                uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws, int force_splits,
                                hipStream_t s);
+size_t nc_attention_static_max_row_heads(void);
+int nc_launch_attention_static(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
+                               bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new, uint32_t* amax_ws,
+                               int force_splits, hipStream_t s);
 struct NcRopeSrc;
 int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, const int32_t* cache_seqlens, int window_left,
                               bf16_t* out, int B, int H, int Hkv, int Tmax, uint32_t* counters, void* partials, size_t partial_bytes,
