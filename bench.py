@@ -6,13 +6,15 @@ Workload (the headline decode configuration): nanochat d26 (n_embd 1664, 13 head
 vocab 32768, window pattern SSSL), bf16 weights with FP8 linears, random init seed 2; one prompt of
 random token ids is prefilled at batch 1, the KV cache is replicated to 64 rows, and greedy decoding
 runs through Engine.generate until the context reaches 2048 tokens.  A "step" is one iteration of that
-loop: sample for all 64 rows + one GPT.forward(ids[64,1], kv_cache).  The prompt length is chosen so
-that the last timed step ends at context 2048 (1792 prompt tokens for the default 8 + 248 steps).
+loop: sample for all 64 rows + one GPT.forward(ids[64,1], kv_cache).  The run is: W warm-up steps, P steps
+with a HIP event pair around every kernel launch (the roofline figures), then the K timed steps, the last
+of which brings the context to 2048; the prompt is 2048 - (W + P + K) tokens long: 1792 for the default
+8 + 16 + 232, i.e. 256 new tokens.
 
 One JSON line is printed with tokens/s, the roofline of the dominant kernel (decode attention, HBM
-bound; its time is measured with HIP events on the launch stream in extra steps right after the timed
-region), FP8 GEMM rates at the isolated Float8Linear shapes, and a CPU baseline (the CPU oracle, a
-port of the reference's CPU behaviour, timed on this box's host cores on a bounded sample).
+bound), the rate of every decode linear against the HBM peak, FP8 GEMM rates at the isolated Float8Linear
+shapes, and a CPU baseline (the CPU oracle, a port of the reference's CPU behaviour, timed on this box's
+host cores on a bounded sample of the decode step and of the isolated GEMM shapes).
 """
 import argparse
 import ctypes as C
@@ -150,6 +152,32 @@ def gemm_rates(device, library_gemm=False):
     return out
 
 
+def cpu_gemm_baseline(cores, budget_s=6.0):
+    """The reference's own CPU call for the isolated Float8Linear shapes (torch._scaled_mm on e4m3 operands, nanochat/fp8.py:143-153)
+    and the fp8-emulated fp32 matmul beside it, on a row sample of M (the work is linear in M): GFLOP/s per shape."""
+    from oracle import fp8_ref
+    torch.set_num_threads(cores)
+    out = {}
+    g = torch.Generator().manual_seed(0)
+    for K, N in [(1664, 4992), (1664, 1664), (1664, 6656), (6656, 1664)]:
+        M = 512                                   # of the 8192 rows
+        a = torch.randn(M, K, generator=g).bfloat16()
+        w = ((torch.rand(N, K, generator=g) * 2 - 1) * (3.0 / K) ** 0.5).bfloat16()
+        a8, ia, _ = fp8_ref.to_fp8(a)
+        w8, iw, _ = fp8_ref.to_fp8(w)
+        rec = {}
+        for name, fn, rows in (("emulated_fp32_matmul", fp8_ref.scaled_mm_emulated, M), ("torch_scaled_mm", fp8_ref.scaled_mm_library, 16)):
+            fn(a8[:rows], w8, ia, iw)
+            n, t0 = 0, time.time()
+            while n < 1 or (time.time() - t0 < budget_s / 8 and n < 20):
+                fn(a8[:rows], w8, ia, iw)
+                n += 1
+            rec[name + "_gflops"] = round(2.0 * rows * N * K * n / (time.time() - t0) / 1e9, 2)
+            rec[name + "_rows_timed"] = rows
+        out[f"K{K}_N{N}"] = rec
+    return out
+
+
 def cpu_baseline(budget_s=25.0):
     """One decode step of the CPU oracle at the same shape (d26, 64 rows, context 1792), bf16 with
     fp8-emulated linears, weights re-quantized on every call as the reference does (fp8.py:136)."""
@@ -206,25 +234,39 @@ def cpu_baseline(budget_s=25.0):
     return {"value": round(BATCH * steps / spent, 3), "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"{steps} decode step(s) of the CPU oracle at d26, 64 rows, context {ctx} (random-filled cache), bf16 + "
                       f"fp8-emulated linears with per-call weight quantization as in the reference; setup {setup_s:.0f}s not timed",
-            "s_per_step": round(spent / steps, 3)}
+            "s_per_step": round(spent / steps, 3),
+            "fp8_gemm_m8192": cpu_gemm_baseline(cores)}
+
+
+def attention_sources_digest():
+    """SHA-256 over the sources of the decode-attention kernel: ties a counter measurement to the code it was taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in ("nc_attention.hip", "nc_rope.h", "nc_common.h"):
+        h.update(open(os.path.join(ROOT, "nanochat_amd", "csrc", f), "rb").read())
+    return h.hexdigest()
 
 
 def measured_traffic():
     """HBM bytes per attention launch from the hardware counters (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc runs of this
     script, scaled by what the same counters read for the --copy-probe-mib pass).  The counters cannot be collected from
-    inside this process, so the figure is read from the summary committed next to the profiles; None if absent."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "attn_partial_d26_b64_traffic.json")
+    inside this process, so the figure is read from the summary committed next to the profiles, which names the kernel
+    sources it was measured on: (bytes, note); bytes is None if the summary is absent or was taken on other sources."""
+    path = os.path.join(ROOT, "profiles", "attn_partial_d26_b64_traffic.json")
     try:
         with open(path) as f:
-            return json.load(f)["hbm_bytes_per_launch"]
+            rec = json.load(f)
+        if rec.get("kernel_sources_sha256") != attention_sources_digest():
+            return None, "profiles/attn_partial_d26_b64_traffic.json was measured on other kernel sources than this tree holds"
+        return rec["hbm_bytes_per_launch"], "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script on these kernel sources (profiles/)"
     except (OSError, KeyError, ValueError):
-        return None
+        return None, "no counter summary under profiles/"
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=248)
+    ap.add_argument("--steps", type=int, default=232)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
@@ -249,16 +291,14 @@ def main():
 
     D26["window_pattern"] = args.window_pattern
     K, W, P = args.steps, args.warmup, max(1, args.profile_steps)
-    total_new = W + K + P
-    prompt_len = CONTEXT - (W + K)            # the last timed step brings the context to 2048
-    assert prompt_len >= 1, "steps + warmup must stay below the 2048-token context"
+    total_new = W + P + K
+    prompt_len = CONTEXT - total_new          # the last timed step brings the context to 2048
+    assert prompt_len >= 1, "warmup + profile steps + steps must stay below the 2048-token context"
     model = build_model(device)
     engine = Engine(model, RangeTokenizer())
     g = torch.Generator().manual_seed(2)
     prompt = torch.randint(0, D26["vocab_size"], (prompt_len,), generator=g).tolist()
 
-    # Engine.generate sizes the decode cache as prompt + max_tokens; the profiled extra steps run past the
-    # timed region, so the rotary/cache bound is 2048 + P (the rotary table covers 10x the context).
     # one-off work (FP8 weight quantization of the plan, workspace allocation) is kept out of the time to first token
     for _ in engine.generate(prompt[:64], num_samples=2, max_tokens=2, temperature=0.0):
         pass
@@ -271,7 +311,29 @@ def main():
     for _ in range(W - 1):
         next(gen)
     torch.cuda.synchronize()
+
+    # ---- kernel-level timing, HIP events on the launch stream, same process and state, inside the configured context:
+    # the forwards of these P steps see contexts prompt_len + W + 1 .. prompt_len + W + P
+    lib.nc_profile_enable(1)
+    for _ in range(P):
+        next(gen)
+    torch.cuda.synchronize()
+    prof = {c: read_profile(lib, c) for c in range(5)}
+    E, H, Hkv, V = D26["n_embd"], D26["n_head"], D26["n_kv_head"], D26["vocab_size"]
+    linears = {}
+    for name, (N, Kd) in (("qkv", ((H + 2 * Hkv) * 128, E)), ("attn_c_proj", (E, H * 128)), ("c_fc", (4 * E, E)), ("mlp_c_proj", (E, 4 * E)),
+                          ("lm_head", (V, E))):
+        ms, units, n = C.c_double(), C.c_double(), C.c_int64()
+        assert lib.nc_profile_read_gemm(N, Kd, C.byref(ms), C.byref(units), C.byref(n)) == 0
+        if n.value:
+            us = ms.value * 1e3 / n.value
+            # a decode linear streams its e4m3 weight once: N * K bytes (the 64 activation rows are L2 traffic)
+            linears[name] = {"weight_bytes": N * Kd, "launches_timed": n.value, "avg_launch_us": round(us, 2),
+                             "gbps": round(N * Kd / us / 1e3, 1), "frac_hbm_peak": round(N * Kd / (us * 1e-6) / HBM_PEAK, 4)}
+    lib.nc_profile_enable(0)
+
     step_times = []
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(K):
         t1 = time.perf_counter()
@@ -280,14 +342,6 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     tok_per_s = BATCH * K / elapsed
-
-    # ---- kernel-level timing, HIP events on the launch stream, same process and state
-    lib.nc_profile_enable(1)
-    for _ in range(P):
-        next(gen)
-    torch.cuda.synchronize()
-    prof = {c: read_profile(lib, c) for c in range(5)}
-    lib.nc_profile_enable(0)
     gen.close()
     if args.copy_probe_mib > 0:
         n = args.copy_probe_mib * (1 << 20) // 2
@@ -298,13 +352,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     att_ms, _, att_n = prof[0]
-    ctx_mid = CONTEXT + P // 2                 # profiled steps sit just past the timed region
-    att_bytes_step = attention_bytes_per_step(model, BATCH, ctx_mid)
+    # the P profiled forwards ran at cache lengths prompt_len + W .. prompt_len + W + P - 1 (each then sees one more key: itself)
     launches_per_step = model.config.n_layer
+    att_bytes_step = sum(attention_bytes_per_step(model, BATCH, prompt_len + W + j + 1) for j in range(P)) / P
     att_avg_s = att_ms * 1e-3 / att_n
     att_bytes_launch = att_bytes_step / launches_per_step
     achieved = att_bytes_launch / att_avg_s
     per_step_ms = {name: round(prof[c][0] / P, 3) for c, name in enumerate(["attention", "fp8_gemm", "quantize", "rows", "sampler"])}
+    traffic, traffic_note = measured_traffic() if args.window_pattern == "SSSL" else (None, "counter summary exists for window pattern SSSL only")
+    weight_bytes_step = sum(v["weight_bytes"] * (1 if k == "lm_head" else model.config.n_layer) for k, v in linears.items())
 
     result = {
         "metric": "decode tokens/sec @ d26 bs64 ctx2048",
@@ -319,18 +375,25 @@ def main():
         "vs_baseline": None,
         "dtype": "fp8_e4m3 x fp8_e4m3 -> fp32 acc (linears), bf16 (KV cache, activations)",
         "data": "synthetic: random token ids, random-init weights of the d26 architecture (seed 2)",
-        "config": {"workload": f"nanochat d26 decode, batch 64, context 1792->2048, greedy, window pattern {args.window_pattern}, "
+        "config": {"workload": f"nanochat d26 decode (BASELINE configs[3]), batch 64, prompt {prompt_len} tokens, {total_new} new tokens, "
+                               f"timed steps at context {CONTEXT - K}->{CONTEXT}, greedy, window pattern {args.window_pattern}, "
                                "Engine.generate loop (sample + GPT.forward with KV cache per step)",
-                   "batch": BATCH, "context_end": CONTEXT, "prompt_tokens": prompt_len},
+                   "batch": BATCH, "context_end": CONTEXT, "prompt_tokens": prompt_len, "new_tokens": total_new,
+                   "profiled_steps_context": [prompt_len + W + 1, prompt_len + W + P]},
         "tpot_ms_median": round(sorted(step_times)[len(step_times) // 2] * 1e3, 4),
         "ttft_s": round(ttft, 3),
         "roofline": {"bound": "hbm", "kernel": "attn_partial_kernel (+combine) per layer launch",
                      "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4),
-                     "traffic": measured_traffic() if args.window_pattern == "SSSL" else None,
+                     "traffic": traffic, "traffic_source": traffic_note,
                      "bytes_per_launch": int(att_bytes_launch), "avg_launch_us": round(att_avg_s * 1e6, 2),
                      "launches_timed": att_n},
         "kernel_ms_per_step": per_step_ms,
+        # the weight-streaming linears of the decode step against the HBM peak (HIP events around each launch, in-step)
+        "decode_linears": linears,
+        # the reference's MBU numerator with the bytes really streamed: e4m3 weights + KV read at the profiled context
+        "step_bytes": {"weights_e4m3": weight_bytes_step, "kv_read": int(att_bytes_step),
+                       "frac_hbm_peak_whole_step": round((weight_bytes_step + att_bytes_step) / (elapsed / K) / HBM_PEAK, 4)},
     }
     if not args.no_gemm:
         result["fp8_gemm_m8192"] = gemm_rates(device, args.library_gemm)

@@ -263,6 +263,8 @@ int nc_gpt_forward_tapped(const nc_model_desc* model /*host*/, const nc_cache_de
  * safe; at most 16384 launches are recorded per enable. */
 int nc_profile_enable(int on);
 int nc_profile_read(int cls, double* total_ms /*host*/, double* total_units /*host*/, int64_t* count /*host*/);
+/* The FP8 GEMM launches (class 1) of one weight shape [N,K] only: the decode step's four linears and lm_head apart. */
+int nc_profile_read_gemm(int N, int K, double* total_ms /*host*/, double* total_units /*host*/, int64_t* count /*host*/);
 
 #ifdef __cplusplus
 }

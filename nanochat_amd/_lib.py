@@ -14,7 +14,7 @@ EXPORTS = [
     "nc_fp8_small_m_workspace_bytes", "nc_fp8_linear_small_m",
     "nc_rmsnorm", "nc_embed_norm_smear", "nc_mix_norm", "nc_relu2", "nc_qkv_rope_append",
     "nc_attention_workspace_bytes", "nc_decode_attention", "nc_kv_cache_prefill", "nc_softcap", "nc_sample",
-    "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read",
+    "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read", "nc_profile_read_gemm",
     "nc_decode_attention_append", "nc_qkv_rope_append_attention", "nc_decode_attention_plan", "nc_gpt_forward_tapped",
     "nc_decode_attention_static", "nc_decode_attention_static_max_row_heads",
 ]
@@ -79,6 +79,7 @@ def _bind(lib):
         "nc_gpt_forward_tapped": (i, [C.POINTER(ModelDesc), C.POINTER(CacheDesc), p, i, i, p, i, p, sz, p, p, p]),
         "nc_profile_enable": (i, [i]),
         "nc_profile_read": (i, [i, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
+        "nc_profile_read_gemm": (i, [i, i, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)     # AttributeError if the symbol is missing

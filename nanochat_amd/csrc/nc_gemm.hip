@@ -914,7 +914,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             which = (K % 128 == 0 && 8 * t256 >= 5 * cus) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
         }
         NC_CHECK_ARG(which == 5 || which == 8 || which == 9, "fp8_gemm: kernels 5, 8 and 9 take an e5m2 operand, not %d", force_kernel);
-        NcProfScope prof(1, 2.0 * M * N * K, s);
+        NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
         int rc = which == 5 ? launch_bl<128, 128, 2, 2, true, 1>(a, b, ep, M, N, K, s) : launch_dl<1>(a, b, ep, M, N, K, which == 9, s);
         if (rc) return rc;
         NC_CHECK_LAUNCH("fp8_gemm");
@@ -946,7 +946,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     }
     int rc = 0;
     if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 9, "fp8_gemm: unknown kernel selector %d", force_kernel);
-    NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s);
+    NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
         // split-K when the caller brought room for the partial sums, finished by a second small kernel

@@ -385,7 +385,7 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     g.A = a, g.a_amax = a_amax, g.inv_a = inv_a, g.B = b, g.inv_b = inv_b, g.segs = segs, g.out = out, g.out_kind = out_kind;
     g.softcap = softcap, g.ldc = ldc, g.out_amax = out_amax, g.partial_out = partials;
     g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
-    NcProfScope prof(1, 2.0 * M * N * K, s);
+    NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
     dim3 grid(nblk, ksplits), block(256);
     if (MB == 4) {
         if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<4, true>), grid, block, 0, s, g);

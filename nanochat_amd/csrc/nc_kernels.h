@@ -109,11 +109,11 @@ int nc_launch_sample(const float* logits, int B, int V, int ld, float temperatur
                      int64_t* out_ids, hipStream_t s);
 
 // ---- optional event timing (nc_profile.hip)
-int nc_prof_begin(int cls, double units, hipStream_t s);
+int nc_prof_begin(int cls, double units, hipStream_t s, int64_t tag = 0);
 void nc_prof_end(int slot, hipStream_t s);
 struct NcProfScope {
     int slot;
     hipStream_t s;
-    NcProfScope(int cls, double units, hipStream_t st) : slot(nc_prof_begin(cls, units, st)), s(st) {}
+    NcProfScope(int cls, double units, hipStream_t st, int64_t tag = 0) : slot(nc_prof_begin(cls, units, st, tag)), s(st) {}
     ~NcProfScope() { nc_prof_end(slot, s); }
 };
