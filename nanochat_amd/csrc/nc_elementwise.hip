@@ -372,6 +372,88 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(NcRopeSrc r, const
     dst[lane + 64] = f32_to_bf16(y2);
 }
 
+// The same for many tokens (prefill), reading the bf16 output of the q|k|v linear: eight lanes share a head, each holding eight
+// consecutive elements of its first half and the eight they pair with in the second half (element j rotates with j + 64), all
+// accesses 16 bytes wide; the mean of squares of the QK-norm is a sum over the 8 lanes.  Same rounding points as rope_head_finish.
+__global__ __launch_bounds__(256) void qkv_rope_append_vec_kernel(NcRopeSrc r, const int32_t* __restrict__ cache_seqlens,
+                                                                  bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+                                                                  bf16_t* __restrict__ q_out, int T, int H, int Hkv, int Tmax, int total_units) {
+    const int part = threadIdx.x & 7;
+    const int unit = blockIdx.x * 32 + (threadIdx.x >> 3);
+    const bool live = unit < total_units;
+    const int heads = H + 2 * Hkv;
+    const int u = live ? unit : total_units - 1;             // idle lanes shadow the last unit (the lane shuffles below need every lane)
+    const int token = u / heads, hh = u % heads;
+    const int b = token / T, t = token % T;
+    const int pos = cache_seqlens[b] + t;
+    const bf16_t* src = r.qkv + (size_t)token * r.ld_qkv + (size_t)hh * 128 + part * 8;
+    const uint4 xa = *(const uint4*)src, xb = *(const uint4*)(src + 64);
+    const uint32_t wa[4] = {xa.x, xa.y, xa.z, xa.w}, wb[4] = {xb.x, xb.y, xb.z, xb.w};
+    float x1[8], x2[8], o1[8], o2[8];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        x1[2 * j] = bf16_lo(wa[j]), x1[2 * j + 1] = bf16_hi(wa[j]);
+        x2[2 * j] = bf16_lo(wb[j]), x2[2 * j + 1] = bf16_hi(wb[j]);
+    }
+    if (hh < H + Hkv) {
+        const int rp = pos < r.rope_len ? (pos < 0 ? 0 : pos) : r.rope_len - 1;
+        const uint4 cv = *(const uint4*)(r.cos_t + (size_t)rp * 64 + part * 8), sv = *(const uint4*)(r.sin_t + (size_t)rp * 64 + part * 8);
+        const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w}, sw[4] = {sv.x, sv.y, sv.z, sv.w};
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float c = (e & 1) ? bf16_hi(cw[e >> 1]) : bf16_lo(cw[e >> 1]);
+            const float sn = (e & 1) ? bf16_hi(sw[e >> 1]) : bf16_lo(sw[e >> 1]);
+            o1[e] = rbf(rbf(x1[e] * c) + rbf(x2[e] * sn));
+            o2[e] = rbf(rbf(x1[e] * (-sn)) + rbf(x2[e] * c));
+            ss += o1[e] * o1[e] + o2[e] * o2[e];
+        }
+        ss += __shfl_xor(ss, 1);
+        ss += __shfl_xor(ss, 2);
+        ss += __shfl_xor(ss, 4);
+        const float rstd = 1.0f / sqrtf(ss / 128.0f + RMS_EPS);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            o1[e] = rbf(rbf(o1[e] * rstd) * 1.2f);
+            o2[e] = rbf(rbf(o2[e] * rstd) * 1.2f);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) o1[e] = x1[e], o2[e] = x2[e];
+        if (r.ve_table) {
+            const int hv = hh - H - Hkv;
+            int64_t tok = r.idx[token];
+            if (tok < 0 || tok >= r.vocab_rows) tok = 0;
+            const bf16_t* ve = r.ve_table + ((size_t)tok * Hkv + hv) * 128 + part * 8;
+            const uint4 va = *(const uint4*)ve, vb = *(const uint4*)(ve + 64);
+            const bf16_t* xg = r.xn + (size_t)token * r.ld_xn;
+            float dot = 0.f;
+#pragma unroll
+            for (int c = 0; c < 12; c++) dot += bf16_to_f32(xg[c]) * rbf(r.ve_gate_w[hv * 12 + c]);
+            const float gate = rbf(3.0f * rbf(sigmoidf_(rbf(dot))));
+            const uint32_t ea[4] = {va.x, va.y, va.z, va.w}, eb[4] = {vb.x, vb.y, vb.z, vb.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v1 = (e & 1) ? bf16_hi(ea[e >> 1]) : bf16_lo(ea[e >> 1]);
+                const float v2 = (e & 1) ? bf16_hi(eb[e >> 1]) : bf16_lo(eb[e >> 1]);
+                o1[e] = rbf(o1[e] + rbf(gate * v1));
+                o2[e] = rbf(o2[e] + rbf(gate * v2));
+            }
+        }
+    }
+    if (!live) return;
+    bf16_t* dst;
+    if (hh < H) dst = q_out + ((size_t)token * H + hh) * 128;
+    else {
+        if (pos < 0 || pos >= Tmax) return;
+        const bool is_k = hh < H + Hkv;
+        dst = (is_k ? k_cache : v_cache) + (((size_t)b * Tmax + pos) * Hkv + (is_k ? hh - H : hh - H - Hkv)) * 128;
+    }
+    dst += part * 8;
+    *(uint4*)dst = make_uint4(pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3]), pack_bf16(o1[4], o1[5]), pack_bf16(o1[6], o1[7]));
+    *(uint4*)(dst + 64) = make_uint4(pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3]), pack_bf16(o2[4], o2[5]), pack_bf16(o2[6], o2[7]));
+}
+
 // ------------------------------------------------------------------------------------------------
 // KVCache.prefill (nanochat/engine.py:123-137): the first n positions of every (layer, row) of a source cache go to
 // every row of a destination cache with a longer time axis; a one-row source is broadcast over the rows.  Each
@@ -516,9 +598,17 @@ static int launch_rope_impl(const bf16_t* qkv, int ld_qkv, NcPartialSrc pq, cons
     NC_CHECK_ARG(!ve_table || (ve_gate_w && xn && idx && ld_xn >= 12), "qkv_rope_append: value embedding needs gate weights, xn and idx");
     const int total = B * T * (H + 2 * Hkv);
     NcProfScope prof(3, 4.0 * total * 128, s);
-    const NcRopeSrc r{qkv, ld_qkv, pq, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin, rope_len, vocab_rows};
-    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, r, cache_seqlens, k_cache, v_cache, q_out, T, H,
-                       Hkv, Tmax, total);
+    const NcRopeSrc r{qkv, ld_qkv, pq, xn, ld_xn, idx, ve_table, ve_gate_w, cos, sin, rope_len, vocab_rows, nullptr, nullptr};
+    // many tokens of finished bf16 rows: the 16-byte-wide kernel (8 lanes per head); a few tokens, or rows still in split partials:
+    // one wave per head
+    const bool wide = qkv && total >= 2048 && ld_qkv % 8 == 0 && ld_xn % 8 == 0 &&
+                      ((((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)q_out | (uintptr_t)cos | (uintptr_t)sin | (uintptr_t)ve_table) & 15) == 0);
+    if (wide)
+        hipLaunchKernelGGL(qkv_rope_append_vec_kernel, dim3((total + 31) / 32), dim3(256), 0, s, r, cache_seqlens, k_cache, v_cache, q_out, T, H,
+                           Hkv, Tmax, total);
+    else
+        hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 3) / 4), dim3(256), 0, s, r, cache_seqlens, k_cache, v_cache, q_out, T, H,
+                           Hkv, Tmax, total);
     NC_CHECK_LAUNCH("qkv_rope_append");
     return 0;
 }

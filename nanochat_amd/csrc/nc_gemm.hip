@@ -471,12 +471,58 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bl_kernel(const uint8_t* 
     bl_epilogue<BM, BN, WGM, WGN, OUT_KIND>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
+
+// Per-process caches of what never changes while the process lives: the number of CUs of a device, and which kernels have had their
+// dynamic LDS limit raised on which device (hipFuncSetAttribute costs microseconds per call, a launch-bound caller notices).
+#include <atomic>
+namespace {
+constexpr int NC_GEMM_MAX_DEVICES = 64;
+int current_device() {
+    int dev = 0;
+    return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < NC_GEMM_MAX_DEVICES ? dev : 0;
+}
+int cu_count() {
+    static std::atomic<int> cached[NC_GEMM_MAX_DEVICES];
+    const int dev = current_device();
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        cus = 256;
+        (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+// slot: one per kernel family that asks for dynamic LDS (the attribute is set for the instantiation actually launched, so the
+// cache is keyed by the function pointer as well)
+hipError_t reserve_lds(const void* fn, int bytes) {
+    struct Entry {
+        std::atomic<const void*> fn;
+        std::atomic<int> bytes;
+    };
+    static Entry done[NC_GEMM_MAX_DEVICES][32];
+    const int dev = current_device();
+    for (auto& e : done[dev]) {
+        const void* f = e.fn.load(std::memory_order_acquire);
+        if (f == fn && e.bytes.load(std::memory_order_relaxed) >= bytes) return hipSuccess;
+        if (f == nullptr || f == fn) {
+            const hipError_t rc = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+            if (rc == hipSuccess) {
+                e.bytes.store(bytes, std::memory_order_relaxed);
+                e.fn.store(fn, std::memory_order_release);
+            }
+            return rc;
+        }
+    }
+    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);      // table full: just set it
+}
+}  // namespace
+
 template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE, int A_FMT, int OUT_KIND>
 static int launch_bl_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
     const void* fn = (const void*)gemm_bl_kernel<BM, BN, WGM, WGN, OUT_KIND, INTERLEAVE, A_FMT>;
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipError_t e = reserve_lds(fn, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     hipLaunchKernelGGL((gemm_bl_kernel<BM, BN, WGM, WGN, OUT_KIND, INTERLEAVE, A_FMT>), dim3(tiles_m * tiles_n), dim3(64 * WGM * WGN), lds_bytes, s, a, b,
                        ep, M, N, K, tiles_m, tiles_n);
@@ -847,7 +893,7 @@ static int launch_dl_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& 
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
     const size_t lds_bytes = 2 * 512 * 128 + (persistent ? 8 * 4096 : 0);
     const void* fn = persistent ? (const void*)gemm_dlp_kernel<A_FMT, RELU2> : (const void*)gemm_dl_kernel<A_FMT, RELU2>;
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipError_t e = reserve_lds(fn, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     if (persistent)
         hipLaunchKernelGGL((gemm_dlp_kernel<A_FMT, RELU2>), dim3(256), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m / 8, (N + 127) / 128);
@@ -874,7 +920,7 @@ template <int BM, int BN>
 static int launch_tile(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const size_t lds_bytes = 2 * (size_t)(BM + BN) * 128;
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, BN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipError_t e = reserve_lds((const void*)gemm_tile_kernel<BM, BN>, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     hipLaunchKernelGGL((gemm_tile_kernel<BM, BN>), dim3(tiles_m * tiles_n), dim3(256), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     return 0;
@@ -908,8 +954,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: e5m2 operands need M*K and N*K below 2^31");
         int which = force_kernel;
         if (which == 0) {
-            int dev = 0, cus = 256;
-            if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            const int cus = cu_count();
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             which = (K % 128 == 0 && 8 * t256 >= 5 * cus) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
         }
@@ -928,8 +973,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         if (M <= 128) which = 1;
         else if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31)) which = 4;   // past the 32-bit buffer offsets
         else {
-            int dev = 0, cus = 256;
-            if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            const int cus = cu_count();
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             const long rounds = (t256 + cus - 1) / cus;
             if (out_kind != 1 && K % 128 == 0 && 8 * t256 >= 5 * cus) {

@@ -82,6 +82,7 @@ def compute_window_sizes(config):
 
 class GPT(nn.Module):
     SOFTCAP = 15.0
+    WORKSPACE_CACHE_BYTES = 2 << 30       # step workspaces kept alive between calls (one per (batch, tokens) shape seen)
 
     def __init__(self, config, pad_vocab_size_to=64):
         super().__init__()
@@ -278,7 +279,9 @@ class GPT(nn.Module):
         ws = self._workspaces.get((B, T))
         if ws is None:
             nbytes = _lib.lib().nc_gpt_workspace_bytes(C.byref(md), B, T)
-            if len(self._workspaces) > 8:       # prefill lengths vary: keep the table small
+            # prefill lengths vary: the table is bounded by the bytes it holds, not by its entry count
+            held = sum(w.numel() for w in self._workspaces.values())
+            if held + nbytes > self.WORKSPACE_CACHE_BYTES:
                 self._workspaces.clear()
             ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
             self._workspaces[(B, T)] = ws

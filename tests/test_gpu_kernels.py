@@ -465,12 +465,12 @@ def test_float8linear_backward_matches_oracle(ops, B, K, N):
 
 
 # ================================================================== (4) row kernels
-def ulp_close(got, want, max_frac_off=0.002):
+def ulp_close(got, want, max_frac_off=0.002, max_ulp=1):
     """bf16 tensors equal except for rare one-ulp differences (fp32 summation order)."""
     gi = got.view(torch.int16).int()
     wi = want.view(torch.int16).int()
     diff = (gi - wi).abs()
-    assert diff.max().item() <= 1, diff.max().item()
+    assert diff.max().item() <= max_ulp, diff.max().item()
     assert (diff != 0).float().mean().item() <= max_frac_off, (diff != 0).float().mean().item()
 
 
@@ -543,18 +543,19 @@ def test_embed_norm_smear(ops, B, T, with_prev, E):
     ulp_close(got.cpu(), want, 0.01)
 
 
-@pytest.mark.parametrize("H,Hkv,T,with_ve", [(13, 13, 1, True), (13, 13, 1, False), (4, 2, 5, True), (16, 4, 1, True)])
+@pytest.mark.parametrize("H,Hkv,T,with_ve", [(13, 13, 1, True), (13, 13, 1, False), (4, 2, 5, True), (16, 4, 1, True),
+                                             (13, 13, 60, True), (16, 4, 64, True), (5, 5, 150, False)])    # many tokens: the 16-byte-wide kernel
 def test_qkv_rope_append(ops, H, Hkv, T, with_ve):
     say(f"qkv_rope_append H={H} Hkv={Hkv} T={T} ve={with_ve}")
     g = torch.Generator().manual_seed(2)
-    B, Tmax, V = 3, 40, 300
+    B, Tmax, V = 3, (40 if T <= 5 else 200), 300
     E = H * 128
     qkv = torch.randn(B, T, (H + 2 * Hkv) * 128, generator=g).bfloat16()
     xn = torch.randn(B, T, E, generator=g).bfloat16()
     idx = torch.randint(0, V, (B, T), generator=g)
     ve_table = (torch.randn(V, Hkv * 128, generator=g) * 0.5).bfloat16() if with_ve else None
     gate_w = (torch.rand(Hkv, 12, generator=g) - 0.5) if with_ve else None
-    cos, sin = gpt_ref.rotary_tables(64, 128, torch.bfloat16)
+    cos, sin = gpt_ref.rotary_tables(256, 128, torch.bfloat16)
     seq = torch.tensor([7, 0, 30], dtype=torch.int32)
     kc = torch.randn(B, Tmax, Hkv, 128, generator=g).bfloat16()
     vc = torch.randn(B, Tmax, Hkv, 128, generator=g).bfloat16()
@@ -577,8 +578,10 @@ def test_qkv_rope_append(ops, H, Hkv, T, with_ve):
     kd, vd = kc.to(DEV), vc.to(DEV)
     got_q = ops.qkv_rope_append(qkv.to(DEV), xn.to(DEV), idx.to(DEV), ve_table.to(DEV) if with_ve else None,
                                 gate_w.to(DEV) if with_ve else None, cos.to(DEV), sin.to(DEV), seq.to(DEV), kd, vd, H, Hkv)
-    ulp_close(got_q.cpu(), q, 0.01)
-    ulp_close(kd.cpu(), kc_want, 0.01)
+    # q and k end with `rounded(x * rstd) * 1.2, rounded`: where the sum of squares differs in its last fp32 bit and flips the first
+    # rounding by one step, the gain of 1.2 can spread that over two steps of the result (a handful of elements in a million)
+    ulp_close(got_q.cpu(), q, 0.01, max_ulp=2)
+    ulp_close(kd.cpu(), kc_want, 0.01, max_ulp=2)
     ulp_close(vd.cpu(), vc_want, 0.01)
 
 
