@@ -44,6 +44,17 @@ int nc_fp8_quantize_tensorwise_as(const void* x, int x_dtype, int64_t n, int fp8
 int nc_fp8_encode_with_scale(const uint16_t* x, int64_t n, float scale, int fp8_format, uint8_t* out, int encoder,
                              nc_stream_t stream);
 
+/* The same quantization in ONE launch where the tensor allows it (bf16 input, n a multiple of 16, up to roughly 30 million
+ * elements: what the registers of the workgroups resident on the chip hold): every element is read from memory once, the
+ * workgroups meet on the tensor's amax, the payload is converted from registers.  Other tensors take the two passes of
+ * nc_fp8_quantize_tensorwise_as; results are bit-identical either way.  state: nc_fp8_quantize_state_bytes() bytes, 128-byte
+ * aligned, ALL ZERO before the first call with it; every call leaves it all zero (word 320 excepted, which is scratch),
+ * so one allocation serves all calls that do not overlap in time.  If the on-chip meeting ever timed out (it cannot while the
+ * device runs this library's kernels alone) the scale comes out as NaN and word 257 of the state stays set. */
+size_t nc_fp8_quantize_state_bytes(void);
+int nc_fp8_quantize_tensorwise_fused(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
+                                     float* inv_scale_out, void* state, int encoder, nc_stream_t stream);
+
 /* dst[cols][rows] = transpose of the fp8 payload src[rows][cols]: the memory rearrangement of _to_col_major and
  * .t().contiguous() at nanochat/fp8.py:110-118,169,181-182 (the backward GEMMs want the summed index contiguous in
  * both operands).  rows and cols multiples of 16, pointers 16-byte aligned. */

@@ -5,6 +5,7 @@
 // (one fp32 rounding); clamp to +-448; round to nearest even into OCP e4m3fn; inv = 1.0f / scale
 // with an IEEE divide.  HBM traffic: the amax pass reads the tensor once, the convert pass reads
 // it again (normally from L2 / infinity cache) and writes one byte per element.
+#include <atomic>
 #include "nc_common.h"
 #include "nc_kernels.h"
 
@@ -171,6 +172,196 @@ int nc_launch_quantize(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* 
     else launch_quantize_fmt<1>(x, x_dtype, n, out, scale_out, inv_out, amax_ws, encoder, g1, g2, s);
     NC_CHECK_LAUNCH("fp8_quantize");
     return 0;
+}
+
+// ---------------------------------------------------------------- one launch: amax, grid-wide meeting, convert
+// For tensors that fit in the registers of the workgroups the chip can hold at once (up to ~30 M bf16 elements): every thread loads
+// its share once and keeps it, the workgroups meet on the tensor's amax, and the payload is converted from registers.  HBM sees the
+// algorithmic 3 bytes per element and the three launches (clear, amax, convert) become one.
+//
+// The meeting needs every workgroup of the grid to be resident, which holds because the grid is sized to what the device can hold of
+// this kernel alone (hipOccupancyMaxActiveBlocksPerMultiprocessor x CUs): a workgroup that has to wait for a slot taken by some other
+// kernel gets it when that kernel ends, and nothing the other kernel does waits for this one.  The wait is bounded all the same: a
+// workgroup that gives up marks the state's error word and the scale comes out as NaN instead of the kernel hanging.
+//
+// state: all zero before the first call, left all zero by every call (the last workgroup to leave clears it).  Slot k
+// (k = blockIdx.x % 8) lives on its own 128-byte line: word 0 the running maximum, word 1 the arrivals (one address would
+// serialize the grid's atomics at ~6 ns each).  Line 8: departures, the sticky error mark, slots reported.  Line 9: the flag
+// that the last reported slot raises and one lane per workgroup watches.  Line 10, word 0: scratch of the two-pass path.
+#define QF_SLOTS 8
+#define QF_STRIDE 32
+#define QF_DEPART (QF_SLOTS * QF_STRIDE)
+#define QF_ERROR (QF_SLOTS * QF_STRIDE + 1)
+#define QF_SLOTS_DONE (QF_SLOTS * QF_STRIDE + 2)
+#define QF_FLAG ((QF_SLOTS + 1) * QF_STRIDE)
+#define QF_SCRATCH ((QF_SLOTS + 2) * QF_STRIDE)
+template <int FMT, bool HW_CVT, int G>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void quantize_fused_kernel(const bf16_t* __restrict__ x, int64_t n16, uint8_t* __restrict__ out,
+                                                             float* __restrict__ scale_out, float* __restrict__ inv_out,
+                                                             uint32_t* __restrict__ state, uint32_t spin_limit) {
+    __shared__ uint32_t red[4];
+    __shared__ uint32_t amax_sh;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    // group g of this thread: 16 elements (32 bytes in, 16 bytes out) at group index (blockIdx.x * G + g) * 256 + tid
+    uint4 ra[G], rb[G];
+    uint32_t m = 0;
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        int64_t idx = ((int64_t)blockIdx.x * G + g) * 256 + tid;
+        idx = idx < n16 ? idx : n16 - 1;                   // a slot past the end re-reads the last group (its maximum is already counted)
+        const v4i* p = (const v4i*)x + idx * 2;
+        const v4i a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
+        ra[g] = make_uint4((uint32_t)a[0], (uint32_t)a[1], (uint32_t)a[2], (uint32_t)a[3]);
+        rb[g] = make_uint4((uint32_t)b[0], (uint32_t)b[1], (uint32_t)b[2], (uint32_t)b[3]);
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const uint32_t wd[8] = {ra[g].x, ra[g].y, ra[g].z, ra[g].w, rb[g].x, rb[g].y, rb[g].z, rb[g].w};
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t lo = (wd[j] & 0x7fffu) << 16, hi = wd[j] & 0x7fff0000u;
+            m = m > lo ? m : lo;
+            m = m > hi ? m : hi;
+        }
+    }
+    m = wave_max_u32(m);
+    if (lane == 0) red[w] = m;
+    __syncthreads();
+    if (w == 0) {
+        const uint32_t k = blockIdx.x % QF_SLOTS;
+        uint32_t* slot = state + k * QF_STRIDE;
+        bool gave_up = false;
+        if (lane == 0) {
+            uint32_t t = red[0];
+            for (int i = 1; i < 4; i++) t = t > red[i] ? t : red[i];
+            // the maximum first, its acknowledgement awaited (a returning atomic), then the arrival: whoever sees all arrivals sees all maxima
+            const uint32_t before = __hip_atomic_fetch_max(slot, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("" ::"v"(before) : "memory");
+            const uint32_t in_slot = (gridDim.x - k + QF_SLOTS - 1) / QF_SLOTS;       // workgroups that use this slot
+            const uint32_t used = gridDim.x < QF_SLOTS ? gridDim.x : QF_SLOTS;        // slots in use
+            // the last arrival of a slot reports the slot; the last slot to be reported raises the flag everyone watches
+            if (__hip_atomic_fetch_add(slot + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_slot - 1) {
+                if (__hip_atomic_fetch_add(state + QF_SLOTS_DONE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == used - 1)
+                    __hip_atomic_store(state + QF_FLAG, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            uint32_t spins = 0;
+            while (__hip_atomic_load(state + QF_FLAG, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+                if (++spins > spin_limit) {
+                    gave_up = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(8);
+            }
+        }
+        gave_up = __builtin_amdgcn_readfirstlane((int)gave_up) != 0;
+        uint32_t am = lane < QF_SLOTS ? __hip_atomic_load(state + lane * QF_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+        am = wave_max_u32(am);
+        if (gave_up) {
+            am = 0x7fc00000u;                                // NaN: the scale and the payload come out as NaN
+            if (lane == 0) __hip_atomic_store(state + QF_ERROR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0) {
+            amax_sh = am;
+            // leave; the last one out puts the state back to zero for the next call (everyone has read what it needs by now)
+            const uint32_t gone = __hip_atomic_fetch_add(state + QF_DEPART, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (gone == gridDim.x - 1 && !gave_up) {
+                for (int i = 0; i < QF_SLOTS; i++) {
+                    __hip_atomic_store(state + i * QF_STRIDE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(state + i * QF_STRIDE + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                __hip_atomic_store(state + QF_SLOTS_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(state + QF_FLAG, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(state + QF_DEPART, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __syncthreads();
+    const float scale = scale_from_amax(__uint_as_float(amax_sh), fp8_max<FMT>());
+    if (blockIdx.x == 0 && tid == 0) {
+        if (scale_out) *scale_out = scale;
+        *inv_out = 1.0f / scale;
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const int64_t idx = ((int64_t)blockIdx.x * G + g) * 256 + tid;
+        if (idx >= n16) continue;
+        const uint32_t wd[8] = {ra[g].x, ra[g].y, ra[g].z, ra[g].w, rb[g].x, rb[g].y, rb[g].z, rb[g].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float y0 = fp8_clamp<FMT>(bf16_lo(wd[2 * j]) * scale), y1 = fp8_clamp<FMT>(bf16_hi(wd[2 * j]) * scale);
+            const float y2 = fp8_clamp<FMT>(bf16_lo(wd[2 * j + 1]) * scale), y3 = fp8_clamp<FMT>(bf16_hi(wd[2 * j + 1]) * scale);
+            o[j] = fp8_pack4<FMT, HW_CVT>(y0, y1, y2, y3);
+        }
+        __builtin_nontemporal_store(v4i{(int)o[0], (int)o[1], (int)o[2], (int)o[3]}, (v4i*)out + idx);
+    }
+}
+
+// how many workgroups of quantize_fused_kernel<.., G> the current device holds at once (0: unknown, do not use the kernel)
+template <int FMT, bool HW_CVT, int G>
+static int fused_capacity() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    int cap = cached[dev].load(std::memory_order_relaxed);
+    if (cap == 0) {
+        int per_cu = 0, cus = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quantize_fused_kernel<FMT, HW_CVT, G>, 256, 0) != hipSuccess) per_cu = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
+        cap = per_cu * cus;
+        if (cap <= 0) cap = -1;
+        cached[dev].store(cap, std::memory_order_relaxed);
+    }
+    return cap > 0 ? cap : 0;
+}
+
+template <int FMT, bool HW_CVT, int G>
+static bool try_fused(const bf16_t* x, int64_t n16, uint8_t* out, float* scale_out, float* inv_out, uint32_t* state, hipStream_t s) {
+    const int64_t blocks = (n16 + 256 * (int64_t)G - 1) / (256 * (int64_t)G);
+    // half of the capacity: two such grids launched on two streams at the same time still both fit (callers that overlap more
+    // than that on one GPU could starve each other's meeting until the bounded wait gives up)
+    if (blocks > (int64_t)fused_capacity<FMT, HW_CVT, G>() / 2) return false;
+    hipLaunchKernelGGL((quantize_fused_kernel<FMT, HW_CVT, G>), dim3((unsigned)blocks), dim3(256), 0, s, x, n16, out, scale_out, inv_out, state,
+                       1u << 22);       // ~4 M polls of a few hundred ns each before a workgroup gives up
+    return true;
+}
+
+template <int FMT, bool HW_CVT>
+static bool try_fused_any(const bf16_t* x, int64_t n16, uint8_t* out, float* scale_out, float* inv_out, uint32_t* state, hipStream_t s) {
+    // The largest share per thread that still leaves a workgroup for every other CU: few workgroups keep the meeting cheap (its atomics and
+    // its pollers share a handful of memory lines), long shares keep many loads in flight per thread.
+    const int64_t per_wg = 128;          // (half of the CUs at least)
+    if (n16 >= 8 * per_wg * 256 && try_fused<FMT, HW_CVT, 8>(x, n16, out, scale_out, inv_out, state, s)) return true;
+    if (n16 >= 4 * per_wg * 256 && try_fused<FMT, HW_CVT, 4>(x, n16, out, scale_out, inv_out, state, s)) return true;
+    if (n16 >= 2 * per_wg * 256 && try_fused<FMT, HW_CVT, 2>(x, n16, out, scale_out, inv_out, state, s)) return true;
+    return try_fused<FMT, HW_CVT, 1>(x, n16, out, scale_out, inv_out, state, s) || try_fused<FMT, HW_CVT, 2>(x, n16, out, scale_out, inv_out, state, s) ||
+           try_fused<FMT, HW_CVT, 4>(x, n16, out, scale_out, inv_out, state, s) || try_fused<FMT, HW_CVT, 8>(x, n16, out, scale_out, inv_out, state, s);
+}
+
+// state: NC_QUANTIZE_STATE_BYTES (1 KB + 16).  Tensors the one-launch kernel does not take (fp32 input, an element count that is
+// not a multiple of 16, more elements than fit on the chip) go through the two passes, with the state's last word as their scratch.
+int nc_launch_quantize_fused(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* out, float* scale_out, float* inv_out,
+                             uint32_t* state, int encoder, hipStream_t s) {
+    NC_CHECK_ARG(n >= 0, "fp8_quantize: negative element count");
+    NC_CHECK_ARG(inv_out && state && (n == 0 || (x && out)), "fp8_quantize: null pointer");
+    NC_CHECK_ARG(x_dtype == 0 || x_dtype == 1, "fp8_quantize: dtype must be 0 (bf16) or 1 (fp32)");
+    NC_CHECK_ARG(fmt == 0 || fmt == 1, "fp8_quantize: format must be 0 (e4m3fn) or 1 (e5m2)");
+    NC_CHECK_ARG(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)state & 127) == 0,
+                 "fp8_quantize: pointers must be 16-byte aligned (the state 128-byte aligned)");
+    if (x_dtype == 0 && n >= 16 && n % 16 == 0) {
+        NcProfScope prof(2, 3.0 * n, s);
+        const bf16_t* xb = (const bf16_t*)x;
+        bool done;
+        if (fmt == 0) done = encoder == 0 ? try_fused_any<0, true>(xb, n / 16, out, scale_out, inv_out, state, s)
+                                          : try_fused_any<0, false>(xb, n / 16, out, scale_out, inv_out, state, s);
+        else done = encoder == 0 ? try_fused_any<1, true>(xb, n / 16, out, scale_out, inv_out, state, s)
+                                 : try_fused_any<1, false>(xb, n / 16, out, scale_out, inv_out, state, s);
+        if (done) {
+            NC_CHECK_LAUNCH("fp8_quantize");
+            return 0;
+        }
+    }
+    return nc_launch_quantize(x, x_dtype, n, fmt, out, scale_out, inv_out, state + QF_SCRATCH, encoder, s);
 }
 
 // Convert only, with amax already reduced into amax_ws by a producer kernel.

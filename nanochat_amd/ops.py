@@ -26,12 +26,15 @@ def _need_cuda(*tensors):
             raise RuntimeError("nanochat_amd ops run on the GPU only (got a CPU tensor); there is no CPU fallback")
 
 
-def _amax_slot(device):
-    """One uint32 of scratch per device and stream for quantize calls that bring no workspace."""
+def _quantize_state(device):
+    """The quantizer's state block (zero before first use, left zero by every call), one per device and stream."""
     key = (device.index, torch.cuda.current_stream().cuda_stream)
     t = _SCRATCH.get(key)
     if t is None:
-        t = torch.zeros(64, dtype=torch.int32, device=device)
+        nbytes = _lib.lib().nc_fp8_quantize_state_bytes()
+        raw = torch.zeros(nbytes + 128, dtype=torch.uint8, device=device)
+        off = (-raw.data_ptr()) % 128
+        t = raw[off:off + nbytes]
         _SCRATCH[key] = t
     return t
 
@@ -52,10 +55,10 @@ def fp8_quantize(x, encoder=0, fp8_dtype=torch.float8_e4m3fn):
     x = x.contiguous()
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     scales = torch.empty(2, dtype=torch.float32, device=x.device)
-    ws = _amax_slot(x.device)
-    rc = _lib.lib().nc_fp8_quantize_tensorwise_as(_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _FP8_FORMATS[fp8_dtype],
-                                                  _ptr(out), C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4),
-                                                  _ptr(ws), encoder, _stream())
+    state = _quantize_state(x.device)
+    rc = _lib.lib().nc_fp8_quantize_tensorwise_fused(_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _FP8_FORMATS[fp8_dtype],
+                                                     _ptr(out), C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4),
+                                                     _ptr(state), encoder, _stream())
     _lib.check(rc)
     return out.view(fp8_dtype), scales[1], scales[0]
 

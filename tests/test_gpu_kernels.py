@@ -90,6 +90,46 @@ def test_quantize_matches_oracle_bitwise(ops, shape, dtype):
     assert torch.equal(payload.view(torch.uint8).cpu(), want_p.view(torch.uint8))
 
 
+def test_quantize_one_launch_form_against_the_two_passes_and_its_state(ops):
+    """The one-launch quantizer (every element read once, the workgroups meet on the amax) against the two-pass entry, bit for
+    bit, on back-to-back calls of different sizes sharing one state block, which every call must leave all zero."""
+    say("quantize: one launch vs two passes")
+    import ctypes as C
+    from nanochat_amd import _lib
+    lib = _lib.lib()
+    nbytes = lib.nc_fp8_quantize_state_bytes()
+    raw = torch.zeros(nbytes + 128, dtype=torch.uint8, device=DEV)
+    off = (-raw.data_ptr()) % 128
+    state = raw[off:off + nbytes]
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    for shape, fmt in (((8192, 1664), 0), ((64, 6656), 0), ((16,), 0), ((4096, 4992), 1), ((8192, 6656), 0), ((48, 16), 1), ((333, 77), 0)):
+        x = torch.randn(shape, device=DEV, generator=g)
+        x = torch.where(torch.rand(shape, device=DEV, generator=g) < 0.001, x * 20, x).bfloat16()
+        outs = []
+        for entry in ("fused", "two_pass"):
+            out = torch.empty(shape, dtype=torch.uint8, device=DEV)
+            sc = torch.zeros(2, dtype=torch.float32, device=DEV)
+            if entry == "fused":
+                rc = lib.nc_fp8_quantize_tensorwise_fused(x.data_ptr(), 0, x.numel(), fmt, out.data_ptr(), sc.data_ptr(), sc.data_ptr() + 4,
+                                                          state.data_ptr(), 0, stream)
+            else:
+                ws = torch.zeros(1, dtype=torch.int32, device=DEV)
+                rc = lib.nc_fp8_quantize_tensorwise_as(x.data_ptr(), 0, x.numel(), fmt, out.data_ptr(), sc.data_ptr(), sc.data_ptr() + 4,
+                                                       ws.data_ptr(), 0, stream)
+            _lib.check(rc)
+            outs.append((out, sc))
+        assert torch.equal(outs[0][0], outs[1][0]), shape
+        assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32)), shape
+        words = state.view(torch.int32).cpu()
+        assert not words[:320].any(), f"{shape}: the state was not left zero: {words[:320].nonzero().flatten().tolist()}"
+    # a NaN anywhere makes the amax and with it the scales NaN, as in the reference (abs().max() propagates it)
+    x = torch.randn(4096, 64, device=DEV, generator=g).bfloat16()
+    x[1234, 5] = float("nan")
+    payload, inv, scale = ops.fp8_quantize(x)
+    assert torch.isnan(scale).item() and torch.isnan(inv).item()
+
+
 def test_quantize_zero_tensor_and_invariants(ops):
     say("quantize zeros / sign symmetry")
     p, inv, s = ops.fp8_quantize(torch.zeros(4096, dtype=torch.bfloat16, device=DEV))
