@@ -8,44 +8,91 @@
 //   S^T = K . Q^T   (v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = the wave's 32 queries held in registers):
 //                   a lane ends up with 16 scores of ONE query (column lane % 32), so the running max / sum of the
 //                   online softmax are per-lane scalars plus one exchange with lane ^ 32;
-//   O^T = V^T . P^T (same instruction, A = V^T from LDS, B = P^T): the B operand is exactly the S^T accumulator
-//                   registers converted to bf16 (the key order inside a 16-key chunk is the accumulator's row order,
-//                   and V^T is read in that order), and the output columns are again the lane's own query, so the
-//                   softmax rescale is a per-lane multiply.
-// A workgroup is 4 waves x 32 queries of one (row, head); keys go through LDS in blocks of 32: K as [key][d]
-// (rows padded to 272 B), V transposed to [d][key] (rows padded to 72 B) while it is staged.  The loads of the next
-// block are in flight while the current one is multiplied.
+//   O^T = V^T . P^T (same instruction, A = V^T, B = P^T): the B operand is exactly the S^T accumulator registers converted to
+//                   bf16 (the key order inside a 16-key chunk is the accumulator's row order, and V^T is read in that order),
+//                   and the output columns are again the lane's own query, so the softmax rescale is a per-lane multiply.
+// Keys and values go through LDS in blocks of 32, both as [key][d] (K rows padded to 272 B, V rows to 320 B); the V^T operand
+// comes out of LDS through the transposing read (ds_read_b64_tr_b16), so nothing is shuffled while staging.  The loads of the
+// next block are in flight while the current one is multiplied.
 #include "nc_common.h"
 #include "nc_kernels.h"
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s* lds_v4s_t;
+typedef __attribute__((address_space(3))) uint8_t* lds_u8_t;
 
 #define PF_KPITCH 272          // bytes per K row in LDS (256 + 16)
-#define PF_VPITCH 72           // bytes per V^T row in LDS (64 + 8)
-#define PF_NEG (-1.0e30f)
+#define PF_VPITCH 320          // bytes per V row in LDS (256 + 64: four consecutive keys start 16 banks apart)
+#define PF_KBYTES (32 * PF_KPITCH)
+#define PF_VBYTES (32 * PF_VPITCH)
+#define PF_MASKED (-1.0e30f)   // raw score of a key that the query does not see
+#ifndef PF_OPT_COND
+#define PF_OPT_COND 1
+#endif
+#ifndef PF_OPT_XCD
+#define PF_OPT_XCD 1
+#endif
+#ifndef PF_OPT_WAVES
+#define PF_OPT_WAVES 1
+#endif
+#if PF_OPT_WAVES
+#define PF_WAVES_ATTR __attribute__((amdgpu_waves_per_eu(2, 2)))
+#else
+#define PF_WAVES_ATTR
+#endif
+#ifndef PF_LAZY
+#define PF_LAZY 6.0f
+#endif
+#define PF_M_FLOOR (-1.0e20f)  // running maximum (scaled units) before any visible key: far above PF_MASKED * scale, far below any score
 
 __device__ __forceinline__ v8bf as_v8bf(uint4 v) { return __builtin_bit_cast(v8bf, v); }
 
-// GS = query heads of one kv head that share a workgroup (1, 2 or 4): wave w serves head (w % GS) of the group and the (w / GS)-th
-// block of 32 queries, so a workgroup covers 128 / GS queries of GS heads and the keys and values it stages are used by all of them.
-// Keys go through LDS 64 at a time (two sub-blocks of 32, each laid out and multiplied as described above): one pair of barriers and
-// one round of loads in flight per 64 keys.  A wave skips a sub-block that none of its queries can see (past the causal diagonal, or
-// wholly before the window of its first query).  Tiles are handed out from the end of the sequence, longest key ranges first.
-template <int GS>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+// GS = query heads of one kv head that share a workgroup (1, 2 or 4), KS = waves that share one block of 32 queries and split
+// its keys between them (1 or 2), GS * KS <= 4.  Wave w serves head (w % GS) of the group, key share (w / GS) % KS and the
+// (w / (GS * KS))-th block of 32 queries, so a workgroup covers 128 / (GS * KS) queries of GS heads and the keys and values it
+// stages are used by all of its waves.  Keys go through LDS 64 at a time (two sub-blocks of 32, each laid out and multiplied as
+// described above): one pair of barriers and one round of loads in flight per 64 keys.  With KS = 1 a wave works through both
+// sub-blocks, with KS = 2 through one of them, and the two partial softmax states of a query block are merged through LDS at the end:
+// that doubles the number of workgroups when a launch has too few of them to fill the chip (a single long prompt).
+// A wave skips a sub-block that none of its queries can see (past the causal diagonal, or wholly before the window of its first
+// query), and a sub-block that all of its queries see in full takes the path without the mask arithmetic.  The running maximum only
+// triggers a rescale of the 64 output accumulators when it moved for some lane of the wave.  Tiles are handed out from the end of the
+// sequence, longest key ranges first.
+template <int GS, int KS>
+__global__ __launch_bounds__(256) PF_WAVES_ATTR void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                                                            const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
                                                            uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax) {
-    constexpr int QT = 128 / GS;                               // queries per workgroup
-    __shared__ __align__(16) uint8_t lds_k[2][32 * PF_KPITCH];
-    __shared__ __align__(16) uint8_t lds_v[2][128 * PF_VPITCH];
+    constexpr int QT = 128 / (GS * KS);                        // queries per workgroup
+    __shared__ __align__(16) uint8_t lds[2 * PF_KBYTES + 2 * PF_VBYTES];
     __shared__ float red[4];
+    uint8_t* const lds_k = lds;
+    uint8_t* const lds_v = lds + 2 * PF_KBYTES;
+    const lds_u8_t lds_v3 = (lds_u8_t)lds + 2 * PF_KBYTES;     // the same place as an LDS address, for the transposing reads
     const int G = H / Hkv, parts = G / GS;                     // workgroups per kv head along the head axis
-    const int qb0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * QT, hk = blockIdx.y / parts, b = blockIdx.z;
+    // Workgroups go to the eight XCDs in turn by their linear index, and each XCD has an L2 of its own: the (tile, head) pairs of a
+    // row are numbered so that one XCD gets a contiguous run of them, i.e. all tiles of a few heads, and the keys and values of a head
+    // are then read into one L2 instead of all eight.  Within a head the tiles come from the end of the sequence, longest first.
+    const int b = blockIdx.z;
+    int qb0, hy;
+    {
+        const int nx = gridDim.x, total = nx * (int)gridDim.y, lid = (int)blockIdx.x + nx * (int)blockIdx.y;
+#if PF_OPT_XCD
+        const int xcd = lid & 7, slot = lid >> 3;
+        const int unit = xcd * (total >> 3) + min(xcd, total & 7) + slot;
+#else
+        const int unit = lid;
+#endif
+        hy = unit / nx;
+        qb0 = (nx - 1 - unit % nx) * QT;
+    }
+    const int hk = hy / parts;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int h = hk * G + (blockIdx.y % parts) * GS + wave % GS;
-    const int qw0 = qb0 + (wave / GS) * 32;                    // first query of this wave
+    const int h = hk * G + (hy % parts) * GS + wave % GS;
+    const int ks = (wave / GS) % KS;                           // which of the KS key shares this wave takes
+    const int qw0 = qb0 + (wave / (GS * KS)) * 32;             // first query of this wave
     const int col = lane & 31, hl = lane >> 5;
 
     int pos0 = cache_seqlens[b];
@@ -55,9 +102,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     const bool q_ok = t < T;
     const int qpos = pos0 + (q_ok ? t : T - 1);
     const int q_lo = window_left < 0 ? 0 : max(0, qpos - window_left);
-    // what the wave as a whole can see: keys [w_lo, w_hi]
-    const int w_hi = pos0 + min(qw0 + 31, T - 1);
-    const int w_lo = window_left < 0 ? 0 : max(0, pos0 + min(qw0, T - 1) - window_left);
 
     // key range of the workgroup
     const int t_last = min(qb0 + QT - 1, T - 1);
@@ -66,6 +110,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     int k_lo = window_left < 0 ? 0 : pos0 + qb0 - window_left;
     if (k_lo < 0) k_lo = 0;
     const int kb_first = k_lo & ~63;
+
+    // what the wave as a whole can see: keys [w_lo, w_hi]; what every one of its queries sees in full: keys [f_lo, f_hi]
+    const int qpos_first = pos0 + min(qw0, T - 1), qpos_last = pos0 + min(qw0 + 31, T - 1);
+    const int w_hi = qpos_last;
+    const int w_lo = window_left < 0 ? 0 : max(0, qpos_first - window_left);
+    const int f_hi = min(qpos_first, k_hi);
+    const int f_lo = window_left < 0 ? 0 : max(0, qpos_last - window_left);
 
     // Q fragments: B operand of K.Q^T, lane = (query col, d half hl): Q[query][16c + 8hl .. +7]
     v8bf qf[8];
@@ -80,90 +131,113 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[dt][r] = 0.f;
-    float m_run = PF_NEG, l_run = 0.f;
+    float m_run = PF_M_FLOOR, l_run = 0.f;
     const float sc = 1.4426950408889634f * 0.08838834764831845f;     // log2(e) / sqrt(128)
 
     // staging: thread = (16-byte chunk ch of a key, key pair kp): keys 2kp, 2kp+1 of each 32-key sub-block
     const int ch = tid & 15, kp = tid >> 4;
-    const size_t key_stride = (size_t)Hkv * 128;
+    const uint32_t key_stride = (uint32_t)Hkv * 128;
     const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + ch * 8;
     const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + ch * 8;
     uint4 rk[2][2], rv[2][2];
+    // Load j (0..7) of the 64 keys from kb on: sub-block j / 4, key 2 kp + (j / 2) % 2 of it, K for even j and V for odd j.  Keys past
+    // the end of the workgroup's range are read from its last key instead (no query gives them any weight), so no load is conditional.
+    auto fetch_one = [&](int kb, int j) {
+        const int sb = j >> 2, i = (j >> 1) & 1;
+#if PF_OPT_COND
+        const int key = kb + 32 * sb + 2 * kp + i;
+        const bool ok = key <= k_hi;
+        const uint32_t off = (uint32_t)key * key_stride;
+        if (j & 1) rv[sb][i] = ok ? *(const uint4*)(vbase + off) : make_uint4(0, 0, 0, 0);
+        else rk[sb][i] = ok ? *(const uint4*)(kbase + off) : make_uint4(0, 0, 0, 0);
+#else
+        const uint32_t off = (uint32_t)min(kb + 32 * sb + 2 * kp + i, k_hi) * key_stride;      // (one row's cache fits 32 bits: checked at launch)
+        if (j & 1) rv[sb][i] = *(const uint4*)(vbase + off);
+        else rk[sb][i] = *(const uint4*)(kbase + off);
+#endif
+    };
     auto fetch = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) fetch_one(kb, j);
+    };
+    auto stage = [&]() {
 #pragma unroll
         for (int sb = 0; sb < 2; sb++)
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                const int key = kb + 32 * sb + 2 * kp + i;
-                const bool ok = key <= k_hi;
-                rk[sb][i] = ok ? *(const uint4*)(kbase + (size_t)key * key_stride) : make_uint4(0, 0, 0, 0);
-                rv[sb][i] = ok ? *(const uint4*)(vbase + (size_t)key * key_stride) : make_uint4(0, 0, 0, 0);
+                *(uint4*)(lds_k + sb * PF_KBYTES + (2 * kp + i) * PF_KPITCH + ch * 16) = rk[sb][i];
+                *(uint4*)(lds_v + sb * PF_VBYTES + (2 * kp + i) * PF_VPITCH + ch * 16) = rv[sb][i];
             }
     };
-    auto stage = [&]() {
-#pragma unroll
-        for (int sb = 0; sb < 2; sb++) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) *(uint4*)(lds_k[sb] + (2 * kp + i) * PF_KPITCH + ch * 16) = rk[sb][i];
-            // V^T[d = 8ch + e][keys 2kp, 2kp+1] as one dword per e
-            const uint32_t a[4] = {rv[sb][0].x, rv[sb][0].y, rv[sb][0].z, rv[sb][0].w}, c[4] = {rv[sb][1].x, rv[sb][1].y, rv[sb][1].z, rv[sb][1].w};
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint32_t lo = (e & 1) ? (a[e >> 1] >> 16) : (a[e >> 1] & 0xffffu);
-                const uint32_t hi = (e & 1) ? (c[e >> 1] >> 16) : (c[e >> 1] & 0xffffu);
-                *(uint32_t*)(lds_v[sb] + (8 * ch + e) * PF_VPITCH + 4 * kp) = lo | (hi << 16);
-            }
-        }
-    };
-    // one sub-block of 32 keys starting at kb, staged in slot sb
-    auto sub_block = [&](int kb, int sb) {
+    // Transposed read of V (ds_read_b64_tr_b16): in every group of 16 lanes, lane r points at four consecutive d of key r / 4
+    // (d offset 4 (r % 4)), and lane i receives element d = i of the 16 the group covers, for those four keys.  The groups are
+    // (d half of the 32-row block, key half hl), which makes the result the A operand of the second product as laid out below.
+    const uint32_t vtr_off = (uint32_t)(4 * hl + ((lane & 15) >> 2)) * PF_VPITCH + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+    // one sub-block of 32 keys starting at kb, staged in slot sb; MASKED = some (query, key) pair of it is not visible
+    auto sub_block = [&](int kb, int sb, bool masked) {
         // ---- S^T = K . Q^T : rows = keys kb + 8*(r/4) + 4*hl + r%4, column = this lane's query
         v16f s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
+        const uint8_t* kt = lds_k + sb * PF_KBYTES;
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            const v8bf kf = as_v8bf(*(const uint4*)(lds_k[sb] + col * PF_KPITCH + (16 * c + 8 * hl) * 2));
+            const v8bf kf = as_v8bf(*(const uint4*)(kt + col * PF_KPITCH + (16 * c + 8 * hl) * 2));
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], s, 0, 0, 0);
         }
         // ---- mask, online softmax (per lane = per query; the other half of the keys sits in lane ^ 32)
-        float mx = PF_NEG;
+        if (masked) {                      // wave-uniform
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int key = kb + 8 * (r >> 2) + 4 * hl + (r & 3);
-            const bool vis = key <= qpos && key >= q_lo && key <= k_hi;
-            s[r] = vis ? s[r] * sc : PF_NEG;
-            mx = fmaxf(mx, s[r]);
+            for (int r = 0; r < 16; r++) {
+                const int key = kb + 8 * (r >> 2) + 4 * hl + (r & 3);
+                const bool vis = key <= qpos && key >= q_lo && key <= k_hi;
+                s[r] = vis ? s[r] : PF_MASKED;
+            }
         }
+        float mx = s[0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        const float corr = exp2f(m_run - m_new);
-        m_run = m_new;
+        // (a sub-block with nothing visible for this lane leaves the maximum where it was: PF_MASKED * sc lies below the floor,
+        // and its weights come out as exp2(-huge) = 0)
+        // The reference point of the exponentials only follows the maximum when it has moved by more than PF_LAZY (in log2 units)
+        // for some lane of the wave: until then the weights may exceed 1 (by at most 2^PF_LAZY, nothing for fp32 sums or bf16
+        // weights), the quotient sum(p v) / sum(p) is the same, and the 64 accumulators are spared the multiply.
+        const float m_new = fmaxf(m_run, mx * sc);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run + PF_LAZY) != 0) {      // wave-uniform
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= corr;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] *= corr;
+            m_run = m_new;
+        }
         float psum = 0.f;
         v8bf pf[2];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            // a fully masked block leaves m_new at PF_NEG: exp2f(0) would be 1, so masked entries are zeroed explicitly
-            const float p = s[r] > 0.5f * PF_NEG ? exp2f(s[r] - m_new) : 0.f;
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[r], sc, -m_run));
             psum += p;
             pf[r >> 3][r & 7] = (__bf16)p;
         }
-        l_run = l_run * corr + psum;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) o[dt][r] *= corr;
+        l_run += psum;
         // ---- O^T += V^T . P^T : chunk c2 of 16 keys uses accumulator rows 8*c2 .. 8*c2+7, i.e. keys
         //      kb + 16*c2 + 4*hl + {0..3} and kb + 16*c2 + 8 + 4*hl + {0..3}; V^T is read in the same order
 #pragma unroll
         for (int c2 = 0; c2 < 2; c2++)
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const uint8_t* vrow = lds_v[sb] + (32 * dt + col) * PF_VPITCH + (16 * c2 + 4 * hl) * 2;
-                const uint2 lo = *(const uint2*)vrow, hi = *(const uint2*)(vrow + 16);
-                const v8bf vf = as_v8bf(make_uint4(lo.x, lo.y, hi.x, hi.y));
+                const lds_u8_t vblk = lds_v3 + sb * PF_VBYTES + vtr_off + 16 * c2 * PF_VPITCH + 32 * dt * 2;
+                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)vblk);
+                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)(vblk + 8 * PF_VPITCH));
+                const v8bf vf = __builtin_bit_cast(v8bf, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
                 o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[c2], o[dt], 0, 0, 0);
             }
+    };
+    // (wave-uniform tests: a skipped sub-block holds no key that any query of this wave sees)
+    auto visit = [&](int kb, int sb) {
+        if (kb <= w_hi && kb + 31 >= w_lo) sub_block(kb, sb, !(kb >= f_lo && kb + 31 <= f_hi));
     };
 
     if (kb_first <= k_hi) fetch(kb_first);
@@ -172,16 +246,45 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
         stage();
         __syncthreads();
         if (kb + 64 <= k_hi) fetch(kb + 64);
-        // (wave-uniform tests: a skipped sub-block holds no key that any query of this wave sees)
-        if (kb <= w_hi && kb + 31 >= w_lo) sub_block(kb, 0);
-        if (kb + 32 <= w_hi && kb + 63 >= w_lo) sub_block(kb + 32, 1);
+        if (KS == 1) {
+#pragma unroll 1
+            for (int sb = 0; sb < 2; sb++) visit(kb + 32 * sb, sb);
+        } else {
+            visit(kb + 32 * ks, ks);
+        }
+    }
+
+    if (KS == 2) {
+        // the wave with the odd sub-blocks hands its state to its partner through the tile memory: [value][lane] floats,
+        // values 0..63 the accumulators, 64 the maximum, 65 the sum
+        __syncthreads();
+        float* xch = (float*)lds + (wave / (2 * GS) * GS + wave % GS) * (66 * 64);
+        if (ks == 1) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) xch[(16 * dt + r) * 64 + lane] = o[dt][r];
+            xch[64 * 64 + lane] = m_run;
+            xch[65 * 64 + lane] = l_run;
+        }
+        __syncthreads();
+        if (ks == 0) {
+            const float m2 = xch[64 * 64 + lane], l2 = xch[65 * 64 + lane];
+            const float m_new = fmaxf(m_run, m2);
+            const float wa = __builtin_amdgcn_exp2f(m_run - m_new), wb = __builtin_amdgcn_exp2f(m2 - m_new);
+            l_run = l_run * wa + l2 * wb;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * wa + xch[(16 * dt + r) * 64 + lane] * wb;
+        }
     }
 
     // ---- finish: total weight of the query = both lane halves
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     float am = 0.f;
-    if (q_ok) {
+    if (q_ok && ks == 0) {
         bf16_t* orow = out + (((size_t)b * T + t) * H + h) * 128;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
@@ -209,20 +312,30 @@ int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf
     NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && out, "prefill_attention: null pointer");
     NC_CHECK_ARG(B > 0 && T > 0 && H > 0 && Hkv > 0 && Tmax > 0 && H % Hkv == 0, "prefill_attention: bad shape");
     NC_CHECK_ARG(B <= 65535 && H <= 65535, "prefill_attention: more than 65535 rows or heads in one launch");
+    NC_CHECK_ARG((long long)Tmax * Hkv * 128 < (1LL << 31), "prefill_attention: one row of the cache must stay below 2^31 elements");
     NC_CHECK_ARG((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15) == 0,
                  "prefill_attention: pointers must be 16-byte aligned");
     NcProfScope prof(0, 0.0, s);
     const int G = H / Hkv;
     const int GS = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);       // query heads of a kv head per workgroup
-    const int QT = 128 / GS;
+    // two waves per query block, each with half of the keys, when whole-key-range workgroups would not give every CU two of them
+    const long long wgs1 = (long long)B * Hkv * (G / GS) * ((T + 128 / GS - 1) / (128 / GS));
+#ifdef PF_FORCE_KS
+    const int KS = GS <= 2 ? PF_FORCE_KS : 1;
+#else
+    const int KS = (GS <= 2 && wgs1 < 2LL * nc_cu_count()) ? 2 : 1;
+#endif
+    const int QT = 128 / (GS * KS);
     const dim3 grid((T + QT - 1) / QT, Hkv * (G / GS), B);
     NC_CHECK_ARG(grid.y <= 65535, "prefill_attention: too many heads in one launch");
-#define PF_LAUNCH(GG)                                                                                                                  \
-    hipLaunchKernelGGL(attn_prefill_kernel<GG>, grid, dim3(256), 0, s, q, k_cache, v_cache, cache_seqlens, window_left, seqlens_include_new, \
-                       out, amax_ws, T, H, Hkv, Tmax)
-    if (GS == 4) PF_LAUNCH(4);
-    else if (GS == 2) PF_LAUNCH(2);
-    else PF_LAUNCH(1);
+#define PF_LAUNCH(GG, KK)                                                                                                              \
+    hipLaunchKernelGGL((attn_prefill_kernel<GG, KK>), grid, dim3(256), 0, s, q, k_cache, v_cache, cache_seqlens, window_left,          \
+                       seqlens_include_new, out, amax_ws, T, H, Hkv, Tmax)
+    if (GS == 4) PF_LAUNCH(4, 1);
+    else if (GS == 2 && KS == 2) PF_LAUNCH(2, 2);
+    else if (GS == 2) PF_LAUNCH(2, 1);
+    else if (KS == 2) PF_LAUNCH(1, 2);
+    else PF_LAUNCH(1, 1);
 #undef PF_LAUNCH
     NC_CHECK_LAUNCH("prefill_attention");
     return 0;

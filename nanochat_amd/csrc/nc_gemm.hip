@@ -517,6 +517,8 @@ hipError_t reserve_lds(const void* fn, int bytes) {
 }
 }  // namespace
 
+int nc_cu_count() { return cu_count(); }
+
 template <int BM, int BN, int WGM, int WGN, bool INTERLEAVE, int A_FMT, int OUT_KIND>
 static int launch_bl_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;

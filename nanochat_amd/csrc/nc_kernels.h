@@ -88,6 +88,8 @@ int nc_launch_attention(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_
                         int counters_are_zero, hipStream_t s);
 
 // many query positions per row (nc_attention_prefill.hip): flash-attention forward on the bf16 matrix cores
+// compute units of the current device (looked up once per process and device)
+int nc_cu_count();
 int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
                                 int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                                 uint32_t* amax_ws, hipStream_t s);
