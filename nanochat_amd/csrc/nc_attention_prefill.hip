@@ -28,23 +28,7 @@ typedef __attribute__((address_space(3))) uint8_t* lds_u8_t;
 #define PF_KBYTES (32 * PF_KPITCH)
 #define PF_VBYTES (32 * PF_VPITCH)
 #define PF_MASKED (-1.0e30f)   // raw score of a key that the query does not see
-#ifndef PF_OPT_COND
-#define PF_OPT_COND 1
-#endif
-#ifndef PF_OPT_XCD
-#define PF_OPT_XCD 1
-#endif
-#ifndef PF_OPT_WAVES
-#define PF_OPT_WAVES 1
-#endif
-#if PF_OPT_WAVES
-#define PF_WAVES_ATTR __attribute__((amdgpu_waves_per_eu(2, 2)))
-#else
-#define PF_WAVES_ATTR
-#endif
-#ifndef PF_LAZY
-#define PF_LAZY 6.0f
-#endif
+#define PF_LAZY 6.0f           // log2 units the running maximum may lag behind before the accumulators are rescaled
 #define PF_M_FLOOR (-1.0e20f)  // running maximum (scaled units) before any visible key: far above PF_MASKED * scale, far below any score
 
 __device__ __forceinline__ v8bf as_v8bf(uint4 v) { return __builtin_bit_cast(v8bf, v); }
@@ -61,7 +45,7 @@ __device__ __forceinline__ v8bf as_v8bf(uint4 v) { return __builtin_bit_cast(v8b
 // triggers a rescale of the 64 output accumulators when it moved for some lane of the wave.  Tiles are handed out from the end of the
 // sequence, longest key ranges first.
 template <int GS, int KS>
-__global__ __launch_bounds__(256) PF_WAVES_ATTR void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                                                            const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
                                                            uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax) {
@@ -79,12 +63,8 @@ __global__ __launch_bounds__(256) PF_WAVES_ATTR void attn_prefill_kernel(const b
     int qb0, hy;
     {
         const int nx = gridDim.x, total = nx * (int)gridDim.y, lid = (int)blockIdx.x + nx * (int)blockIdx.y;
-#if PF_OPT_XCD
         const int xcd = lid & 7, slot = lid >> 3;
         const int unit = xcd * (total >> 3) + min(xcd, total & 7) + slot;
-#else
-        const int unit = lid;
-#endif
         hy = unit / nx;
         qb0 = (nx - 1 - unit % nx) * QT;
     }
@@ -141,20 +121,16 @@ __global__ __launch_bounds__(256) PF_WAVES_ATTR void attn_prefill_kernel(const b
     const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + ch * 8;
     uint4 rk[2][2], rv[2][2];
     // Load j (0..7) of the 64 keys from kb on: sub-block j / 4, key 2 kp + (j / 2) % 2 of it, K for even j and V for odd j.  Keys past
-    // the end of the workgroup's range are read from its last key instead (no query gives them any weight), so no load is conditional.
+    // the end of the workgroup's range come as zeros.  (The conditional form is deliberate: with unconditional loads of clamped
+    // addresses the compiler issues all eight in one burst, the wave then waits in the memory pipeline's queue instead of computing,
+    // and the kernel was measured at half the speed.)
     auto fetch_one = [&](int kb, int j) {
         const int sb = j >> 2, i = (j >> 1) & 1;
-#if PF_OPT_COND
         const int key = kb + 32 * sb + 2 * kp + i;
         const bool ok = key <= k_hi;
         const uint32_t off = (uint32_t)key * key_stride;
         if (j & 1) rv[sb][i] = ok ? *(const uint4*)(vbase + off) : make_uint4(0, 0, 0, 0);
         else rk[sb][i] = ok ? *(const uint4*)(kbase + off) : make_uint4(0, 0, 0, 0);
-#else
-        const uint32_t off = (uint32_t)min(kb + 32 * sb + 2 * kp + i, k_hi) * key_stride;      // (one row's cache fits 32 bits: checked at launch)
-        if (j & 1) rv[sb][i] = *(const uint4*)(vbase + off);
-        else rk[sb][i] = *(const uint4*)(kbase + off);
-#endif
     };
     auto fetch = [&](int kb) {
 #pragma unroll
@@ -320,11 +296,7 @@ int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf
     const int GS = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);       // query heads of a kv head per workgroup
     // two waves per query block, each with half of the keys, when whole-key-range workgroups would not give every CU two of them
     const long long wgs1 = (long long)B * Hkv * (G / GS) * ((T + 128 / GS - 1) / (128 / GS));
-#ifdef PF_FORCE_KS
-    const int KS = GS <= 2 ? PF_FORCE_KS : 1;
-#else
     const int KS = (GS <= 2 && wgs1 < 2LL * nc_cu_count()) ? 2 : 1;
-#endif
     const int QT = 128 / (GS * KS);
     const dim3 grid((T + QT - 1) / QT, Hkv * (G / GS), B);
     NC_CHECK_ARG(grid.y <= 65535, "prefill_attention: too many heads in one launch");
