@@ -34,26 +34,19 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float(
 __device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
 
-// round-to-nearest-even fp32 -> bf16 (NaN kept quiet)
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
-}
+// fp32 -> bf16, round to nearest even (NaN stays NaN): gfx950's own convert (v_cvt_pk_bf16_f32), one instruction where the integer form (NaN test,
+// rounding increment, shift) takes six; the row kernels round after every elementary operation, so this is most of their arithmetic
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
 // value of f after rounding to bf16, as fp32 (one rounding site of a bf16 eager op)
 __device__ __forceinline__ float rbf(float f) { return bf16_to_f32(f32_to_bf16(f)); }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
-}
-
-// two fp32 -> packed bf16 pair with the hardware convert (round to nearest even), low half = first value
+// two fp32 -> packed bf16 pair (one convert instruction), low half = first value
 typedef __bf16 nc_bf16x2 __attribute__((ext_vector_type(2)));
 typedef float nc_f32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pack_bf16_hw(float lo, float hi) {
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     const nc_f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, nc_bf16x2));
 }
+__device__ __forceinline__ uint32_t pack_bf16_hw(float lo, float hi) { return pack_bf16(lo, hi); }
 
 // ---------------------------------------------------------------- e4m3fn (OCP) encode
 // |y| must already be clamped to <= 448.  Round to nearest even, subnormals down to 2^-9.
