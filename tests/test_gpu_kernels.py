@@ -689,6 +689,37 @@ def test_attention_many_queries_per_row(ops, T, window, H, Hkv, seqlens):
     attn_case(ops, 2, T, H, Hkv, 512, seqlens, window, 0, seed=T + H)
 
 
+@pytest.mark.parametrize("B,T,H,Hkv,window", [(64, 40, 8, 8, -1), (64, 100, 8, 4, 48), (70, 33, 4, 1, -1)])
+def test_attention_many_rows_of_many_queries(ops, B, T, H, Hkv, window):
+    """Enough (row, head, tile) units that every query block gets a wave of its own with the whole key range (launches with
+    few units split the keys of a block between two waves instead: the cases above)."""
+    say(f"attention prefill B={B} T={T} H={H}/{Hkv} window={window}")
+    g = torch.Generator().manual_seed(B + T)
+    seqlens = torch.randint(0, 128 - T, (B,), generator=g).tolist()
+    attn_case(ops, B, T, H, Hkv, 128, seqlens, window, 0, seed=B * T)
+
+
+@pytest.mark.parametrize("T,gain", [(300, 0.02), (300, 0.2), (130, 1.0)])
+def test_attention_prefill_scores_that_keep_growing(ops, T, gain):
+    """Every key scores higher than the one before it (by `gain` per key on average, in units of the softmax exponent), so the running
+    maximum moves in every block: slowly (the reference point of the exponentials lags behind and weights exceed 1), or by a lot
+    (a rescale per block, early keys vanishing)."""
+    say(f"attention prefill growing scores T={T} gain={gain}")
+    g = torch.Generator().manual_seed(T)
+    B, H, Tmax = 2, 2, 320
+    direction = torch.randn(128, generator=g)
+    direction = direction / direction.norm()
+    q = (direction * 128 ** 0.5 + 0.05 * torch.randn(B, T, H, 128, generator=g)).bfloat16()      # q . direction / sqrt(128) ~ 1
+    ramp = torch.arange(Tmax, dtype=torch.float32)[None, :, None, None] * gain
+    kc = (ramp * direction + 0.3 * torch.randn(B, Tmax, H, 128, generator=g)).bfloat16()
+    vc = torch.randn(B, Tmax, H, 128, generator=g).bfloat16()
+    seq = torch.tensor([0, Tmax - T], dtype=torch.int32)
+    for window in (-1, 40):
+        want = attention_with_kvcache(q, kc, vc, None, None, seq, (window, 0))
+        got = ops.decode_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), seq.to(DEV), window_left=window).cpu()
+        assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2), (window, (got.float() - want.float()).abs().max().item())
+
+
 def test_attention_through_the_plugin_seam(ops):
     """flash_attn_with_kvcache as the model calls it: in-place insert, caller advances, then decode."""
     say("flash_attn seam")
