@@ -200,7 +200,7 @@ int nc_softcap(const uint16_t* raw, float* out, int64_t n, float softcap, nc_str
 
 /* (5) Next-token selection: nanochat/engine.py:140-156.  logits fp32 [B,ld]; temperature 0 =>
  * argmax (first index on ties).  Otherwise noise holds Exp(1) draws, [B,k] with top-k (k =
- * min(top_k,V) <= 256; rank j of the descending top-k list uses noise[b,j]) or [B,V] without
+ * min(top_k,V) <= 4096; rank j of the descending top-k list uses noise[b,j]) or [B,V] without
  * (top_k <= 0), and the draw is argmax_j softmax_j / noise_j, which is what torch.multinomial
  * computes.  out_ids int64 [B]. */
 int nc_sample(const float* logits, int B, int V, int ld, float temperature, int top_k, const float* noise,

@@ -11,7 +11,7 @@
 #include "nc_kernels.h"
 
 #define SAMPLE_THREADS 256
-#define MAX_TOP_K 256
+#define MAX_TOP_K 4096          // the larger of the two instantiations below (256 and 4096 candidates in LDS)
 
 __global__ __launch_bounds__(256) void softcap_kernel(const bf16_t* __restrict__ raw, float* __restrict__ out, int64_t n, float softcap) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -73,16 +73,17 @@ __device__ __forceinline__ void scan_row(const float* __restrict__ lr, int V, in
     for (int i = done + tid; i < V; i += SAMPLE_THREADS) f(lr[i], i);
 }
 
+template <int KMAX>
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, int V, int ld, float temperature,
                                                                 int top_k, const float* __restrict__ noise, int64_t* __restrict__ out_ids) {
     __shared__ float sval[4];
     __shared__ int sidx[4];
     __shared__ uint32_t hist[256];
     __shared__ uint32_t sel_prefix, sel_need;
-    __shared__ unsigned long long cand[MAX_TOP_K];    // (key << 32) | ~index : sorts by value desc, index asc
+    __shared__ unsigned long long cand[KMAX];         // (key << 32) | ~index : sorts by value desc, index asc
     __shared__ uint32_t cand_count;
     __shared__ uint32_t scan[SAMPLE_THREADS];
-    __shared__ float probs[MAX_TOP_K];
+    __shared__ float probs[KMAX];
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* lr = logits + (size_t)row * ld;
 
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
         const uint32_t key = fkey(lr[i]);
         if (key > kth) {
             const uint32_t slot = atomicAdd(&cand_count, 1u);
-            if (slot < MAX_TOP_K) cand[slot] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
+            if (slot < KMAX) cand[slot] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
         } else if (key == kth) eq_local++;
     }
     scan[tid] = eq_local;
@@ -171,22 +172,27 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     for (int i = i0; i < i1 && rank < need_eq; i++) {
         if (fkey(lr[i]) == kth) {
             const uint32_t slot = gt_count + rank;
-            if (slot < MAX_TOP_K) cand[slot] = ((unsigned long long)kth << 32) | (uint32_t)(~(uint32_t)i);
+            if (slot < KMAX) cand[slot] = ((unsigned long long)kth << 32) | (uint32_t)(~(uint32_t)i);
             rank++;
         }
     }
-    for (int j = tid; j < MAX_TOP_K; j += SAMPLE_THREADS)
+    // the sort works on the next power of two at or above k (at least one entry per thread)
+    int nsort = SAMPLE_THREADS;
+    while (nsort < (int)k) nsort <<= 1;
+    for (int j = tid; j < nsort; j += SAMPLE_THREADS)
         if ((uint32_t)j >= k) cand[j] = 0ull;      // padding sorts last
     __syncthreads();
 
-    // ---- bitonic sort, descending, MAX_TOP_K entries, one per thread
-    for (int size = 2; size <= MAX_TOP_K; size <<= 1) {
+    // ---- bitonic sort, descending
+    for (int size = 2; size <= nsort; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            const int j = tid, partner = j ^ stride;
-            if (partner > j && j < MAX_TOP_K) {
-                const bool desc = ((j & size) == 0);
-                const unsigned long long a = cand[j], c = cand[partner];
-                if ((a < c) == desc) cand[j] = c, cand[partner] = a;
+            for (int j = tid; j < nsort; j += SAMPLE_THREADS) {
+                const int partner = j ^ stride;
+                if (partner > j) {
+                    const bool desc = ((j & size) == 0);
+                    const unsigned long long a = cand[j], c = cand[partner];
+                    if ((a < c) == desc) cand[j] = c, cand[partner] = a;
+                }
             }
             __syncthreads();
         }
@@ -194,17 +200,16 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
 
     // ---- softmax over the k sorted values / T, then the draw
     const float vmax = fkey_inv((uint32_t)(cand[0] >> 32)) / temperature;
-    float e = 0.f;
-    if ((uint32_t)tid < k) e = expf(fkey_inv((uint32_t)(cand[tid] >> 32)) / temperature - vmax);
-    probs[tid] = e;
+    for (uint32_t j = tid; j < (uint32_t)nsort; j += SAMPLE_THREADS)
+        probs[j] = j < k ? expf(fkey_inv((uint32_t)(cand[j] >> 32)) / temperature - vmax) : 0.f;
     __syncthreads();
     float denom = 0.f;
     for (uint32_t j = 0; j < k; j++) denom += probs[j];     // same order on every thread: deterministic
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    if ((uint32_t)tid < k) {
-        bv = (e / denom) / noise[(size_t)row * k + tid];
-        bi = tid;
+    for (uint32_t j = tid; j < k; j += SAMPLE_THREADS) {    // ascending ranks per thread: the first of equal quotients wins
+        const float qv = (probs[j] / denom) / noise[(size_t)row * k + j];
+        if (qv > bv) bv = qv, bi = (int)j;
     }
     block_argmax(bv, bi, sval, sidx);
     if (tid == 0) {
@@ -232,7 +237,10 @@ int nc_launch_sample(const float* logits, int B, int V, int ld, float temperatur
     const int k_eff = (top_k > 0 && top_k < V) ? top_k : 0;
     NC_CHECK_ARG(k_eff <= MAX_TOP_K, "sample: top_k %d exceeds the supported maximum of %d (or pass 0 for none)", top_k, MAX_TOP_K);
     NcProfScope prof(4, 4.0 * B * V, s);
-    hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(SAMPLE_THREADS), 0, s, logits, V, ld, temperature, k_eff, noise, out_ids);
+    if (k_eff <= 256)
+        hipLaunchKernelGGL(sample_kernel<256>, dim3(B), dim3(SAMPLE_THREADS), 0, s, logits, V, ld, temperature, k_eff, noise, out_ids);
+    else
+        hipLaunchKernelGGL(sample_kernel<MAX_TOP_K>, dim3(B), dim3(SAMPLE_THREADS), 0, s, logits, V, ld, temperature, k_eff, noise, out_ids);
     NC_CHECK_LAUNCH("sample");
     return 0;
 }

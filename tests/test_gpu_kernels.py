@@ -786,7 +786,9 @@ def test_sample_argmax_first_index_on_ties(ops):
 
 
 @pytest.mark.parametrize("temperature,top_k,V", [(1.0, 50, 32768), (0.6, 50, 32768), (0.8, 1, 1000), (1.0, 256, 5000),
-                                                 (1.3, None, 4096), (1.0, 500, 262)])
+                                                 (1.3, None, 4096), (1.0, 500, 262),
+                                                 # more candidates than threads: the 4096-entry instantiation, sorts of 512 .. 4096
+                                                 (1.0, 257, 32768), (0.9, 1000, 32768), (1.0, 4096, 32768), (0.7, 3000, 5000)])
 def test_sample_matches_oracle_given_the_same_noise(ops, temperature, top_k, V):
     say(f"sample T={temperature} k={top_k} V={V}")
     g = torch.Generator().manual_seed(7)
