@@ -978,10 +978,12 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             const int cus = cu_count();
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             const long rounds = (t256 + cus - 1) / cus;
-            if (out_kind != 1 && K % 128 == 0 && 8 * t256 >= 5 * cus) {
-                // 256x256 tiles fed straight into LDS whenever they occupy at least 5/8 of the CUs (below that the
-                // 128x128 tiles, four times as many, fill the chip better); from two rounds of tiles on, the
-                // persistent form, which neither rounds the last round up nor pays a prologue per tile
+            const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+            if (out_kind != 1 && K % 128 == 0 && (8 * t256 >= 5 * cus || t128 > 2 * cus)) {
+                // 256x256 tiles fed straight into LDS whenever they occupy at least 5/8 of the CUs, or the 128x128 tiles, four times
+                // as many, would not fit the chip in one round of two workgroups per CU (below that the small tiles fill the chip
+                // better: 18 us against 22 for 1280 x 4992 x 1664, but 25 against 22.4 for 1792 rows); from two rounds of tiles on,
+                // the persistent form, which neither rounds the last round up nor pays a prologue per tile
                 which = (t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8;
             } else {
                 // 256x256 tiles move half the bytes per flop through L2 and LDS but run one workgroup per CU: take them
