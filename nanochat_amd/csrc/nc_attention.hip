@@ -304,7 +304,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         if (nsplit == 1) {
             const bf16_t o = f32_to_bf16(a / ls);
             out[((size_t)row * H + head) * 128 + d] = o;
-            am = fmaxf(am, fabsf(bf16_to_f32(o)));
+            am = amax_fold(am, bf16_to_f32(o));
         } else {
             float* p = partials + (((size_t)row * H + head) * nsplit + split) * PART_STRIDE;
             if (d == 0) coherent_store_f1(p, mm), coherent_store_f1(p + 1, ls);
@@ -328,17 +328,17 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             }
             const bf16_t o = f32_to_bf16(a / ls);
             out[((size_t)row * H + head) * 128 + d] = o;
-            am = fmaxf(am, fabsf(bf16_to_f32(o)));
+            am = amax_fold(am, bf16_to_f32(o));
         }
         if (threadIdx.x == 0) __hip_atomic_store(&counters[row * Hkv + hp * HP], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (amax_ws) {
         // one publication per workgroup (only the first threads hold output values)
-        am = wave_max(am);
+        am = wave_amax(am);
         __syncthreads();
         if (lane == 0) merge[wave][0][0] = am;
         __syncthreads();
-        if (threadIdx.x == 0) amax_publish(amax_ws, fmaxf(fmaxf(merge[0][0][0], merge[1][0][0]), fmaxf(merge[2][0][0], merge[3][0][0])));
+        if (threadIdx.x == 0) amax_publish(amax_ws, amax_join(amax_join(merge[0][0][0], merge[1][0][0]), amax_join(merge[2][0][0], merge[3][0][0])));
     }
 }
 

@@ -270,15 +270,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const uint2 pk = make_uint2(pack_bf16(o[dt][4 * g4] * inv_l, o[dt][4 * g4 + 1] * inv_l),
                                             pack_bf16(o[dt][4 * g4 + 2] * inv_l, o[dt][4 * g4 + 3] * inv_l));
                 *(uint2*)(orow + d) = pk;
-                am = fmaxf(am, fmaxf(fmaxf(fabsf(bf16_lo(pk.x)), fabsf(bf16_hi(pk.x))), fmaxf(fabsf(bf16_lo(pk.y)), fabsf(bf16_hi(pk.y)))));
+                am = amax_fold(amax_fold(amax_fold(amax_fold(am, bf16_lo(pk.x)), bf16_hi(pk.x)), bf16_lo(pk.y)), bf16_hi(pk.y));
             }
     }
     if (amax_ws) {
-        am = wave_max(am);
+        am = wave_amax(am);
         __syncthreads();
         if (lane == 0) red[wave] = am;
         __syncthreads();
-        if (tid == 0) amax_publish(amax_ws, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+        if (tid == 0) amax_publish(amax_ws, amax_join(amax_join(red[0], red[1]), amax_join(red[2], red[3])));
     }
 }
 

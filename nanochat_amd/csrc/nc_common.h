@@ -146,6 +146,16 @@ __device__ __forceinline__ float wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
     return v;
 }
+// Running maximum of magnitudes that a NaN survives, as it survives the reference's x.abs().max() (nanochat/fp8.py:92): magnitudes are
+// compared as unsigned bit patterns, which order like the values for non-negative floats and put every NaN above infinity.  (fmaxf
+// returns the other operand when one is NaN, which would hide a NaN activation from the scale of the next FP8 linear.)
+__device__ __forceinline__ float amax_join(float a, float b) {            // both already magnitudes (sign bit clear)
+    const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+    return __uint_as_float(ua > ub ? ua : ub);
+}
+__device__ __forceinline__ float amax_fold(float am, float x) { return amax_join(am, __uint_as_float(__float_as_uint(x) & 0x7fffffffu)); }
+// relu that keeps a NaN, as torch.relu does (fmaxf(x, 0) would turn it into 0)
+__device__ __forceinline__ float relu_keep_nan(float x) { return x < 0.f ? 0.f : x; }
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -154,6 +164,8 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     }
     return v;
 }
+
+__device__ __forceinline__ float wave_amax(float am) { return __uint_as_float(wave_max_u32(__float_as_uint(am))); }
 
 // ---------------------------------------------------------------- cross-workgroup hand-off without cache flushes
 // Split results travel between workgroups through device-scope relaxed atomic accesses: such stores are

@@ -15,13 +15,13 @@
 
 __device__ __forceinline__ void block_amax_commit(float local_abs_max, uint32_t* amax_ws, float* red) {
     if (!amax_ws) return;
-    float m = wave_max(local_abs_max);
+    float m = wave_amax(local_abs_max);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
     __syncthreads();
     if (lane == 0) red[w] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < nw; i++) m = fmaxf(m, red[i]);
+        for (int i = 1; i < nw; i++) m = amax_join(m, red[i]);
         amax_publish(amax_ws, m);
     }
 }
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) void mix_norm_kernel(bf16_t* __restrict__ x, c
     for (int c = threadIdx.x; c < cols; c += 256) {
         const bf16_t o = f32_to_bf16(rowbuf[c] * rstd);
         xn_out[base + c] = o;
-        am = fmaxf(am, fabsf(bf16_to_f32(o)));
+        am = amax_fold(am, bf16_to_f32(o));
     }
     block_amax_commit(am, amax_ws, red);
 }
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 o[j] = pack_bf16(v[it][2 * j] * rstd, v[it][2 * j + 1] * rstd);
-                am = fmaxf(am, fmaxf(fabsf(bf16_lo(o[j])), fabsf(bf16_hi(o[j]))));
+                am = amax_fold(amax_fold(am, bf16_lo(o[j])), bf16_hi(o[j]));
             }
             *(uint4*)(xn_out + base + c) = make_uint4(o[0], o[1], o[2], o[3]);
         }
@@ -325,18 +325,18 @@ __global__ __launch_bounds__(256) void relu2_kernel(const bf16_t* __restrict__ h
         uint32_t w[4] = {v.x, v.y, v.z, v.w}, o[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            float a = fmaxf(bf16_lo(w[j]), 0.f), b = fmaxf(bf16_hi(w[j]), 0.f);
+            float a = relu_keep_nan(bf16_lo(w[j])), b = relu_keep_nan(bf16_hi(w[j]));
             a = rbf(a * a), b = rbf(b * b);
-            am = fmaxf(am, fmaxf(a, b));
+            am = amax_join(amax_join(am, a), b);
             o[j] = pack_bf16(a, b);
         }
         ((uint4*)out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
     }
     if (blockIdx.x == 0)
         for (int64_t i = nvec * 8 + threadIdx.x; i < n; i += blockDim.x) {
-            float a = fmaxf(bf16_to_f32(h[i]), 0.f);
+            float a = relu_keep_nan(bf16_to_f32(h[i]));
             a = rbf(a * a);
-            am = fmaxf(am, a);
+            am = amax_join(am, a);
             out[i] = f32_to_bf16(a);
         }
     block_amax_commit(am, amax_ws, red);

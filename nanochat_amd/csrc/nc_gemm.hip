@@ -38,7 +38,7 @@ struct EpilogueArgs {
 
 // relu(bf16(v))^2, to be rounded to bf16 by the caller's pack: the two eager ops of nanochat/gpt.py:139 on a bf16 tensor
 __device__ __forceinline__ float relu2_of(float v) {
-    const float h = fmaxf(rbf(v), 0.f);
+    const float h = relu_keep_nan(rbf(v));
     return h * h;
 }
 // largest of eight non-negative bf16 values in a 16-byte vector, the first `count` of them
@@ -247,7 +247,7 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             const int m = m0 + wm * WROWS + row;
             const uint4 v = *(const uint4*)(reg + row * ROWB + ((c ^ (row & 7)) << 4));
             if (m >= M || n >= N) continue;
-            if (relu2) am = fmaxf(am, max_bf16x8(v, N - n));
+            if (relu2) am = amax_join(am, max_bf16x8(v, N - n));
             bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
             if (n + 8 <= N) {
                 if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
@@ -261,7 +261,7 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             }
         }
         if (relu2) {
-            am = wave_max(am);
+            am = wave_amax(am);
             if (lane == 0) amax_publish(ep.out_amax, am);
         }
     } else {
@@ -735,7 +735,7 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
             const int m = m0 + g.wm * 64 + i * 16 + row;
             const uint4 v = make_uint4((uint32_t)rd[it][0], (uint32_t)rd[it][1], (uint32_t)rd[it][2], (uint32_t)rd[it][3]);
             if (m >= M || n_st >= N) continue;
-            if (relu2) am = fmaxf(am, max_bf16x8(v, N - n_st));
+            if (relu2) am = amax_join(am, max_bf16x8(v, N - n_st));
             bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n_st;
             if (n_st + 8 <= N) {
                 if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
@@ -751,7 +751,7 @@ __device__ __forceinline__ void dlp_epilogue(v4f (&acc)[4][8], uint8_t* reg, con
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads are done before the next 16 rows overwrite the region
     }
     if (relu2) {
-        am = wave_max(am);
+        am = wave_amax(am);
         if (g.lane == 0) amax_publish(ep.out_amax, am);
     }
 }

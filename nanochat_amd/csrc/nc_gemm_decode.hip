@@ -213,9 +213,9 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
                 if (g.out_kind == 2) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        const float t = fmaxf(rbf(v[r]), 0.f);
+                        const float t = relu_keep_nan(rbf(v[r]));
                         v[r] = rbf(t * t);
-                        if (n + r < N) am = fmaxf(am, v[r]);
+                        if (n + r < N) am = amax_join(am, v[r]);
                     }
                 }
                 bf16_t* o = (bf16_t*)g.out + (size_t)m * g.ldc + n;
@@ -226,11 +226,11 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
         }
     }
     if (g.out_kind == 2 && g.out_amax) {
-        am = wave_max(am);
+        am = wave_amax(am);
         if (lane == 0) red[wave] = am;
         __syncthreads();
         if (tid == 0) {
-            am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            am = amax_join(amax_join(red[0], red[1]), amax_join(red[2], red[3]));
             amax_publish(g.out_amax, am);
         }
     }
@@ -282,20 +282,20 @@ __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __res
             if (out_kind == 2) {
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const float t = fmaxf(rbf(v[r]), 0.f);
+                    const float t = relu_keep_nan(rbf(v[r]));
                     v[r] = rbf(t * t);
-                    am = fmaxf(am, v[r]);
+                    am = amax_join(am, v[r]);
                 }
             }
             *(uint2*)((bf16_t*)out + (size_t)m * ldc + n) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
         }
     }
     if (out_kind == 2 && out_amax) {
-        am = wave_max(am);
+        am = wave_amax(am);
         if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = am;
         __syncthreads();
         if (threadIdx.x == 0) {
-            am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            am = amax_join(amax_join(red[0], red[1]), amax_join(red[2], red[3]));
             amax_publish(out_amax, am);
         }
     }

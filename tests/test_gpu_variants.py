@@ -253,6 +253,40 @@ def test_one_layer_models_against_the_oracle(cfg_kwargs, B):
         assert ulps <= 4 and frac < 0.02, (frac, ulps)
 
 
+@pytest.mark.parametrize("where", ["embedding", "cache"])
+def test_a_nan_activation_reaches_every_logit_as_in_the_reference(where):
+    """x.abs().max() of a tensor that holds a NaN is NaN (nanochat/fp8.py:92), so the scale of the next FP8 linear is NaN and with it
+    every row of that linear's output, not only the row the NaN sits in.  The fused kernels fold the amax into their epilogues; they
+    must not lose the NaN on the way (fmaxf would), and relu must keep it (torch.relu does)."""
+    say(f"NaN propagation from the {where}")
+    from nanochat_amd.engine import KVCache
+    cfg_kwargs = dict(sequence_len=64, vocab_size=1024, n_layer=3, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
+    rt, model = build_pair(cfg_kwargs, seed=23)
+    cfg = rt.cfg
+    B, P = 3, 9
+    prompt = torch.arange(B * P).reshape(B, P) * 7 % cfg.vocab_size + 1        # all ids distinct
+    nxt = torch.tensor([[900], [901], [902]])
+    if where == "embedding":
+        bad = int(prompt[0, 2])                                                 # only row 0 meets the poisoned table row
+        rt.p["transformer.wte.weight"][bad, 5] = float("nan")
+        model.transformer.wte.weight.data[bad, 5] = float("nan")
+    cache = decode_ref.new_cache(cfg, B, P + 1, torch.bfloat16)
+    dec = KVCache(B, cfg.n_kv_head, P + 1, 128, cfg.n_layer, DEV, torch.bfloat16)
+    want = gpt_ref.forward(rt, prompt, cache)[:, -1]
+    got = model.forward_last(prompt.to(DEV), kv_cache=dec).cpu()
+    if where == "embedding":
+        assert torch.isnan(want).all(), "the oracle itself should be all NaN here"
+        assert torch.isnan(got).all(), f"{(~torch.isnan(got)).sum().item()} finite logits left after a NaN embedding"
+        return
+    assert torch.isfinite(want).all() and torch.isfinite(got).all()
+    cache.k_cache[1, 1, 3, 0, 7] = float("nan")                                 # layer 1, row 1, position 3, kv head 0
+    dec.k_cache[1, 1, 3, 0, 7] = float("nan")
+    want = gpt_ref.forward(rt, nxt, cache)[:, -1]
+    got = model.forward_last(nxt.to(DEV), kv_cache=dec).cpu()
+    assert torch.isnan(want).all(), "the oracle itself should be all NaN here"
+    assert torch.isnan(got).all(), f"{(~torch.isnan(got)).sum().item()} finite logits left after a NaN key in the cache"
+
+
 def test_layer_by_layer_taps_against_the_oracle():
     """The residual stream as every layer reads it and every layer's attention output, HIP against the oracle, on a prefill
     and on a decode step.  Layer 0 sees identical inputs and must agree to bf16 rounding; deeper layers may drift no more than
