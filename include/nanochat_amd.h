@@ -68,7 +68,7 @@ int nc_fp8_transpose(const uint8_t* src, int rows, int cols, uint8_t* dst, nc_st
  * softcap*tanh(bf16(v)/softcap), i.e. lm_head followed by nanochat/gpt.py:512-515.
  * kernel: 0 auto, 1 small-M (M<=128), 4 plain-load tile 128x128 (any operand size), 5/6/7 buffer-load tiles
  * 128x128 / 256x128 / 256x256 (operands below 2 GiB each), 8 direct-to-LDS 256x256 tiles and 9 their persistent
- * form (bf16 output, K a multiple of 128; 9 also needs ceil(M/256) in {8,16,...,256}), 10 buffer-load tile 64x128.
+ * form (bf16 output, K a multiple of 128; 9 also needs ceil(M/256) in {8,16,...,256}), 10 / 11 buffer-load tiles 64x128 / 96x128.
  * workspace (may be NULL): lets the small-M kernel split K over workgroups (fp32 partial sums, added
  * in a fixed order by a finishing kernel); size from nc_fp8_small_m_workspace_bytes(), 16-byte aligned. */
 int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b,

@@ -969,7 +969,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     }
 
     // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256,
-    // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent, 10 buffer-load tile 64x128
+    // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent, 10 / 11 buffer-load tiles 64x128 / 96x128
     int which = force_kernel;
     if (which == 0) {
         if (M <= 128) which = 1;
@@ -989,15 +989,20 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
                 // 256x256 tiles move half the bytes per flop through L2 and LDS but run one workgroup per CU: take them
                 // when their count fills whole rounds of the CUs well, else the 128x128 tiles (two workgroups per CU)
                 which = (M >= 1024 && N >= 512 && 10 * t256 >= 8 * rounds * cus && rounds <= 2) ? 7 : 5;
-                // a short prompt against a narrow weight leaves half of the CUs without a 128x128 tile, and each tile's K loop is
-                // one dependent step after the other: half-height tiles put a workgroup on twice as many CUs with half the
-                // MFMA work per step (512..1024 rows x 1664 columns: 8 us against 10.7 at K = 1664, 21 against 31 at K = 6656)
-                if (which == 5 && 2 * t128 <= cus && out_kind != 2) which = 10;
+                // a prompt of a few hundred to two thousand rows against a narrow weight leaves CUs without a 128x128 tile, and each
+                // tile's K loop is one dependent step after the other: lower tiles put a workgroup on more CUs with less MFMA work per
+                // step, as long as they still fit one round of one workgroup per CU (512..1024 rows x 1664 columns with 64-row tiles:
+                // 8 us against 10.7 at K = 1664, 21 against 31 at K = 6656; 1792 rows with 96-row tiles: 10.0 / 11.5 and 27.9 / 30.5)
+                if (which == 5 && out_kind != 2) {
+                    const long tn = (N + 127) / 128;
+                    if ((long)((M + 63) / 64) * tn <= cus) which = 10;
+                    else if ((long)((M + 95) / 96) * tn <= cus) which = 11;
+                }
             }
         }
     }
     int rc = 0;
-    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 10, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 11, "fp8_gemm: unknown kernel selector %d", force_kernel);
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
@@ -1019,6 +1024,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     else if (which == 8) rc = launch_dl<0>(a, b, ep, M, N, K, false, s);
     else if (which == 9) rc = launch_dl<0>(a, b, ep, M, N, K, true, s);
     else if (which == 10) rc = launch_bl<64, 128, 2, 2, true>(a, b, ep, M, N, K, s);
+    else if (which == 11) rc = launch_bl<96, 128, 2, 2, true>(a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");

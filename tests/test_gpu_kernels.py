@@ -172,6 +172,7 @@ def make_operands(M, N, K, seed, outliers=True):
     (2048, 6656, 1664, 0), (8192, 4992, 256, 0),
     # half-height buffer-load tiles (what a short prompt's projections take): ragged M and N, K tail, the shapes of the choice
     (300, 320, 256, 10), (129, 72, 80, 10), (513, 1664, 1664, 10), (1000, 1664, 6656, 10), (512, 1664, 6656, 0), (1024, 1280, 1280, 0),
+    (300, 320, 256, 11), (193, 72, 80, 11), (1792, 1664, 1664, 11), (1792, 1664, 6656, 0),
 ])
 def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     say(f"gemm M={M} N={N} K={K} kernel={kernel}")
@@ -189,7 +190,7 @@ def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     assert rel_l2(got, exact) < 0.08
 
 
-@pytest.mark.parametrize("kernel,M", [(1, 48), (4, 128), (5, 256), (6, 128), (7, 256), (8, 256), (9, 2048), (10, 200)])
+@pytest.mark.parametrize("kernel,M", [(1, 48), (4, 128), (5, 256), (6, 128), (7, 256), (8, 256), (9, 2048), (10, 200), (11, 200)])
 def test_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
     say(f"gemm exact powers of two kernel={kernel}")
     g = torch.Generator().manual_seed(9)
@@ -237,7 +238,7 @@ def test_gemm_stacked_weights_use_their_own_scales(ops):
     a_big = torch.randn(2048, K, generator=g).bfloat16()
     a8b, iab, _ = fp8_ref.to_fp8(a_big)
     want_big = torch.cat([fp8_ref.scaled_mm_emulated(a8b, p, iab, inv) for p, inv, _ in q], dim=1)
-    for kernel in (5, 7, 8, 9, 10):
+    for kernel in (5, 7, 8, 9, 10, 11):
         got = ops.fp8_gemm(a8b.to(DEV), w8.to(DEV), iab.to(DEV), inv_w.to(DEV), seg_ends=[256, 384, 512], kernel=kernel).cpu()
         assert rel_l2(got, want_big) < 2e-3, kernel
 
