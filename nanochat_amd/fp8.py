@@ -115,4 +115,6 @@ def convert_to_float8_training(module, *, config=None, module_filter_fn=None):
                 if module_filter_fn is None or module_filter_fn(child, fqn):
                     setattr(mod, name, Float8Linear.from_float(child))
     walk(module)
+    if hasattr(module, "invalidate_plan"):      # a model that caches quantized weights per module starts over
+        module.invalidate_plan()
     return module

@@ -107,7 +107,10 @@ class GPT(nn.Module):
         self.rotary_seq_len = config.sequence_len * 10
         self._plan = None
         self._plan_key = None
+        self._plan_params = None
         self._workspaces = {}
+        # anything that replaces parameter tensors drops the weight plan (the per-call check below only looks at versions)
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module.invalidate_plan())
 
     # -------------------------------------------------------------------------------------------
     @torch.no_grad()
@@ -147,7 +150,7 @@ class GPT(nn.Module):
             self.transformer.wte.to(dtype=COMPUTE_DTYPE)
             for ve in self.value_embeds.values():
                 ve.to(dtype=COMPUTE_DTYPE)
-        self._plan = None
+        self.invalidate_plan()
 
     def get_device(self):
         return self.transformer.wte.weight.device
@@ -195,12 +198,24 @@ class GPT(nn.Module):
         mods.append(self.lm_head)
         return mods
 
+    def invalidate_plan(self):
+        """Forget the quantized-weight plan: the next forward rebuilds it.  Called by everything here that replaces parameter
+        tensors (load_state_dict, .to() / .cuda() / dtype casts, the FP8 module swap); call it after assigning a parameter by hand."""
+        self._plan = None
+        self._plan_params = None
+
+    def _apply(self, fn, recurse=True):
+        self.invalidate_plan()
+        return super()._apply(fn, recurse)
+
     def _current_plan_key(self):
-        key = []
-        for p in self.parameters():
-            key.append(p.data_ptr())
-            key.append(p._version)
-        return tuple(key)
+        """What the plan was built from, cheaply enough for every decode step: the storage addresses and in-place version counters
+        of the parameters seen when the plan was built (walking the module tree for them costs most of a millisecond at d26, a
+        kept list some tens of microseconds).  A parameter object replaced by another one is caught by invalidate_plan(), not here."""
+        params = self._plan_params
+        if params is None:
+            params = self._plan_params = list(self.parameters())
+        return tuple([(p._version, p.data_ptr()) for p in params])
 
     def _build_plan(self):
         """Quantize every FP8 linear once, stack q|k|v, and fill the C descriptors."""
@@ -272,7 +287,7 @@ class GPT(nn.Module):
         key = self._current_plan_key()
         if self._plan is None or key != self._plan_key:
             self._build_plan()
-            self._plan_key = key
+            self._plan_key = self._current_plan_key()
         return self._plan[0]
 
     def _workspace(self, md, B, T, device):
@@ -369,4 +384,4 @@ class GPT(nn.Module):
         assert not missing and not extra, f"state mismatch: missing {missing[:3]} extra {extra[:3]}"
         for k, v in state.items():
             own[k].copy_(v.to(own[k].dtype))
-        self._plan = None
+        self.invalidate_plan()

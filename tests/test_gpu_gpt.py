@@ -668,3 +668,43 @@ def test_full_size_d32_gqa_batch128_ragged_rows():
     rel = rel_l2(l4, logits[pick])
     print(f"d32 GQA: rows in a batch of 4 vs in the batch of 128: rel-L2 {rel:.4f}")
     assert rel < 0.1
+
+
+def test_weight_changes_are_noticed_by_the_next_forward():
+    """The quantized copies of the FP8 weights are cached between calls; every way of changing a weight that the module API offers
+    must refresh them: an in-place update, load_state_dict (copying and assigning), a cast of a child module, and the explicit call
+    for a parameter assigned by hand."""
+    say("weight plan refresh")
+    from nanochat_amd.engine import KVCache
+    cfg_kwargs = dict(sequence_len=64, vocab_size=512, n_layer=2, n_head=2, n_kv_head=2, n_embd=256, window_pattern="L")
+    _, model = build_pair(cfg_kwargs, seed=31)
+    ids = torch.arange(12, device=DEV).reshape(1, 12) * 5 % 512
+
+    def logits():
+        return model.forward_last(ids, kv_cache=KVCache(1, 2, 16, 128, 2, DEV, torch.bfloat16)).clone()
+    base = logits()
+    assert torch.equal(base, logits())                                   # cached plan, same answer
+    w = model.transformer.h[1].mlp.c_proj.weight
+    with torch.no_grad():
+        w.mul_(1.5)                                                      # in place: version counter
+    changed = logits()
+    assert not torch.equal(changed, base)
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    with torch.no_grad():
+        w.mul_(1.0 / 1.5)
+    restored = logits()
+    assert not torch.equal(restored, changed)
+    model.load_state_dict(state)                                         # copy into the existing tensors
+    assert torch.equal(logits(), changed)
+    with torch.no_grad():
+        w.mul_(1.0 / 1.5)
+    model.load_state_dict(state, assign=True)                            # new parameter objects
+    assert torch.equal(logits(), changed)
+    model.lm_head.weight = torch.nn.Parameter(model.lm_head.weight.detach() * 2.0)      # by hand: needs the explicit call
+    model.invalidate_plan()
+    doubled = logits()
+    assert not torch.equal(doubled, changed)
+    model.value_embeds.to(torch.float32)                                 # a child cast: same parameter objects, new storage
+    model.value_embeds.to(torch.bfloat16)
+    assert torch.equal(logits(), doubled)
+
