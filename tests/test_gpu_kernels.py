@@ -643,6 +643,29 @@ def test_kv_cache_prefill_copy(ops, src_rows, dst_rows, n):
     assert torch.equal(d.cpu(), want)
 
 
+def test_kv_cache_created_from_a_prefill_cache_equals_zeros_then_prefill():
+    """KVCache(..., prefill_from=src) skips the zero fill of what the copy overwrites; the tensors must come out as from
+    KVCache(...) + prefill(src), whatever the allocator hands back (the block is dirtied first)."""
+    say("kv cache prefill_from")
+    from nanochat_amd.engine import KVCache
+    g = torch.Generator().manual_seed(3)
+    L, Hkv, n, Td, B = 3, 2, 37, 100, 5
+    src = KVCache(1, Hkv, 64, 128, L, DEV, torch.bfloat16)
+    src.k_cache.copy_(torch.randn(src.k_cache.shape, generator=g).bfloat16())
+    src.v_cache.copy_(torch.randn(src.v_cache.shape, generator=g).bfloat16())
+    src.advance(n)
+    src.prev_embedding = torch.randn(1, 1, 16, generator=g).to(DEV)
+    want = KVCache(B, Hkv, Td, 128, L, DEV, torch.bfloat16)
+    want.prefill(src)
+    dirty = torch.full((2 * L * B * Td * Hkv * 128 + 4096,), 3.0, dtype=torch.bfloat16, device=DEV)
+    del dirty                                               # the caching allocator hands this block to the next request
+    got = KVCache(B, Hkv, Td, 128, L, DEV, torch.bfloat16, prefill_from=src)
+    assert torch.equal(got.k_cache, want.k_cache) and torch.equal(got.v_cache, want.v_cache)
+    assert torch.equal(got.cache_seqlens, want.cache_seqlens) and got.get_pos() == n
+    assert torch.equal(got.prev_embedding, want.prev_embedding)
+    assert not got.k_cache[:, :, n:].any() and not got.v_cache[:, :, n:].any()
+
+
 # ================================================================== (3) attention
 def attn_case(ops, B, T, H, Hkv, Tmax, seqlens, window, splits, seed=0):
     g = torch.Generator().manual_seed(seed)
