@@ -271,7 +271,9 @@ class Engine:
             if all(r.completed for r in rows):
                 break
             sampled_dev = sample_next_token(logits, rng, temperature, top_k)
-            run_ahead = ahead and not (max_tokens is not None and produced + 1 >= max_tokens)
+            # (not in front of the first token: the caller gets it as soon as it is sampled, as in the reference's loop, where the
+            # time to the first token ends before the first decode forward)
+            run_ahead = ahead and produced > 0 and not (max_tokens is not None and produced + 1 >= max_tokens)
             if run_ahead:
                 host_ids.copy_(sampled_dev[:, 0], non_blocking=True)
                 ids_ready.record()
