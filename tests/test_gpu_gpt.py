@@ -708,3 +708,51 @@ def test_weight_changes_are_noticed_by_the_next_forward():
     model.value_embeds.to(torch.bfloat16)
     assert torch.equal(logits(), doubled)
 
+
+def test_decode_step_captured_in_a_graph_replays_like_the_eager_step():
+    """The decode forward makes no allocation of its own, clears its counters with a kernel and reads positions from device memory,
+    so a caller may capture it in a HIP graph.  Replayed several times, with eager work and synchronisations in between, every replay
+    must give the logits and the cache of the eager step bit for bit."""
+    say("decode step under graph capture")
+    from nanochat_amd.engine import KVCache
+    cfg_kwargs = dict(sequence_len=64, vocab_size=1024, n_layer=3, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
+    _, model = build_pair(cfg_kwargs, seed=41)
+    B, P, steps = 4, 9, 5
+    g = torch.Generator().manual_seed(42)
+    prompt = torch.randint(0, 1024, (B, P), generator=g).to(DEV)
+    toks = [torch.randint(0, 1024, (B, 1), generator=g).to(DEV) for _ in range(steps)]
+
+    def fresh():
+        c = KVCache(B, 2, P + steps + 1, 128, 3, DEV, torch.bfloat16)
+        model.forward_last(prompt, kv_cache=c)
+        return c
+    eager, graphed, scratch = fresh(), fresh(), fresh()
+    static_idx = torch.zeros(B, 1, dtype=torch.long, device=DEV)
+    static_prev = graphed.prev_embedding.clone()          # the smear state lives in one buffer that the graph updates itself
+    graphed.prev_embedding = static_prev
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                           # warm-up of the step's workspace outside the capture
+        model.forward_last(toks[0], kv_cache=scratch)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_logits = model.forward_last(static_idx, kv_cache=graphed)
+        static_prev.copy_(graphed.prev_embedding)
+    graphed.prev_embedding = static_prev
+    # the capture advanced the host mirror of the position and, being a capture, nothing on the device
+    graphed._pos0 -= 1
+    graphed._pos_max -= 1
+    assert int(graphed.cache_seqlens[0]) == P
+    for step, tok in enumerate(toks):
+        want = model.forward_last(tok, kv_cache=eager).clone()     # the program's own eager work between the replays
+        torch.cuda.synchronize()
+        static_idx.copy_(tok)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_logits, want), f"replay {step}: max |diff| {(static_logits - want).abs().max().item()}"
+        assert torch.equal(graphed.cache_seqlens, eager.cache_seqlens)
+    assert torch.equal(graphed.k_cache[:, :, :P + steps], eager.k_cache[:, :, :P + steps])
+    assert torch.equal(graphed.v_cache[:, :, :P + steps], eager.v_cache[:, :, :P + steps])
+
