@@ -56,16 +56,29 @@ struct Carver {
 
 struct Workspace {
     bf16_t *x, *x0, *xn, *xb, *o, *qkv, *qh, *y, *h, *h2, *xl;
+    bf16_t* x2;                // second residual-stream buffer of the one- and two-row decode step (see fused_rows())
     uint8_t* a8;
     float* inv;
     uint32_t *amax, *attn_counters;
     // handle of amax site i (tagged: NC_AMAX_SLOTS words on separate lines, see amax_read / amax_publish)
     uint32_t* site(int i) const { return nc_amax_slotted(amax + (size_t)i * NC_AMAX_SLOTS * NC_AMAX_STRIDE); }
     int zero_words;
-    uint8_t *gemm_parts, *attn_parts;
+    uint8_t *gemm_parts, *gemm_parts2, *attn_parts;
     size_t gemm_part_bytes, attn_part_bytes;
     size_t total;
 };
+
+// One or two rows (a chat session's decode step): the residual/norm passes and the relu^2 pass are folded into the linears that consume
+// them (NcRowRecipe), five launches per layer instead of eight.  Each such linear reads its input recipe's partial sums from one
+// buffer and writes its own into the other, and the residual stream alternates between two buffers in the same way, because the
+// workgroups of one launch must not overwrite what their neighbours still read.
+bool fused_rows(const nc_model_desc* m, int M) {
+    const int E = m->n_embd, qkv_w = (m->n_head + 2 * m->n_kv_head) * 128;
+    if (M > NC_RECIPE_MAX_ROWS || E > 2048 || 4 * E > NC_RECIPE_MAX_K || E % 8 != 0) return false;
+    // every linear of a layer must leave split partial sums (the recipe of the next one reads them)
+    return nc_gemm_decode_splits(qkv_w, E) > 1 && nc_gemm_decode_splits(E, m->n_head * 128) > 1 && nc_gemm_decode_splits(4 * E, E) > 1 &&
+           nc_gemm_decode_splits(E, 4 * E) > 1;
+}
 
 Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     const size_t M = (size_t)B * T, E = m->n_embd;
@@ -74,6 +87,7 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     Carver c(base);
     Workspace w;
     w.x = c.take<bf16_t>(M * E);
+    w.x2 = c.take<bf16_t>(fused_rows(m, (int)M) ? M * E : 0);
     w.x0 = c.take<bf16_t>(M * E);
     w.xn = c.take<bf16_t>(M * E);
     w.xb = c.take<bf16_t>(M * E);
@@ -112,6 +126,7 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     }
     w.gemm_part_bytes = gneed;
     w.gemm_parts = c.take<uint8_t>(gneed);
+    w.gemm_parts2 = c.take<uint8_t>(fused_rows(m, (int)M) ? gneed : 0);
     w.attn_part_bytes = max_splits > 1 ? nc_attn_partial_bytes(B, T, m->n_head) / 16 * max_splits : 0;
     w.attn_parts = c.take<uint8_t>(w.attn_part_bytes);
     w.total = (c.off + 255) & ~(size_t)255;
@@ -139,20 +154,34 @@ int tap_copy(bf16_t* dst, const bf16_t* src, size_t elems, hipStream_t s) {
 struct LinearRunner {
     const Workspace& w;
     hipStream_t s;
+    // The same linear with its input rows made inside the kernel (one or two rows); the partial sums go to `parts_buf`.
+    int run_recipe(const NcRowRecipe& recipe, int rows, int site, const uint8_t* w8, const float* inv_w, NcGemmSegs segs, int N, int K,
+                   uint8_t* parts_buf, NcPartialSrc* src) const {
+        int used = 1;
+        const int want = nc_gemm_decode_splits(N, K);
+        // (a single split would need the epilogue in the GEMM; every linear of a layer splits K, and the recipe path relies on it)
+        NC_CHECK_ARG(want > 1, "gpt_forward: the fused small-batch step needs split linears (N=%d K=%d)", N, K);
+        TRY(nc_launch_gemm_decode(nullptr, 1, nullptr, nullptr, w8, inv_w, segs, nullptr, 0, 0.f, nullptr, rows, N, K, N, (float*)parts_buf,
+                                  w.gemm_part_bytes, want, &used, s, &recipe));
+        *src = NcPartialSrc{(const float*)parts_buf, used, N, (size_t)rows * N, w.site(site), inv_w,
+                            segs.nseg > 1 ? segs.end[0] : 0x7fffffff, segs.nseg > 2 ? segs.end[1] : 0x7fffffff};
+        return 0;
+    }
     int run(const bf16_t* in, int rows, int site, const uint8_t* w8, const float* inv_w, NcGemmSegs segs, void* out, int out_kind,
-            float softcap, uint32_t* out_amax, int N, int K, int ldc, NcPartialSrc* src) const {
+            float softcap, uint32_t* out_amax, int N, int K, int ldc, NcPartialSrc* src, uint8_t* parts_buf = nullptr) const {
         if (src) *src = NO_PARTIALS;
+        uint8_t* const pbuf = parts_buf ? parts_buf : w.gemm_parts;
         if (rows <= 128) {
             int used = 1;
             TRY(nc_launch_gemm_decode(in, 1, w.site(site), nullptr, w8, inv_w, segs, out, out_kind, softcap, out_amax, rows, N, K, ldc,
-                                      (float*)w.gemm_parts, w.gemm_part_bytes, src || out_kind == 2 ? 0 : 1, &used, s));
+                                      (float*)pbuf, w.gemm_part_bytes, src || out_kind == 2 ? 0 : 1, &used, s));
             if (used == 1) return 0;
             if (src) {
-                *src = NcPartialSrc{(const float*)w.gemm_parts, used, N, (size_t)rows * N, w.site(site), inv_w,
+                *src = NcPartialSrc{(const float*)pbuf, used, N, (size_t)rows * N, w.site(site), inv_w,
                                     segs.nseg > 1 ? segs.end[0] : 0x7fffffff, segs.nseg > 2 ? segs.end[1] : 0x7fffffff};
                 return 0;
             }
-            return nc_launch_finish_partials((const float*)w.gemm_parts, used, w.site(site), nullptr, inv_w, segs, out, out_kind, softcap,
+            return nc_launch_finish_partials((const float*)pbuf, used, w.site(site), nullptr, inv_w, segs, out, out_kind, softcap,
                                              out_amax, rows, N, ldc, s);
         }
         // large M: explicit convert pass, tiled GEMM; relu^2 (out_kind 2) is a separate kernel there
@@ -205,7 +234,59 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
         if (pending_parts.parts) return nc_launch_mix_norm_p(w.x, pending_parts, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
         return nc_launch_mix_norm(w.x, pending_add, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
     };
-    for (int i = 0; i < L; i++) {
+    // (measured at d26: one row 1.43 -> 1.3 ms per step; with two rows the row arithmetic done twice by every workgroup costs what the
+    // three launches save, so only one row takes this path)
+    const bool fused = T == 1 && M == 1 && fused_rows(m, M);
+    bf16_t *xcur = w.x, *xalt = w.x2;            // fused step: the residual stream alternates between the two
+    uint8_t *pin = w.gemm_parts, *pout = w.gemm_parts2;      // ... and so do the partial sums: pending_parts always sits in `pin`
+    for (int i = 0; i < L && fused; i++) {
+        const nc_layer_desc& ly = m->layers[i];
+        NC_CHECK_ARG(ly.w_qkv && ly.inv_qkv && ly.w_attn_proj && ly.w_fc && ly.w_mlp_proj, "gpt_forward: layer %d has no FP8 weights", i);
+        // q|k|v linear on rows it makes itself: x += mlp_out(prev layer); [save backout]; x = rl*x + xl*x0; xn = norm(x)
+        NcRowRecipe mix1{};
+        mix1.kind = 1, mix1.x_in = xcur, mix1.x_out = xalt, mix1.add = nullptr, mix1.padd = pending_parts, mix1.x0 = w.x0;
+        mix1.resid_lambda = m->resid_lambdas + i, mix1.x0_lambda = m->x0_lambdas + i;
+        mix1.save = (i > 0 && (i - 1) == L / 2) ? w.xb : nullptr, mix1.xn_out = w.xn, mix1.amax_out = w.site(site);
+        NcGemmSegs qkv_segs{3, {H * 128, (H + Hkv) * 128, qkv_w, 0}};
+        NcPartialSrc qsrc;
+        TRY(lin.run_recipe(mix1, M, site, ly.w_qkv, ly.inv_qkv, qkv_segs, qkv_w, E, pout, &qsrc));
+        { bf16_t* t = xcur; xcur = xalt; xalt = t; }
+        { uint8_t* t = pin; pin = pout; pout = t; }          // the q|k|v partial sums are in `pin` now
+        site++;
+        if (tap_x) TRY(tap_copy(tap_x + (size_t)i * M * E, xcur, (size_t)M * E, s));
+        bf16_t* kc = kv->k_cache + (size_t)i * layer_elems;
+        bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
+        const NcRopeSrc rope{nullptr, qkv_w, qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len, m->padded_vocab,
+                             nullptr, nullptr};
+        TRY(nc_launch_attention_fused(rope, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, H, Hkv, kv->max_seq_len, w.attn_counters,
+                                      w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s));
+        if (tap_y) TRY(tap_copy(tap_y + (size_t)i * M * H * 128, w.y, (size_t)M * H * 128, s));
+        // attention c_proj reads y as before; its partial sums go to the other buffer (the q|k|v ones are consumed by now)
+        TRY(lin.run(w.y, M, site, ly.w_attn_proj, ly.inv_attn_proj, one_seg(E), w.o, 0, 0.f, nullptr, E, H * 128, E, &pending_parts, pout));
+        NC_CHECK_ARG(pending_parts.parts, "gpt_forward: the fused small-batch step needs a split attention projection");
+        { uint8_t* t = pin; pin = pout; pout = t; }
+        site++;
+        // c_fc on rows it makes itself: x += attn_out; xn = norm(x)
+        NcRowRecipe mix2{};
+        mix2.kind = 1, mix2.x_in = xcur, mix2.x_out = xalt, mix2.padd = pending_parts, mix2.xn_out = w.xn, mix2.amax_out = w.site(site);
+        NcPartialSrc fsrc;
+        TRY(lin.run_recipe(mix2, M, site, ly.w_fc, ly.inv_fc, one_seg(4 * E), 4 * E, E, pout, &fsrc));
+        { bf16_t* t = xcur; xcur = xalt; xalt = t; }
+        { uint8_t* t = pin; pin = pout; pout = t; }
+        site++;
+        // MLP projection on rows it makes itself: h2 = relu(c_fc(xn))^2
+        NcRowRecipe act{};
+        act.kind = 2, act.padd = fsrc, act.amax_out = w.site(site);
+        TRY(lin.run_recipe(act, M, site, ly.w_mlp_proj, ly.inv_mlp_proj, one_seg(E), E, 4 * E, pout, &pending_parts));
+        { uint8_t* t = pin; pin = pout; pout = t; }
+        site++;
+    }
+    if (fused && xcur != w.x) {
+        // the last pass below works on w.x
+        const hipError_t e = hipMemcpyAsync(w.x, xcur, (size_t)M * E * sizeof(bf16_t), hipMemcpyDeviceToDevice, s);
+        if (e != hipSuccess) NC_FAIL(-2, "gpt_forward: copy of the residual rows failed: %s", hipGetErrorString(e));
+    }
+    for (int i = 0; i < L && !fused; i++) {
         const nc_layer_desc& ly = m->layers[i];
         NC_CHECK_ARG(ly.w_qkv && ly.inv_qkv && ly.w_attn_proj && ly.w_fc && ly.w_mlp_proj, "gpt_forward: layer %d has no FP8 weights", i);
         // x += mlp_out(prev layer); [save backout]; x = rl*x + xl*x0; xn = norm(x)

@@ -20,6 +20,7 @@
 //            2 bf16 relu(bf16(v))^2 plus atomic amax of the result (MLP activation, gpt.py:139).
 #include "nc_common.h"
 #include "nc_kernels.h"
+#include "nc_rope.h"
 
 #define MFMA_F8(acc, b, a) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4((b), (a), (acc), 0, 0, 0, 0, 0, 0)
 
@@ -38,6 +39,7 @@ struct DecodeGemmArgs {
     float* partial_out;       // ksplits > 1: [ksplits][M][N] raw fp32 sums
     int ksplits, ksteps_per_split;
     int M, N, K;
+    NcRowRecipe recipe;       // A_MODE 2
 };
 
 __device__ __forceinline__ float dg_seg_scale(const DecodeGemmArgs& g, int col) {
@@ -48,12 +50,180 @@ __device__ __forceinline__ float dg_seg_scale(const DecodeGemmArgs& g, int col) 
     return g.inv_b[s];
 }
 
-template <int MB, bool A_BF16>
+// The rows of A from a recipe, as bf16 in `rowbuf` ([M][K]); returns their amax.  Thread t owns elements 8t .. 8t+7 (+2048 per further
+// pass) of a row, the mapping of mix_norm_vec_kernel, and every sum runs in that kernel's order.  Everything a row needs is asked for
+// before anything is waited for (the work is a trip to memory and two reductions; the trips are what it costs).
+template <int KIND>
+__device__ __forceinline__ float recipe_rows(const NcRowRecipe& r, bf16_t* rowbuf, float* red, int M, int K, bool writer) {
+    const int tid = threadIdx.x;
+    const bool has_parts = r.padd.parts != nullptr;
+    const uint32_t p_amax_lane = has_parts ? amax_load_lane(r.padd.a_amax) : 0u;
+    const float p_inv_b = has_parts ? r.padd.inv_b[0] : 0.f;
+    float am = 0.f;
+    if (KIND == 1) {
+        const float rl_raw = r.resid_lambda ? *r.resid_lambda : 0.f, xl_raw = r.x0_lambda ? *r.x0_lambda : 0.f;
+        const int c = tid * 8;
+        const bool live = c < K;                     // K <= 2048: one pass
+        for (int m = 0; m < M; m++) {
+            const size_t at = (size_t)m * K + (live ? c : 0);
+            uint4 xv = make_uint4(0, 0, 0, 0), av = xv, zv = xv;
+            float4 a0[8], a1[8];
+            if (live) {
+                xv = *(const uint4*)(r.x_in + at);
+                if (r.add) av = *(const uint4*)(r.add + at);
+                if (r.resid_lambda) zv = *(const uint4*)(r.x0 + at);
+                if (has_parts) {
+                    const float* pp = r.padd.parts + (size_t)m * r.padd.ld + c;
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const float* q = pp + (size_t)(u < r.padd.nsplit ? u : 0) * r.padd.split_stride;
+                        a0[u] = *(const float4*)q;
+                        a1[u] = *(const float4*)(q + 4);
+                    }
+                }
+            }
+            const float p_inv_a = has_parts ? 1.0f / scale_from_amax(amax_from_lanes(p_amax_lane)) : 0.f;
+            const float rl = rbf(rl_raw), xl = rbf(xl_raw);
+            float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            float ss = 0.f;
+            if (live) {
+                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[2 * j] = bf16_lo(xw[j]), v[2 * j + 1] = bf16_hi(xw[j]);
+                if (r.add) {
+                    const uint32_t aw[4] = {av.x, av.y, av.z, av.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        v[2 * j] = rbf(v[2 * j] + bf16_lo(aw[j]));
+                        v[2 * j + 1] = rbf(v[2 * j + 1] + bf16_hi(aw[j]));
+                    }
+                }
+                if (has_parts) {
+                    float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        if (u < r.padd.nsplit) {
+                            acc8[0] += a0[u].x, acc8[1] += a0[u].y, acc8[2] += a0[u].z, acc8[3] += a0[u].w;
+                            acc8[4] += a1[u].x, acc8[5] += a1[u].y, acc8[6] += a1[u].z, acc8[7] += a1[u].w;
+                        }
+                    }
+                    const float* pp = r.padd.parts + (size_t)m * r.padd.ld + c;
+                    for (int sp0 = 8; sp0 < r.padd.nsplit; sp0 += 8) {
+                        float4 b0[8], b1[8];
+#pragma unroll
+                        for (int u = 0; u < 8; u++) {
+                            const float* q = pp + (size_t)(sp0 + u < r.padd.nsplit ? sp0 + u : sp0) * r.padd.split_stride;
+                            b0[u] = *(const float4*)q;
+                            b1[u] = *(const float4*)(q + 4);
+                        }
+#pragma unroll
+                        for (int u = 0; u < 8; u++) {
+                            if (sp0 + u < r.padd.nsplit) {
+                                acc8[0] += b0[u].x, acc8[1] += b0[u].y, acc8[2] += b0[u].z, acc8[3] += b0[u].w;
+                                acc8[4] += b1[u].x, acc8[5] += b1[u].y, acc8[6] += b1[u].z, acc8[7] += b1[u].w;
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = rbf(v[j] + rbf((acc8[j] * p_inv_a) * p_inv_b));
+                }
+                if (r.save && writer)
+                    *(uint4*)(r.save + at) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+                if (r.resid_lambda) {
+                    const uint32_t zw[4] = {zv.x, zv.y, zv.z, zv.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        v[2 * j] = rbf(rbf(rl * v[2 * j]) + rbf(xl * bf16_lo(zw[j])));
+                        v[2 * j + 1] = rbf(rbf(rl * v[2 * j + 1]) + rbf(xl * bf16_hi(zw[j])));
+                    }
+                }
+                if (writer)
+                    *(uint4*)(r.x_out + at) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+#pragma unroll
+                for (int j = 0; j < 8; j++) ss += v[j] * v[j];
+            }
+            ss = block_sum<4>(ss, red);
+            const float rstd = 1.0f / sqrtf(ss / (float)K + RMS_EPS);
+            if (live) {
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    o[j] = pack_bf16(v[2 * j] * rstd, v[2 * j + 1] * rstd);
+                    am = amax_fold(amax_fold(am, bf16_lo(o[j])), bf16_hi(o[j]));
+                }
+                const uint4 ov = make_uint4(o[0], o[1], o[2], o[3]);
+                *(uint4*)(rowbuf + (size_t)m * K + c) = ov;
+                if (writer && r.xn_out) *(uint4*)(r.xn_out + (size_t)m * K + c) = ov;
+            }
+        }
+    } else {
+        // at most four passes of 2048 elements per row (K <= 8192); the partial sums of all of them are asked for at once when the
+        // linear was split in two (the c_fc of a decode step), else pass by pass
+        const bool two = r.padd.nsplit == 2;
+        for (int m = 0; m < M; m++) {
+            const float* pp = r.padd.parts + (size_t)m * r.padd.ld;
+            float4 q0[4][2], q1[4][2];
+            if (two) {
+#pragma unroll
+                for (int ps = 0; ps < 4; ps++) {
+                    const int c = tid * 8 + 2048 * ps;
+                    const float* q = pp + (c < K ? c : 0);
+                    q0[ps][0] = *(const float4*)q, q1[ps][0] = *(const float4*)(q + 4);
+                    q0[ps][1] = *(const float4*)(q + r.padd.split_stride), q1[ps][1] = *(const float4*)(q + r.padd.split_stride + 4);
+                }
+            }
+            const float p_inv_a = 1.0f / scale_from_amax(amax_from_lanes(p_amax_lane));
+#pragma unroll
+            for (int ps = 0; ps < 4; ps++) {
+                const int c = tid * 8 + 2048 * ps;
+                if (c < K) {
+                    float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    if (two) {
+#pragma unroll
+                        for (int u = 0; u < 2; u++) {
+                            acc8[0] += q0[ps][u].x, acc8[1] += q0[ps][u].y, acc8[2] += q0[ps][u].z, acc8[3] += q0[ps][u].w;
+                            acc8[4] += q1[ps][u].x, acc8[5] += q1[ps][u].y, acc8[6] += q1[ps][u].z, acc8[7] += q1[ps][u].w;
+                        }
+                    } else {
+                        for (int sp = 0; sp < r.padd.nsplit; sp++) {
+                            const float* q = pp + (size_t)sp * r.padd.split_stride + c;
+                            const float4 b0 = *(const float4*)q, b1 = *(const float4*)(q + 4);
+                            acc8[0] += b0.x, acc8[1] += b0.y, acc8[2] += b0.z, acc8[3] += b0.w;
+                            acc8[4] += b1.x, acc8[5] += b1.y, acc8[6] += b1.z, acc8[7] += b1.w;
+                        }
+                    }
+                    float h[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const float t = relu_keep_nan(rbf((acc8[j] * p_inv_a) * p_inv_b));
+                        h[j] = rbf(t * t);
+                        am = amax_join(am, h[j]);
+                    }
+                    *(uint4*)(rowbuf + (size_t)m * K + c) = make_uint4(pack_bf16(h[0], h[1]), pack_bf16(h[2], h[3]), pack_bf16(h[4], h[5]), pack_bf16(h[6], h[7]));
+                }
+            }
+        }
+    }
+    am = wave_amax(am);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = am;
+    __syncthreads();
+    am = amax_join(amax_join(red[0], red[1]), amax_join(red[2], red[3]));
+    if (writer && tid == 0) amax_publish(r.amax_out, am);
+    __syncthreads();                                   // the rows are complete in LDS, `red` is free again
+    return am;
+}
+
+// A_MODE 0: A is e4m3 with its inverse scale; 1: bf16 with the amax word of its producer; 2 / 3: made by the kernel from a recipe of
+// kind 1 / 2.
+template <int MB, int A_MODE>
 __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
+    constexpr bool A_BF16 = A_MODE != 0;
     constexpr int ROWS = MB * 16;
     constexpr int A_CH = ROWS * 32 / 256;          // 16-byte LDS chunks per thread per 512-wide sub-chunk
     __shared__ __align__(16) uint8_t lds[2][ROWS * 512];
-    __shared__ float red[4];
+    __shared__ float red[8];
+    __shared__ __align__(16) bf16_t rowbuf[A_MODE == 2 ? NC_RECIPE_MAX_ROWS * 2048 : (A_MODE == 3 ? NC_RECIPE_MAX_ROWS * NC_RECIPE_MAX_K : 8)];
 
     NC_ARG_NOW(g.A); NC_ARG_NOW(g.a_amax); NC_ARG_NOW(g.inv_a); NC_ARG_NOW(g.B); NC_ARG_NOW(g.partial_out); NC_ARG_NOW(g.ksplits);
     NC_ARG_NOW(g.ksteps_per_split); NC_ARG_NOW(g.M); NC_ARG_NOW(g.N); NC_ARG_NOW(g.K);
@@ -73,7 +243,7 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
     const int k_hi = (ks_end << 7) < K ? (ks_end << 7) : K;       // exclusive K bound of this split
 
     // the activation scale is asked for here and looked at only after the first operand loads are on their way
-    const uint32_t amax_lane = A_BF16 ? amax_load_lane(g.a_amax) : 0u;
+    const uint32_t amax_lane = A_MODE == 1 ? amax_load_lane(g.a_amax) : 0u;
     float scale = 1.f, inv_a = A_BF16 ? 0.f : *g.inv_a;
 
     v4f acc[MB];
@@ -89,7 +259,11 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
             const int id = tid + c * 256, row = id >> 5, ch = id & 31;
             const int gk = k0 + ch * 16;
             const bool ok = row < M && gk < k_hi;
-            if (A_BF16) {
+            if (A_MODE >= 2) {
+                const uint4* p = (const uint4*)(rowbuf + (ok ? (size_t)row * K + gk : 0));
+                ra[c][0] = ok ? p[0] : make_uint4(0, 0, 0, 0);
+                ra[c][A_BF16 ? 1 : 0] = ok ? p[1] : make_uint4(0, 0, 0, 0);
+            } else if (A_BF16) {
                 const uint4* p = (const uint4*)((const bf16_t*)g.A + (size_t)row * K + gk);
                 ra[c][0] = ok ? p[0] : make_uint4(0, 0, 0, 0);
                 ra[c][A_BF16 ? 1 : 0] = ok ? p[1] : make_uint4(0, 0, 0, 0);
@@ -154,11 +328,14 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
         }
     };
     {
-        if (nsub > 0) {
-            load_b(kbase, 0);
-            load_a(kbase);
+        if (nsub > 0) load_b(kbase, 0);
+        if (A_MODE >= 2) {
+            // the weights are on their way while the rows are made
+            scale = scale_from_amax(recipe_rows<A_MODE - 1>(g.recipe, rowbuf, red, M, K, blockIdx.x == 0 && blockIdx.y == 0));
+            inv_a = 1.0f / scale;
         }
-        if (A_BF16) {
+        if (nsub > 0) load_a(kbase);
+        if (A_MODE == 1) {
             scale = scale_from_amax(amax_from_lanes(amax_lane));
             inv_a = 1.0f / scale;
         }
@@ -351,9 +528,19 @@ size_t nc_gemm_decode_partial_bytes(int M, int N, int K) {
 // ([ksplits][M][N] fp32, raw sums) and *ksplits_out says how many; out/out_kind are then unused.
 int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
                           const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
-                          int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s) {
-    NC_CHECK_ARG(a && b, "fp8_gemm(decode): null pointer");
-    NC_CHECK_ARG(a_is_bf16 ? (a_amax != nullptr) : (inv_a != nullptr), "fp8_gemm(decode): activation scale missing");
+                          int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s,
+                          const NcRowRecipe* recipe) {
+    const bool made = recipe && recipe->kind != 0;
+    NC_CHECK_ARG((a || made) && b, "fp8_gemm(decode): null pointer");
+    NC_CHECK_ARG(made || (a_is_bf16 ? (a_amax != nullptr) : (inv_a != nullptr)), "fp8_gemm(decode): activation scale missing");
+    if (made) {
+        NC_CHECK_ARG(M <= NC_RECIPE_MAX_ROWS && K % 8 == 0 && K <= (recipe->kind == 1 ? 2048 : NC_RECIPE_MAX_K) && recipe->amax_out,
+                     "fp8_gemm(decode): a row recipe takes at most %d rows of at most %d elements", NC_RECIPE_MAX_ROWS, NC_RECIPE_MAX_K);
+        NC_CHECK_ARG(recipe->kind == 1 ? (recipe->x_in && recipe->x_out && recipe->x_in != recipe->x_out && (!recipe->resid_lambda || (recipe->x0 && recipe->x0_lambda)))
+                                       : (recipe->kind == 2 && recipe->padd.parts), "fp8_gemm(decode): incomplete row recipe");
+        NC_CHECK_ARG(!recipe->padd.parts || (recipe->padd.nsplit >= 1 && recipe->padd.a_amax && recipe->padd.inv_b && recipe->padd.ld >= K),
+                     "fp8_gemm(decode): bad partial-sum source in the row recipe");
+    }
     NC_CHECK_ARG(M >= 1 && M <= 128 && N > 0 && K > 0, "fp8_gemm(decode): bad shape M=%d N=%d K=%d (M <= 128)", M, N, K);
     NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
     NC_CHECK_ARG(((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0, "fp8_gemm: operands must be 16-byte aligned");
@@ -379,20 +566,24 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     }
     if (ksplits_out) *ksplits_out = ksplits;
 
-    const int MB = M <= 64 ? 4 : 8;
+    const int MB = made ? 1 : (M <= 64 ? 4 : 8);
     const int nblk = (N + 63) / 64;
     DecodeGemmArgs g;
     g.A = a, g.a_amax = a_amax, g.inv_a = inv_a, g.B = b, g.inv_b = inv_b, g.segs = segs, g.out = out, g.out_kind = out_kind;
     g.softcap = softcap, g.ldc = ldc, g.out_amax = out_amax, g.partial_out = partials;
     g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
+    g.recipe = made ? *recipe : NcRowRecipe{};
     NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
     dim3 grid(nblk, ksplits), block(256);
-    if (MB == 4) {
-        if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<4, true>), grid, block, 0, s, g);
-        else hipLaunchKernelGGL((gemm_decode_kernel<4, false>), grid, block, 0, s, g);
+    if (MB == 1) {
+        if (recipe->kind == 1) hipLaunchKernelGGL((gemm_decode_kernel<1, 2>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((gemm_decode_kernel<1, 3>), grid, block, 0, s, g);
+    } else if (MB == 4) {
+        if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<4, 1>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((gemm_decode_kernel<4, 0>), grid, block, 0, s, g);
     } else {
-        if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<8, true>), grid, block, 0, s, g);
-        else hipLaunchKernelGGL((gemm_decode_kernel<8, false>), grid, block, 0, s, g);
+        if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<8, 1>), grid, block, 0, s, g);
+        else hipLaunchKernelGGL((gemm_decode_kernel<8, 0>), grid, block, 0, s, g);
     }
     NC_CHECK_LAUNCH("fp8_gemm(decode)");
     return 0;

@@ -32,12 +32,14 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
 // small-M path (nc_gemm_decode.hip): A is e4m3 (+inv_a) or bf16 (+amax, quantized inside the kernel)
 // out_kind: 0 bf16, 1 softcapped fp32, 2 bf16 relu^2 with amax of the result into out_amax.
 // With K split over workgroups the raw fp32 sums land in `partials` [ksplits][M][N] and a consumer finishes them.
+struct NcRowRecipe;
 int nc_gemm_decode_splits(int N, int K);
 size_t nc_gemm_decode_partial_bytes(int M, int N, int K);        // any split count up to 16
 size_t nc_gemm_decode_partial_bytes_auto(int M, int N, int K);   // the split count nc_gemm_decode_splits() picks
 int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, const float* inv_a, const uint8_t* b,
                           const float* inv_b, NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M,
-                          int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s);
+                          int N, int K, int ldc, float* partials, size_t partial_bytes, int ksplits, int* ksplits_out, hipStream_t s,
+                          const NcRowRecipe* recipe = nullptr);     // rows made inside the kernel instead of read from `a`
 int nc_launch_finish_partials(const float* parts, int nsplit, const uint32_t* a_amax, const float* inv_a, const float* inv_b,
                               NcGemmSegs segs, void* out, int out_kind, float softcap, uint32_t* out_amax, int M, int N, int ldc,
                               hipStream_t s);
@@ -52,6 +54,26 @@ struct NcPartialSrc {
     const uint32_t* a_amax;
     const float* inv_b;       // one per segment
     int seg_end0, seg_end1;   // column ends of segments 0 and 1 (INT_MAX when there is a single segment)
+};
+
+// How the rows of a small-M linear's input come to be, when the kernel that used to make them is folded into the linear.  For one or
+// two rows every workgroup of the GEMM repeats the row arithmetic for itself (a few KB from L2, a few hundred instructions), which
+// costs less than the launch it saves; one workgroup also stores what other kernels read (the residual stream, the normalised rows,
+// the amax).  The arithmetic and its order are those of mix_norm / finish_partials, so the results are the same bits.
+#define NC_RECIPE_MAX_ROWS 2
+#define NC_RECIPE_MAX_K 8192
+struct NcRowRecipe {
+    int kind;                   // 0 none; 1 residual add + lambda mix + norm (mix_norm); 2 relu(.)^2 of a split linear (finish_partials)
+    const bf16_t* x_in;         // kind 1: the residual stream [M,K] as it is ...
+    bf16_t* x_out;              //         ... and where its new value goes (another buffer: the other workgroups still read x_in)
+    const bf16_t* add;          //         a bf16 addend, or
+    NcPartialSrc padd;          //         split partial sums to add (kind 2: the linear whose relu^2 the rows are)
+    const bf16_t* x0;           //         with resid_lambda / x0_lambda: x = rl * x + xl * x0
+    const float* resid_lambda;
+    const float* x0_lambda;
+    bf16_t* save;               //         copy of x before the lambda mix (the backout rows), or null
+    bf16_t* xn_out;             //         the normalised rows, for whoever reads them besides this GEMM
+    uint32_t* amax_out;         // the site that receives the amax of the rows
 };
 
 // ---- elementwise / norm / rope (nc_elementwise.hip)

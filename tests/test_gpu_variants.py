@@ -253,6 +253,49 @@ def test_one_layer_models_against_the_oracle(cfg_kwargs, B):
         assert ulps <= 4 and frac < 0.02, (frac, ulps)
 
 
+@pytest.mark.parametrize("cfg_kwargs", [
+    dict(sequence_len=64, vocab_size=1024, n_layer=4, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL"),
+    dict(sequence_len=64, vocab_size=2048, n_layer=3, n_head=13, n_kv_head=13, n_embd=1664, window_pattern="SSL"),
+    dict(sequence_len=64, vocab_size=1024, n_layer=6, n_head=2, n_kv_head=2, n_embd=256, window_pattern="L"),
+])
+def test_one_and_two_row_decode_steps_equal_the_same_rows_in_a_larger_batch(cfg_kwargs):
+    """With one or two rows the residual/norm passes and the relu^2 pass run inside the linears that consume them (five launches per
+    layer instead of eight).  The arithmetic and its order are unchanged, so the logits and the cache must be, bit for bit, those of
+    the same rows decoded as part of a four-row batch that holds each of them twice (same tensorwise amax, eight launches per layer)."""
+    say(f"fused small-batch step {cfg_kwargs['n_embd']}/{cfg_kwargs['n_layer']} layers")
+    from nanochat_amd.engine import KVCache
+    rt, model = build_pair(cfg_kwargs, seed=29)
+    cfg = rt.cfg
+    g = torch.Generator().manual_seed(30)
+    P, steps = 7, 5
+    for B in (1, 2):
+        prompt = torch.randint(0, cfg.vocab_size, (B, P), generator=g)
+        nxts = [torch.randint(0, cfg.vocab_size, (B, 1), generator=g) for _ in range(steps)]
+        small = KVCache(B, cfg.n_kv_head, P + steps, 128, cfg.n_layer, DEV, torch.bfloat16)
+        big = KVCache(4, cfg.n_kv_head, P + steps, 128, cfg.n_layer, DEV, torch.bfloat16)
+        rep = 4 // B
+        model.forward_last(prompt.to(DEV), kv_cache=small)
+        model.forward_last(prompt.repeat(rep, 1).to(DEV), kv_cache=big)
+        for step, nxt in enumerate(nxts):
+            got = model.forward_last(nxt.to(DEV), kv_cache=small)
+            want = model.forward_last(nxt.repeat(rep, 1).to(DEV), kv_cache=big)[:B]
+            assert torch.equal(got, want), f"B={B} step {step}: max |diff| {(got - want).abs().max().item()}"
+        assert torch.equal(small.k_cache, big.k_cache[:, :B]) and torch.equal(small.v_cache, big.v_cache[:, :B])
+    # and against the oracle, like every other path
+    B = 2
+    prompt = torch.randint(0, cfg.vocab_size, (B, P), generator=g)
+    nxts = [torch.randint(0, cfg.vocab_size, (B, 1), generator=g) for _ in range(3)]
+    rt_def = gpt_ref.Runtime(cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+
+    def run(r):
+        c = decode_ref.new_cache(cfg, B, P + 3, torch.bfloat16)
+        return torch.stack([gpt_ref.forward(r, prompt, c)[:, -1]] + [gpt_ref.forward(r, nxt, c)[:, -1] for nxt in nxts])
+    floor_rel, floor_max, want, want_def = oracle_floor(rt, run)
+    dec = KVCache(B, cfg.n_kv_head, P + 3, 128, cfg.n_layer, DEV, torch.bfloat16)
+    got = torch.stack([model.forward_last(prompt.to(DEV), kv_cache=dec).cpu()] + [model.forward_last(nxt.to(DEV), kv_cache=dec).cpu() for nxt in nxts])
+    assert_within_floor(got, want, want_def, floor_rel, floor_max, "fused small-batch step")
+
+
 @pytest.mark.parametrize("where", ["embedding", "cache"])
 def test_a_nan_activation_reaches_every_logit_as_in_the_reference(where):
     """x.abs().max() of a tensor that holds a NaN is NaN (nanochat/fp8.py:92), so the scale of the next FP8 linear is NaN and with it
