@@ -709,15 +709,16 @@ def test_weight_changes_are_noticed_by_the_next_forward():
     assert torch.equal(logits(), doubled)
 
 
-def test_decode_step_captured_in_a_graph_replays_like_the_eager_step():
+@pytest.mark.parametrize("B", [4, 1])
+def test_decode_step_captured_in_a_graph_replays_like_the_eager_step(B):
     """The decode forward makes no allocation of its own, clears its counters with a kernel and reads positions from device memory,
     so a caller may capture it in a HIP graph.  Replayed several times, with eager work and synchronisations in between, every replay
     must give the logits and the cache of the eager step bit for bit."""
-    say("decode step under graph capture")
+    say(f"decode step under graph capture, {B} row(s)")
     from nanochat_amd.engine import KVCache
     cfg_kwargs = dict(sequence_len=64, vocab_size=1024, n_layer=3, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
     _, model = build_pair(cfg_kwargs, seed=41)
-    B, P, steps = 4, 9, 5
+    P, steps = 9, 5
     g = torch.Generator().manual_seed(42)
     prompt = torch.randint(0, 1024, (B, P), generator=g).to(DEV)
     toks = [torch.randint(0, 1024, (B, 1), generator=g).to(DEV) for _ in range(steps)]
