@@ -234,9 +234,8 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
         if (pending_parts.parts) return nc_launch_mix_norm_p(w.x, pending_parts, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
         return nc_launch_mix_norm(w.x, pending_add, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
     };
-    // (measured at d26: one row 1.43 -> 1.3 ms per step; with two rows the row arithmetic done twice by every workgroup costs what the
-    // three launches save, so only one row takes this path)
-    const bool fused = T == 1 && M == 1 && fused_rows(m, M);
+    // (measured at d26, steps without a synchronisation in between: one row 1.30 -> 1.13 ms, two rows 1.37 -> 1.27 ms)
+    const bool fused = T == 1 && fused_rows(m, M);
     bf16_t *xcur = w.x, *xalt = w.x2;            // fused step: the residual stream alternates between the two
     uint8_t *pin = w.gemm_parts, *pout = w.gemm_parts2;      // ... and so do the partial sums: pending_parts always sits in `pin`
     for (int i = 0; i < L && fused; i++) {
