@@ -257,6 +257,8 @@ def test_one_layer_models_against_the_oracle(cfg_kwargs, B):
     dict(sequence_len=64, vocab_size=1024, n_layer=4, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL"),
     dict(sequence_len=64, vocab_size=2048, n_layer=3, n_head=13, n_kv_head=13, n_embd=1664, window_pattern="SSL"),
     dict(sequence_len=64, vocab_size=1024, n_layer=6, n_head=2, n_kv_head=2, n_embd=256, window_pattern="L"),
+    # the widest model the row recipes take: a full 2048-element pass for the norm, four for the relu^2 rows
+    dict(sequence_len=64, vocab_size=1024, n_layer=2, n_head=16, n_kv_head=4, n_embd=2048, window_pattern="SL"),
 ])
 def test_one_and_two_row_decode_steps_equal_the_same_rows_in_a_larger_batch(cfg_kwargs):
     """With one or two rows the residual/norm passes and the relu^2 pass run inside the linears that consume them (five launches per
