@@ -9,7 +9,15 @@
  *     failure on the calling thread (the Python host re-raises it as AssertionError/ValueError,
  *     which is how the reference reports the same conditions);
  *   - bf16 tensors are raw uint16_t bit patterns, e4m3 tensors raw uint8_t (OCP e4m3fn, the
- *     encoding of torch.float8_e4m3fn).
+ *     encoding of torch.float8_e4m3fn);
+ *   - re-entrancy: every entry point may be called from any thread on any stream, and keeps no state between
+ *     calls beyond per-process caches of device facts (CU count, LDS attributes, occupancy), with TWO
+ *     exceptions, both process-wide and not thread-safe: the measurement aid (nc_profile_*: one set of event
+ *     pairs and counters per process, to be switched on by one thread while no other thread launches), and
+ *     nc_decode_attention_static (one scratch array per GPU shared by all its calls: calls on one GPU must not
+ *     overlap in time, whatever stream or thread they come from).  A caller-provided state or workspace block
+ *     (quantizer state, split workspaces, the forward's workspace) serves one call at a time: calls that may
+ *     overlap need a block each.
  */
 #ifndef NANOCHAT_AMD_H
 #define NANOCHAT_AMD_H
@@ -48,12 +56,20 @@ int nc_fp8_encode_with_scale(const uint16_t* x, int64_t n, float scale, int fp8_
  * elements: what the registers of the workgroups resident on the chip hold): every element is read from memory once, the
  * workgroups meet on the tensor's amax, the payload is converted from registers.  Other tensors take the two passes of
  * nc_fp8_quantize_tensorwise_as; results are bit-identical either way.  state: nc_fp8_quantize_state_bytes() bytes, 128-byte
- * aligned, ALL ZERO before the first call with it; every call leaves it all zero (word 320 excepted, which is scratch),
- * so one allocation serves all calls that do not overlap in time.  If the on-chip meeting ever timed out (it cannot while the
- * device runs this library's kernels alone) the scale comes out as NaN and word 257 of the state stays set. */
+ * aligned, ALL ZERO before the first call with it; every call leaves it all zero (words 257 and 320 excepted, see below),
+ * so one allocation serves all calls that do not overlap in time; calls that overlap need a state each.  The one-launch grid
+ * is sized to half of what the GPU holds of it, so that two such grids at once (of this or any other process on the GPU) are
+ * both resident; with more of them at once a workgroup can wait for peers that have no slot yet.  That wait is bounded: a
+ * workgroup whose wait runs out works the amax out by itself from the whole tensor (slow, same bits) and is counted in word
+ * 257 of the state, which no kernel reads or clears -- a host that wants to know reads it; the results are correct either way.
+ * Word 320 is scratch of the two-pass path. */
 size_t nc_fp8_quantize_state_bytes(void);
 int nc_fp8_quantize_tensorwise_fused(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
                                      float* inv_scale_out, void* state, int encoder, nc_stream_t stream);
+/* The same with the bound of the wait given by the caller: spin_limit polls of a few hundred nanoseconds each (the entry above
+ * uses about four million).  0 makes nearly every workgroup take the slow way at once, which is how that way is tested. */
+int nc_fp8_quantize_tensorwise_fused_bounded(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
+                                             float* inv_scale_out, void* state, int encoder, uint32_t spin_limit, nc_stream_t stream);
 
 /* dst[cols][rows] = transpose of the fp8 payload src[rows][cols]: the memory rearrangement of _to_col_major and
  * .t().contiguous() at nanochat/fp8.py:110-118,169,181-182 (the backward GEMMs want the summed index contiguous in

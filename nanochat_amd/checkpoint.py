@@ -36,9 +36,13 @@ def load_checkpoint(checkpoint_dir, step, device):
     return model_data, meta_data
 
 
-def build_model(checkpoint_dir, step=None, device="cuda", fp8=True):
+def build_model(checkpoint_dir, step=None, device="cuda"):
     """GPT on `device` holding the checkpoint's tensors as saved, FP8 linears swapped in with the reference's filter
-    (scripts/base_train.py:178-185) unless fp8=False is asked for.  Returns (model, meta)."""
+    (scripts/base_train.py:178-185).  Returns (model, meta).
+
+    The reference evaluates a checkpoint with plain Linear modules (bf16 matmuls, checkpoint_manager.py:99-104); the path built
+    here is the quantized one only, so a loaded model always runs its block linears and lm_head as e4m3 Float8Linear -- the
+    numerics of the reference's --fp8 training forward, not of its bf16 evaluation."""
     if step is None:
         step = find_last_step(checkpoint_dir)
     device = torch.device(device)
@@ -67,6 +71,5 @@ def build_model(checkpoint_dir, step=None, device="cuda", fp8=True):
     # Float8Linear would do on every call.
     model.load_state_dict({k: v.to(device) for k, v in model_data.items()}, strict=True, assign=True)
     model.eval()
-    if fp8:
-        convert_to_float8_training(model, module_filter_fn=fp8_module_filter)
+    convert_to_float8_training(model, module_filter_fn=fp8_module_filter)
     return model, meta

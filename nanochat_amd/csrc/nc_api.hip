@@ -41,6 +41,13 @@ int nc_fp8_quantize_tensorwise_fused(const void* x, int x_dtype, int64_t n, int 
     return nc_launch_quantize_fused(x, x_dtype, n, fp8_format, out, scale_out, inv_scale_out, (uint32_t*)state, encoder, (hipStream_t)stream);
 }
 
+int nc_fp8_quantize_tensorwise_fused_bounded(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
+                                             float* inv_scale_out, void* state, int encoder, uint32_t spin_limit, nc_stream_t stream) {
+    NC_CHECK_ARG(encoder == 0 || encoder == 1, "fp8_quantize: encoder must be 0 (hardware) or 1 (software)");
+    return nc_launch_quantize_fused(x, x_dtype, n, fp8_format, out, scale_out, inv_scale_out, (uint32_t*)state, encoder, (hipStream_t)stream,
+                                    spin_limit);
+}
+
 int nc_fp8_encode_with_scale(const uint16_t* x, int64_t n, float scale, int fp8_format, uint8_t* out, int encoder, nc_stream_t stream) {
     NC_CHECK_ARG(encoder == 0 || encoder == 1, "fp8_encode: encoder must be 0 (hardware) or 1 (software)");
     return nc_launch_encode_with_scale(x, n, scale, fp8_format, out, encoder, (hipStream_t)stream);

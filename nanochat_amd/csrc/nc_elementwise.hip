@@ -44,11 +44,15 @@ __global__ __launch_bounds__(256) void embed_norm_smear_kernel(const int64_t* __
 
     for (int which = 0; which < (use_prev_token ? 2 : 1); which++) {
         int64_t tok = idx[(size_t)b * T + t - which];
-        if (tok < 0 || tok >= vocab_rows) tok = 0;       // host validates; never read out of bounds
+        // An id outside the table never reads out of bounds; its row becomes NaN, which the tensorwise scales carry into every
+        // logit of the call: the reference's nn.Embedding raises for such an id (gpt.py:470), a kernel cannot, and a silently
+        // substituted row would be worse.  (The host refuses such ids in prompts and forced tokens before they get here.)
+        const bool bad_id = tok < 0 || tok >= vocab_rows;
+        if (bad_id) tok = 0;
         const bf16_t* e = wte + (size_t)tok * E;
         float ss = 0.f;
         for (int c = threadIdx.x; c < E; c += 256) {
-            float v = bf16_to_f32(e[c]);
+            float v = bad_id ? __uint_as_float(0x7fc00000u) : bf16_to_f32(e[c]);
             rowbuf[which * E + c] = v;
             ss += v * v;
         }
@@ -90,7 +94,8 @@ __global__ __launch_bounds__(256) void embed_norm_smear_decode_kernel(const int6
     const int b = blockIdx.x, c0 = threadIdx.x * 8;
     const bool mine = c0 < E;
     int64_t tok = idx[b];
-    if (tok < 0 || tok >= vocab_rows) tok = 0;       // host validates; never read out of bounds
+    const bool bad_id = tok < 0 || tok >= vocab_rows;      // never read out of bounds: the row becomes NaN (see the kernel above)
+    if (bad_id) tok = 0;
     uint4 ev = make_uint4(0, 0, 0, 0), pv = make_uint4(0, 0, 0, 0);
     if (mine) {
         ev = *(const uint4*)(wte + (size_t)tok * E + c0);
@@ -105,6 +110,10 @@ __global__ __launch_bounds__(256) void embed_norm_smear_decode_kernel(const int6
     float v[8], ss = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; j++) v[2 * j] = bf16_lo(ew[j]), v[2 * j + 1] = bf16_hi(ew[j]);
+    if (bad_id) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = __uint_as_float(0x7fc00000u);
+    }
 #pragma unroll
     for (int j = 0; j < 8; j++) ss += v[j] * v[j];
     ss = block_sum<4>(ss, red);

@@ -179,15 +179,26 @@ int nc_launch_quantize(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* 
 // its share once and keeps it, the workgroups meet on the tensor's amax, and the payload is converted from registers.  HBM sees the
 // algorithmic 3 bytes per element and the three launches (clear, amax, convert) become one.
 //
-// The meeting needs every workgroup of the grid to be resident, which holds because the grid is sized to what the device can hold of
-// this kernel alone (hipOccupancyMaxActiveBlocksPerMultiprocessor x CUs): a workgroup that has to wait for a slot taken by some other
-// kernel gets it when that kernel ends, and nothing the other kernel does waits for this one.  The wait is bounded all the same: a
-// workgroup that gives up marks the state's error word and the scale comes out as NaN instead of the kernel hanging.
+// The meeting needs every workgroup of the grid to be resident, which holds because the grid is sized to half of what the device can
+// hold of this kernel alone (hipOccupancyMaxActiveBlocksPerMultiprocessor x CUs): a workgroup that has to wait for a slot taken by
+// some other kernel gets it when that kernel ends, and nothing the other kernel does waits for this one.  Two such grids on one GPU
+// (of this process or of another) still both fit; more of them at once can hold each other's slots.  The wait is therefore bounded
+// (`spin_limit` polls), and a workgroup whose wait runs out does not fail: it works the tensor's amax out by itself, reading the
+// whole tensor once more (slow -- a single workgroup streams at tens of GB/s -- and bit-identical, because the maximum does not
+// depend on who computes it), converts its share and leaves like every other.  Such workgroups are counted in word 257 of the
+// state, which the kernel never reads and never clears: a diagnostic for the host, not a condition.
 //
-// state: all zero before the first call, left all zero by every call (the last workgroup to leave clears it).  Slot k
-// (k = blockIdx.x % 8) lives on its own 128-byte line: word 0 the running maximum, word 1 the arrivals (one address would
-// serialize the grid's atomics at ~6 ns each).  Line 8: departures, the sticky error mark, slots reported.  Line 9: the flag
-// that the last reported slot raises and one lane per workgroup watches.  Line 10, word 0: scratch of the two-pass path.
+// Ordering.  Everything the workgroups exchange (maxima, arrival counts, the flag, departures) is read and written with device-scope
+// atomic operations, which are performed at the device's coherence point, not in an XCD's L2: there is no plain store to make
+// visible, hence no release / acquire fence (each of which would write back or invalidate an XCD's whole L2).  Program order
+// within the one lane that does them is kept by waiting for the value every read-modify-write returns before the next one is
+// issued: the maximum is acknowledged before the arrival is counted, so whoever sees all arrivals sees all maxima.
+//
+// state: all zero before the first call, left all zero by every call, whichever way its workgroups went (the last workgroup to
+// leave clears it; every workgroup leaves exactly once, after it has arrived).  Slot k (k = blockIdx.x % 8) lives on its own
+// 128-byte line: word 0 the running maximum, word 1 the arrivals (one address would serialize the grid's atomics at ~6 ns each).
+// Line 8: departures, the count of workgroups that ever took the slow way (sticky), slots reported.  Line 9: the flag that the
+// last reported slot raises and one lane per workgroup watches.  Line 10, word 0: scratch of the two-pass path.
 #define QF_SLOTS 8
 #define QF_STRIDE 32
 #define QF_DEPART (QF_SLOTS * QF_STRIDE)
@@ -200,7 +211,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
                                                              float* __restrict__ scale_out, float* __restrict__ inv_out,
                                                              uint32_t* __restrict__ state, uint32_t spin_limit) {
     __shared__ uint32_t red[4];
-    __shared__ uint32_t amax_sh;
+    __shared__ uint32_t amax_sh, slow_sh;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     // group g of this thread: 16 elements (32 bytes in, 16 bytes out) at group index (blockIdx.x * G + g) * 256 + tid
     uint4 ra[G], rb[G];
@@ -256,15 +267,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
         gave_up = __builtin_amdgcn_readfirstlane((int)gave_up) != 0;
         uint32_t am = lane < QF_SLOTS ? __hip_atomic_load(state + lane * QF_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
         am = wave_max_u32(am);
-        if (gave_up) {
-            am = 0x7fc00000u;                                // NaN: the scale and the payload come out as NaN
-            if (lane == 0) __hip_atomic_store(state + QF_ERROR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
         if (lane == 0) {
-            amax_sh = am;
-            // leave; the last one out puts the state back to zero for the next call (everyone has read what it needs by now)
+            amax_sh = am;                                    // (not looked at by a workgroup that gave up: the slots were incomplete)
+            slow_sh = gave_up ? 1u : 0u;
+            if (gave_up) __hip_atomic_fetch_add(state + QF_ERROR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // leave; the last one out puts the state back to zero for the next call (everyone has arrived and read what it needs by
+            // now: a workgroup leaves only after its own arrival, with the flag seen or its wait given up)
             const uint32_t gone = __hip_atomic_fetch_add(state + QF_DEPART, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (gone == gridDim.x - 1 && !gave_up) {
+            if (gone == gridDim.x - 1) {
                 for (int i = 0; i < QF_SLOTS; i++) {
                     __hip_atomic_store(state + i * QF_STRIDE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(state + i * QF_STRIDE + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -276,6 +286,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
         }
     }
     __syncthreads();
+    if (slow_sh) {
+        // the meeting did not complete within this workgroup's wait: the maximum over the whole tensor, by this workgroup alone
+        uint32_t mm = 0;
+        for (int64_t idx = tid; idx < n16; idx += 256) {
+            const uint4 a = ((const uint4*)x)[idx * 2], b = ((const uint4*)x)[idx * 2 + 1];
+            const uint32_t wd[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t lo = (wd[j] & 0x7fffu) << 16, hi = wd[j] & 0x7fff0000u;
+                mm = mm > lo ? mm : lo;
+                mm = mm > hi ? mm : hi;
+            }
+        }
+        mm = wave_max_u32(mm);
+        __syncthreads();                                     // red[] was read by wave 0 before the barrier above
+        if (lane == 0) red[w] = mm;
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t t = red[0];
+            for (int i = 1; i < 4; i++) t = t > red[i] ? t : red[i];
+            amax_sh = t;
+        }
+        __syncthreads();
+    }
     const float scale = scale_from_amax(__uint_as_float(amax_sh), fp8_max<FMT>());
     if (blockIdx.x == 0 && tid == 0) {
         if (scale_out) *scale_out = scale;
@@ -316,32 +350,36 @@ static int fused_capacity() {
 }
 
 template <int FMT, bool HW_CVT, int G>
-static bool try_fused(const bf16_t* x, int64_t n16, uint8_t* out, float* scale_out, float* inv_out, uint32_t* state, hipStream_t s) {
+static bool try_fused(const bf16_t* x, int64_t n16, uint8_t* out, float* scale_out, float* inv_out, uint32_t* state, uint32_t spin_limit,
+                      hipStream_t s) {
     const int64_t blocks = (n16 + 256 * (int64_t)G - 1) / (256 * (int64_t)G);
-    // half of the capacity: two such grids launched on two streams at the same time still both fit (callers that overlap more
-    // than that on one GPU could starve each other's meeting until the bounded wait gives up)
+    // half of the capacity: two such grids on one GPU at the same time still both fit (more than that can hold each other's slots
+    // until the bounded wait runs out and the workgroups take the slow way)
     if (blocks > (int64_t)fused_capacity<FMT, HW_CVT, G>() / 2) return false;
     hipLaunchKernelGGL((quantize_fused_kernel<FMT, HW_CVT, G>), dim3((unsigned)blocks), dim3(256), 0, s, x, n16, out, scale_out, inv_out, state,
-                       1u << 22);       // ~4 M polls of a few hundred ns each before a workgroup gives up
+                       spin_limit);
     return true;
 }
 
 template <int FMT, bool HW_CVT>
-static bool try_fused_any(const bf16_t* x, int64_t n16, uint8_t* out, float* scale_out, float* inv_out, uint32_t* state, hipStream_t s) {
+static bool try_fused_any(const bf16_t* x, int64_t n16, uint8_t* out, float* scale_out, float* inv_out, uint32_t* state, uint32_t lim,
+                          hipStream_t s) {
     // The largest share per thread that still leaves a workgroup for every other CU: few workgroups keep the meeting cheap (its atomics and
     // its pollers share a handful of memory lines), long shares keep many loads in flight per thread.
     const int64_t per_wg = 128;          // (half of the CUs at least)
-    if (n16 >= 8 * per_wg * 256 && try_fused<FMT, HW_CVT, 8>(x, n16, out, scale_out, inv_out, state, s)) return true;
-    if (n16 >= 4 * per_wg * 256 && try_fused<FMT, HW_CVT, 4>(x, n16, out, scale_out, inv_out, state, s)) return true;
-    if (n16 >= 2 * per_wg * 256 && try_fused<FMT, HW_CVT, 2>(x, n16, out, scale_out, inv_out, state, s)) return true;
-    return try_fused<FMT, HW_CVT, 1>(x, n16, out, scale_out, inv_out, state, s) || try_fused<FMT, HW_CVT, 2>(x, n16, out, scale_out, inv_out, state, s) ||
-           try_fused<FMT, HW_CVT, 4>(x, n16, out, scale_out, inv_out, state, s) || try_fused<FMT, HW_CVT, 8>(x, n16, out, scale_out, inv_out, state, s);
+    if (n16 >= 8 * per_wg * 256 && try_fused<FMT, HW_CVT, 8>(x, n16, out, scale_out, inv_out, state, lim, s)) return true;
+    if (n16 >= 4 * per_wg * 256 && try_fused<FMT, HW_CVT, 4>(x, n16, out, scale_out, inv_out, state, lim, s)) return true;
+    if (n16 >= 2 * per_wg * 256 && try_fused<FMT, HW_CVT, 2>(x, n16, out, scale_out, inv_out, state, lim, s)) return true;
+    return try_fused<FMT, HW_CVT, 1>(x, n16, out, scale_out, inv_out, state, lim, s) || try_fused<FMT, HW_CVT, 2>(x, n16, out, scale_out, inv_out, state, lim, s) ||
+           try_fused<FMT, HW_CVT, 4>(x, n16, out, scale_out, inv_out, state, lim, s) || try_fused<FMT, HW_CVT, 8>(x, n16, out, scale_out, inv_out, state, lim, s);
 }
 
 // state: NC_QUANTIZE_STATE_BYTES (1 KB + 16).  Tensors the one-launch kernel does not take (fp32 input, an element count that is
 // not a multiple of 16, more elements than fit on the chip) go through the two passes, with the state's last word as their scratch.
+// spin_limit: polls of the meeting's flag (a few hundred ns each) before a workgroup stops waiting and takes the slow way;
+// NC_QUANTIZE_DEFAULT_SPINS in ordinary use, a tiny value from the test that drives the slow way.
 int nc_launch_quantize_fused(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* out, float* scale_out, float* inv_out,
-                             uint32_t* state, int encoder, hipStream_t s) {
+                             uint32_t* state, int encoder, hipStream_t s, uint32_t spin_limit) {
     NC_CHECK_ARG(n >= 0, "fp8_quantize: negative element count");
     NC_CHECK_ARG(inv_out && state && (n == 0 || (x && out)), "fp8_quantize: null pointer");
     NC_CHECK_ARG(x_dtype == 0 || x_dtype == 1, "fp8_quantize: dtype must be 0 (bf16) or 1 (fp32)");
@@ -352,10 +390,10 @@ int nc_launch_quantize_fused(const void* x, int x_dtype, int64_t n, int fmt, uin
         NcProfScope prof(2, 3.0 * n, s);
         const bf16_t* xb = (const bf16_t*)x;
         bool done;
-        if (fmt == 0) done = encoder == 0 ? try_fused_any<0, true>(xb, n / 16, out, scale_out, inv_out, state, s)
-                                          : try_fused_any<0, false>(xb, n / 16, out, scale_out, inv_out, state, s);
-        else done = encoder == 0 ? try_fused_any<1, true>(xb, n / 16, out, scale_out, inv_out, state, s)
-                                 : try_fused_any<1, false>(xb, n / 16, out, scale_out, inv_out, state, s);
+        if (fmt == 0) done = encoder == 0 ? try_fused_any<0, true>(xb, n / 16, out, scale_out, inv_out, state, spin_limit, s)
+                                          : try_fused_any<0, false>(xb, n / 16, out, scale_out, inv_out, state, spin_limit, s);
+        else done = encoder == 0 ? try_fused_any<1, true>(xb, n / 16, out, scale_out, inv_out, state, spin_limit, s)
+                                 : try_fused_any<1, false>(xb, n / 16, out, scale_out, inv_out, state, spin_limit, s);
         if (done) {
             NC_CHECK_LAUNCH("fp8_quantize");
             return 0;

@@ -12,6 +12,7 @@ from dataclasses import dataclass
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import _lib, ops
 from .common import COMPUTE_DTYPE
@@ -35,8 +36,12 @@ def has_ve(layer_idx, n_layer):
 
 
 class Linear(nn.Linear):
-    """Bias-free linear whose weight is cast to the input dtype (gpt.py:45-50).  Only the tiny gates
-    stay in this class at inference; on the GPU they are evaluated inside the fused kernels."""
+    """Linear whose weight is cast to the input's dtype in forward (gpt.py:45-50): master weights stay fp32, the product runs in
+    the activation dtype.  Only the tiny gates (ve_gate [n_kv_head, 12], smear_gate [1, 24]) stay in this class once the FP8
+    filter has run, and GPT.forward evaluates those inside its fused kernels; this forward serves a direct call on the module."""
+
+    def forward(self, x):
+        return F.linear(x, self.weight.to(dtype=x.dtype))
 
 
 class CausalSelfAttention(nn.Module):
@@ -209,13 +214,22 @@ class GPT(nn.Module):
         return super()._apply(fn, recurse)
 
     def _current_plan_key(self):
-        """What the plan was built from, cheaply enough for every decode step: the storage addresses and in-place version counters
-        of the parameters seen when the plan was built (walking the module tree for them costs most of a millisecond at d26, a
-        kept list some tens of microseconds).  A parameter object replaced by another one is caught by invalidate_plan(), not here."""
-        params = self._plan_params
-        if params is None:
-            params = self._plan_params = list(self.parameters())
-        return tuple([(p._version, p.data_ptr()) for p in params])
+        """What the plan was built from, cheaply enough for every decode step: per parameter, which object holds it, where its
+        storage is and its in-place version counter.  The (module, name) slots are listed once per plan (walking the module tree for
+        them costs most of a millisecond at d26; looking the slots up again, some tens of microseconds), so a parameter object that
+        is replaced -- `mod.weight = nn.Parameter(...)`, a swapped-in tensor -- changes the key like an in-place update does.  Only
+        a replaced *module* needs invalidate_plan() (convert_to_float8_training, load_state_dict and .to() call it themselves)."""
+        slots = self._plan_params
+        if slots is None:
+            slots = self._plan_params = [(mod, name, p) for mod in self.modules() for name, p in mod._parameters.items() if p is not None]
+        key = []
+        for mod, name, kept in slots:
+            p = mod._parameters[name]
+            if p is not kept:                    # (the kept reference also keeps the old object's id from being handed out again)
+                self._plan_params = None
+                return None                      # equal to no stored key: the plan is rebuilt and the slots are listed afresh
+            key.append((p._version, p.data_ptr()))
+        return tuple(key)
 
     def _build_plan(self):
         """Quantize every FP8 linear once, stack q|k|v, and fill the C descriptors."""
@@ -285,7 +299,7 @@ class GPT(nn.Module):
 
     def _ensure_plan(self):
         key = self._current_plan_key()
-        if self._plan is None or key != self._plan_key:
+        if self._plan is None or key is None or key != self._plan_key:
             self._build_plan()
             self._plan_key = self._current_plan_key()
         return self._plan[0]

@@ -43,10 +43,22 @@ def _quantize_state(device):
 _FP8_FORMATS = {torch.float8_e4m3fn: 0, torch.float8_e5m2: 1}
 
 
-def fp8_quantize(x, encoder=0, fp8_dtype=torch.float8_e4m3fn):
+QUANTIZE_SLOW_WORD = 257      # uint32 index in the quantizer's state block: workgroups that ever took the slow way (sticky)
+
+
+def quantize_slow_count(device=None):
+    """How many workgroups of the one-launch quantizer ever gave up waiting for their peers on this device and stream, and worked
+    the amax out alone (correct results, slowly): non-zero means more such grids overlapped on the GPU than it holds at once.
+    Reads the device (a synchronisation); for diagnostics and tests."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    return int(_quantize_state(device).view(torch.int32)[QUANTIZE_SLOW_WORD].item())
+
+
+def fp8_quantize(x, encoder=0, fp8_dtype=torch.float8_e4m3fn, spin_limit=None):
     """Tensorwise fp8 quantization of a bf16/fp32 tensor (nanochat/fp8.py:81-107): e4m3fn, or e5m2 for gradients.
 
-    Returns (payload of fp8_dtype with x's shape, inv_scale fp32 0-dim, scale fp32 0-dim)."""
+    Returns (payload of fp8_dtype with x's shape, inv_scale fp32 0-dim, scale fp32 0-dim).  spin_limit (tests): the bound of the
+    one-launch kernel's wait for its peers, in polls; None = the library's default."""
     _need_cuda(x)
     if x.dtype not in (torch.bfloat16, torch.float32):
         raise ValueError(f"fp8_quantize: dtype {x.dtype} not supported (bf16 or fp32)")
@@ -56,9 +68,12 @@ def fp8_quantize(x, encoder=0, fp8_dtype=torch.float8_e4m3fn):
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     scales = torch.empty(2, dtype=torch.float32, device=x.device)
     state = _quantize_state(x.device)
-    rc = _lib.lib().nc_fp8_quantize_tensorwise_fused(_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _FP8_FORMATS[fp8_dtype],
-                                                     _ptr(out), C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4),
-                                                     _ptr(state), encoder, _stream())
+    args = (_ptr(x), 0 if x.dtype == torch.bfloat16 else 1, x.numel(), _FP8_FORMATS[fp8_dtype], _ptr(out), C.c_void_p(scales.data_ptr()),
+            C.c_void_p(scales.data_ptr() + 4), _ptr(state), encoder)
+    if spin_limit is None:
+        rc = _lib.lib().nc_fp8_quantize_tensorwise_fused(*args, _stream())
+    else:
+        rc = _lib.lib().nc_fp8_quantize_tensorwise_fused_bounded(*args, int(spin_limit), _stream())
     _lib.check(rc)
     return out.view(fp8_dtype), scales[1], scales[0]
 
@@ -298,10 +313,19 @@ def decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=-1, seqlens
     return out
 
 
+_ATTN_WS = {}
+
+
 def _attention_workspace(B, T, H, Tmax, device):
-    lib = _lib.lib()
-    ws_bytes = lib.nc_attention_workspace_bytes(B, T, H, Tmax)
-    return torch.empty(ws_bytes, dtype=torch.uint8, device=device), ws_bytes      # the call clears its own counters
+    """Split counters and partial results of the stand-alone attention entries, kept per device and stream and grown on demand
+    (calls on one stream run one after the other, and every call clears its own counters)."""
+    ws_bytes = _lib.lib().nc_attention_workspace_bytes(B, T, H, Tmax)
+    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    ws = _ATTN_WS.get(key)
+    if ws is None or ws.numel() < ws_bytes:
+        ws = torch.empty(max(ws_bytes, 1 << 20), dtype=torch.uint8, device=device)
+        _ATTN_WS[key] = ws
+    return ws, ws_bytes
 
 
 def decode_attention_append(q, k_new, v_new, k_cache, v_cache, cache_seqlens, window_left=-1, splits=0):

@@ -15,7 +15,7 @@ def config_for_depth(depth, sequence_len=2048, vocab_size=32768, window_pattern=
                      n_kv_head=n_kv_head or n_head, n_embd=model_dim, window_pattern=window_pattern)
 
 
-def random_init_model(cfg, device, seed=0, fp8=True):
+def random_init_model(cfg, device, seed=0):
     """Random weights drawn on the device with the distributions of the reference's init_weights (gpt.py:204-268), but
     with non-zero output projections, gates and lambdas so that every kernel does real work.  bf16, FP8 linears."""
     with torch.device("meta"):
@@ -49,8 +49,7 @@ def random_init_model(cfg, device, seed=0, fp8=True):
                 raise RuntimeError(f"unhandled parameter {name}")
         model.to(torch.bfloat16)
     model.eval()
-    if fp8:
-        convert_to_float8_training(model, module_filter_fn=fp8_module_filter)
+    convert_to_float8_training(model, module_filter_fn=fp8_module_filter)
     return model
 
 

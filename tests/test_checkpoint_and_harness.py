@@ -59,7 +59,7 @@ def test_loader_patches_old_checkpoints_and_rejects_mismatches(tmp_path):
     write_checkpoint(d, 5, drop=("resid_lambdas", "x0_lambdas"))
     with open(os.path.join(d, "meta_000005.json"), "w") as f:
         json.dump({"step": 5, "model_config": old_cfg}, f)
-    model, _ = build_model(d, 5, device="cpu", fp8=False)
+    model, _ = build_model(d, 5, device="cpu")
     assert model.config.window_pattern == "L"                      # checkpoint_manager.py:22-27
     assert torch.equal(model.resid_lambdas.float(), torch.ones(3)) and torch.equal(model.x0_lambdas.float(), torch.zeros(3))
     bad = str(tmp_path / "bad")

@@ -3,9 +3,8 @@ against the CPU oracle on the same seeded weights and inputs.
 
 Bars.
   * Repository init (the reference's own init_weights: zero-initialised projections, lm_head std 0.001 -- the weights the
-    stated tolerance is quoted on): logits within 1e-2 abs of the oracle, greedy ids identical to the
-    oracle's wherever the oracle's own top-2 margin exceeds the tolerance (bf16 logits tie often and a
-    tie is decided by summation order).
+    stated tolerance is quoted on): logits within 1e-2 abs of the oracle, the 64 greedy ids identical to the
+    oracle's (asserted strictly on the fixed seed).
   * "Trained-like" init (non-zero projections, O(1) logits, so attention / MLP / smear / KV cache all
     matter): dynamic tensorwise FP8 re-quantizes every activation, which amplifies any last-bit
     difference to the fp8 noise level within a few layers.  The oracle itself moves by rel-L2 ~4e-2
@@ -86,6 +85,13 @@ def oracle_floor(rt, run):
     return rel_l2(b, a), (a - b).abs().max().item(), a, b
 
 
+def bar(what, value, recorded, margin):
+    """A bar written as the value observed when the test was written plus a stated margin; what this run observes is printed, so a
+    drift towards the bar shows in the log before it fails."""
+    print(f"[bar] {what}: observed {value:.5g} (recorded {recorded:.5g} + margin {margin:.5g} = bar {recorded + margin:.5g})")
+    assert value <= recorded + margin, f"{what}: {value} exceeds {recorded} + {margin}"
+
+
 def assert_within_floor(got, want_sdpa, want_def, floor_rel, floor_max, what):
     r1, r2 = rel_l2(got, want_sdpa), rel_l2(got, want_def)
     m1, m2 = (got - want_sdpa).abs().max().item(), (got - want_def).abs().max().item()
@@ -93,20 +99,6 @@ def assert_within_floor(got, want_sdpa, want_def, floor_rel, floor_max, what):
           f"oracle-vs-oracle floor rel_l2 {floor_rel:.4f} max {floor_max:.4f}")
     assert min(r1, r2) <= 1.5 * floor_rel + 1e-3, what
     assert min(m1, m2) <= 1.5 * floor_max + LOGIT_TOL, what
-
-
-def margin_aware_compare(got_ids, want_ids, want_logits):
-    """ids must agree wherever the oracle's top-2 gap is above the logit tolerance."""
-    strict = 0
-    for t, (g, w) in enumerate(zip(got_ids, want_ids)):
-        if g == w:
-            continue
-        strict += 1
-        top2 = torch.topk(want_logits[t], 2).values
-        gap = (top2[0] - top2[1]).item()
-        assert gap <= 2 * LOGIT_TOL, f"token {t}: {g} != {w} although the oracle margin is {gap}"
-        break          # after a legitimate tie-break divergence the sequences are no longer comparable
-    return strict
 
 
 def test_repo_init_logits_and_greedy_ids(d4_repo_pair):
@@ -129,10 +121,10 @@ def test_repo_init_logits_and_greedy_ids(d4_repo_pair):
     same = sum(int(a == b) for a, b in zip(got_ids, want_ids))
     print(f"repo init: max |dlogit| over 64 steps = {worst:.6f}; greedy ids equal on {same}/64 steps")
     assert worst <= LOGIT_TOL
-    for t, (a, b) in enumerate(zip(got_ids, want_ids)):
-        if a != b:
-            top2 = torch.topk(want_logits[t][0], 2).values
-            assert (top2[0] - top2[1]).item() <= 2 * worst + 1e-6, f"step {t}: {a} != {b} with oracle margin {top2[0] - top2[1]}"
+    # strict: on this seed all 64 ids are the oracle's; the oracle's own top-2 margin at a differing step only explains a failure
+    diverged = [(t, a, b, (lambda v: (v[0] - v[1]).item())(torch.topk(want_logits[t][0], 2).values))
+                for t, (a, b) in enumerate(zip(got_ids, want_ids)) if a != b]
+    assert not diverged, f"greedy ids differ from the oracle's at (step, got, want, oracle top-2 margin): {diverged}"
 
 
 def test_prefill_logits_match_oracle(d4_pair):
@@ -162,9 +154,8 @@ def test_prefill_logits_match_oracle(d4_pair):
 
 
 def test_greedy_decode_64_tokens_through_engine(d4_repo_pair):
-    """Engine.generate on the GPU, greedy, 64 tokens, repository init: ids equal to the oracle's; a difference is accepted only
-    where the oracle's own top-2 margin is within twice the stated logit tolerance (bf16 logits tie often at this init).
-    The trained-like counterpart, with a bound derived from the oracle's own sensitivity, is in test_gpu_variants.py."""
+    """Engine.generate on the GPU, greedy, 64 tokens, repository init: all 64 ids equal to the oracle's (strictly; the oracle's own
+    top-2 margin at a differing step is only printed with the failure).  The trained-like counterpart, with a bound derived from the oracle's own sensitivity, is in test_gpu_variants.py."""
     from nanochat_amd.engine import Engine
     from test_engine_host import ByteTokenizer
 
@@ -188,12 +179,12 @@ def test_greedy_decode_64_tokens_through_engine(d4_repo_pair):
             break
     first_div = next((i for i, (a, b) in enumerate(zip(got_ids, want_ids)) if a != b), len(got_ids))
     print(f"repo: greedy ids identical for the first {first_div} of {len(got_ids)} tokens")
+    gap = None
     if first_div < min(len(got_ids), len(want_ids)):
         top2 = torch.topk(want_logits[first_div][0], 2).values
-        gap = (top2[0] - top2[1]).item()
-        assert gap <= 2 * LOGIT_TOL, f"token {first_div} differs although the oracle margin is {gap}"
-    else:
-        assert got_ids == want_ids[:len(got_ids)]
+        gap = (top2[0] - top2[1]).item()          # the diagnostic: how close the oracle's own decision was at the first differing step
+    # strict: all 64 ids identical on this seed
+    assert len(got_ids) == 64 and got_ids == want_ids, f"token {first_div} differs; the oracle's top-2 margin there is {gap}"
 
 
 def test_decode_logits_stepwise_teacher_forced(d4_pair):
@@ -700,10 +691,15 @@ def test_weight_changes_are_noticed_by_the_next_forward():
         w.mul_(1.0 / 1.5)
     model.load_state_dict(state, assign=True)                            # new parameter objects
     assert torch.equal(logits(), changed)
-    model.lm_head.weight = torch.nn.Parameter(model.lm_head.weight.detach() * 2.0)      # by hand: needs the explicit call
-    model.invalidate_plan()
+    model.lm_head.weight = torch.nn.Parameter(model.lm_head.weight.detach() * 2.0)      # a new parameter object, assigned by hand
     doubled = logits()
-    assert not torch.equal(doubled, changed)
+    assert not torch.equal(doubled, changed), "a replaced parameter object went unnoticed: the forward used stale e4m3 weights"
+    blk = model.transformer.h[0].mlp.c_fc
+    blk.weight = torch.nn.Parameter(blk.weight.detach() * 0.5)
+    halved = logits()
+    assert not torch.equal(halved, doubled)
+    blk.weight = torch.nn.Parameter(blk.weight.detach() * 2.0)
+    assert torch.equal(logits(), doubled)
     model.value_embeds.to(torch.float32)                                 # a child cast: same parameter objects, new storage
     model.value_embeds.to(torch.bfloat16)
     assert torch.equal(logits(), doubled)

@@ -130,6 +130,82 @@ def test_quantize_one_launch_form_against_the_two_passes_and_its_state(ops):
     assert torch.isnan(scale).item() and torch.isnan(inv).item()
 
 
+def test_quantize_one_launch_form_when_the_wait_for_the_peers_runs_out(ops):
+    """The bound of the one-launch quantizer's grid-wide wait, set to zero polls from the host: nearly every workgroup stops
+    waiting at once and works the amax out by itself from the whole tensor.  Every kernel exits normally; payload and scales
+    are those of the two-pass entry bit for bit (NaN included), the workgroups that went the slow way are counted in the state's
+    diagnostic word and in nothing else, the state is otherwise left all zero, and the next call with the default bound on the
+    same state is bit-correct and counts nobody."""
+    say("quantize: one launch, the wait given up from the host")
+    import ctypes as C
+    from nanochat_amd import _lib
+    lib = _lib.lib()
+    nbytes = lib.nc_fp8_quantize_state_bytes()
+    raw = torch.zeros(nbytes + 128, dtype=torch.uint8, device=DEV)
+    off = (-raw.data_ptr()) % 128
+    state = raw[off:off + nbytes]
+    words = state.view(torch.int32)
+    SLOW = ops.QUANTIZE_SLOW_WORD
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator(device=DEV).manual_seed(5)
+
+    def two_pass(x, fmt):
+        out = torch.empty(x.shape, dtype=torch.uint8, device=DEV)
+        sc = torch.zeros(2, dtype=torch.float32, device=DEV)
+        ws = torch.zeros(1, dtype=torch.int32, device=DEV)
+        _lib.check(lib.nc_fp8_quantize_tensorwise_as(x.data_ptr(), 0, x.numel(), fmt, out.data_ptr(), sc.data_ptr(), sc.data_ptr() + 4,
+                                                     ws.data_ptr(), 0, stream))
+        return out, sc
+
+    def one_launch(x, fmt, limit):
+        out = torch.empty(x.shape, dtype=torch.uint8, device=DEV)
+        sc = torch.zeros(2, dtype=torch.float32, device=DEV)
+        if limit is None:
+            rc = lib.nc_fp8_quantize_tensorwise_fused(x.data_ptr(), 0, x.numel(), fmt, out.data_ptr(), sc.data_ptr(), sc.data_ptr() + 4,
+                                                      state.data_ptr(), 0, stream)
+        else:
+            rc = lib.nc_fp8_quantize_tensorwise_fused_bounded(x.data_ptr(), 0, x.numel(), fmt, out.data_ptr(), sc.data_ptr(),
+                                                              sc.data_ptr() + 4, state.data_ptr(), 0, limit, stream)
+        _lib.check(rc)
+        return out, sc
+
+    counted = 0
+    for shape, fmt, with_nan in (((2048, 1664), 0, False), ((512, 6656), 1, False), ((64, 6656), 0, False), ((1024, 512), 0, True)):
+        x = torch.randn(shape, device=DEV, generator=g)
+        x = torch.where(torch.rand(shape, device=DEV, generator=g) < 0.001, x * 20, x).bfloat16()
+        if with_nan:
+            x[777, 3] = float("nan")
+        want_out, want_sc = two_pass(x, fmt)
+        got_out, got_sc = one_launch(x, fmt, 0)
+        torch.cuda.synchronize()
+        assert torch.equal(got_sc.view(torch.int32), want_sc.view(torch.int32)), (shape, got_sc, want_sc)
+        if not with_nan:                     # (with a NaN scale every product is NaN whatever the payload bytes are)
+            assert torch.equal(got_out, want_out), shape
+        w = words.cpu()
+        slow_now = int(w[SLOW]) - counted
+        counted = int(w[SLOW])
+        print(f"{shape}: {slow_now} workgroups went the slow way")
+        assert slow_now > 0, "a bound of zero polls was meant to send workgroups the slow way"
+        w[SLOW] = 0
+        assert not w[:320].any(), f"{shape}: the state was not left zero: {w[:320].nonzero().flatten().tolist()}"
+        # the ordinary entry on the same state right behind it
+        got_out, got_sc = one_launch(x, fmt, None)
+        torch.cuda.synchronize()
+        assert torch.equal(got_sc.view(torch.int32), want_sc.view(torch.int32))
+        if not with_nan:
+            assert torch.equal(got_out, want_out), shape
+        assert int(words[SLOW].item()) == counted, "the default bound sent a workgroup the slow way on an idle GPU"
+    # the wrapper the modules use reports the same word for its own state
+    before = ops.quantize_slow_count()
+    x = torch.randn(4096, 1664, device=DEV, generator=g).bfloat16()
+    p0, inv0, s0 = ops.fp8_quantize(x)
+    p1, inv1, s1 = ops.fp8_quantize(x, spin_limit=0)
+    assert torch.equal(p0.view(torch.uint8), p1.view(torch.uint8)) and torch.equal(inv0, inv1) and torch.equal(s0, s1)
+    assert ops.quantize_slow_count() > before
+    p2, inv2, s2 = ops.fp8_quantize(x)
+    assert torch.equal(p0.view(torch.uint8), p2.view(torch.uint8)) and torch.equal(inv0, inv2)
+
+
 def test_quantize_zero_tensor_and_invariants(ops):
     say("quantize zeros / sign symmetry")
     p, inv, s = ops.fp8_quantize(torch.zeros(4096, dtype=torch.bfloat16, device=DEV))

@@ -39,11 +39,15 @@ def both_entries(B, T, H, Hkv, Tmax, window, splits, seed):
     _lib.check(lib.nc_decode_attention(ptr(q), ptr(kc), ptr(vc), ptr(seq), window, ptr(want), B, T, H, Hkv, Tmax, 0, ptr(ws), ws_bytes,
                                        ptr(amax_a), splits, stream))
     # everything the entry point needs exists by now: from here to the comparison nothing may be allocated
+    torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info()[0]           # what the driver reports: sees a hipMalloc that torch's allocator would not
     _lib.check(lib.nc_decode_attention_static(ptr(q), ptr(kc), ptr(vc), ptr(seq), window, ptr(got), B, T, H, Hkv, Tmax, 0, ptr(amax_b),
                                               splits, stream))
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
     torch.cuda.synchronize()
+    # the scratch is 8.65 MB: had the call (or the runtime on its behalf) allocated it, the device's free memory would show it
+    assert free_before - torch.cuda.mem_get_info()[0] < (1 << 20), (free_before, torch.cuda.mem_get_info()[0])
     assert torch.isfinite(want.float()).all()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (got.float() - want.float()).abs().max().item()
     assert amax_a.item() == amax_b.item() and amax_a.item() != 0
@@ -57,6 +61,14 @@ def test_static_scratch_entry_matches_the_workspace_entry_twice_in_a_row():
     heads = C.c_int(0)
     _lib.check(lib.nc_decode_attention_plan(6, 1, 13, -1, 700, 0, C.byref(splits), C.byref(heads)))
     assert splits.value > 1, "the first call was meant to split its keys over workgroups (the case that uses the scratch)"
+    # one call ahead of the measured ones: the first use of the library's device code (its module, with the scratch array in it, is
+    # loaded then) is not what the memory checks below are about
+    warm = torch.zeros(1, 1, 2, 128, dtype=torch.bfloat16, device=DEV)
+    wkv = torch.zeros(1, 8, 2, 128, dtype=torch.bfloat16, device=DEV)
+    _lib.check(lib.nc_decode_attention_static(ptr(warm), ptr(wkv), ptr(wkv), ptr(torch.zeros(1, dtype=torch.int32, device=DEV)), -1,
+                                              ptr(torch.empty_like(warm)), 1, 1, 2, 2, 8, 0, None, 0,
+                                              C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
     both_entries(6, 1, 13, 13, 700, -1, 0, seed=1)                # chosen split count (> 1): counters and partials in use
     both_entries(2, 1, 4, 2, 300, 64, 4, seed=2)                  # smaller, right behind it, on what the first call left
     both_entries(3, 3, 8, 2, 200, -1, 16, seed=3)                 # several queries per row, the maximum split count
