@@ -2,19 +2,18 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (the headline decode configuration): nanochat d26 (n_embd 1664, 13 heads, head_dim 128, 26 layers,
-vocab 32768, window pattern SSSL), bf16 weights with FP8 linears, random init seed 2; one prompt of
-random token ids is prefilled at batch 1, the KV cache is replicated to 64 rows, and greedy decoding
-runs through Engine.generate until the context reaches 2048 tokens.  A "step" is one iteration of that
-loop: sample for all 64 rows + one GPT.forward(ids[64,1], kv_cache).  The run is: W warm-up steps, P steps
-with a HIP event pair around every kernel launch (the roofline figures), then the K timed steps, the last
-of which brings the context to 2048; the prompt is 2048 - (W + P + K) tokens long: 1792 for the default
-8 + 16 + 232, i.e. 256 new tokens.
+Workload (the headline decode configuration, whatever K and W are): nanochat d26 (n_embd 1664, 13 heads, head_dim 128,
+26 layers, vocab 32768, window pattern SSSL), bf16 weights with FP8 linears, random init seed 2; one prompt of 1792 random
+token ids is prefilled at batch 1, the KV cache is replicated to 64 rows, and 256 greedy tokens are decoded through
+Engine.generate, which brings the context to 2048.  A "step" is one iteration of that loop: sample for all 64 rows + one
+GPT.forward(ids[64,1], kv_cache).  Of the 256 steps the first W are warm-up, the LAST K are the timed ones (they end at
+context 2048), the P before them carry a HIP event pair around every kernel launch (the roofline figures), and whatever lies
+between warm-up and those runs untimed; the defaults 8 + 16 + 232 leave nothing in between.
 
-One JSON line is printed with tokens/s, the roofline of the dominant kernel (decode attention, HBM
-bound), the rate of every decode linear against the HBM peak, FP8 GEMM rates at the isolated Float8Linear
-shapes, and a CPU baseline (the CPU oracle, a port of the reference's CPU behaviour, timed on this box's
-host cores on a bounded sample of the decode step and of the isolated GEMM shapes).
+One JSON line is printed with tokens/s, the roofline of the dominant kernel (decode attention, HBM bound), the rate of every
+decode linear against the HBM peak, the same run with every layer reading the whole context (window pattern L), FP8 GEMM rates
+at the isolated Float8Linear shapes, and a CPU baseline (the CPU oracle, a port of the reference's CPU behaviour, timed on this
+box's host cores on bounded samples of the decode configurations and of the isolated GEMM shapes).
 """
 import argparse
 import ctypes as C
@@ -33,6 +32,8 @@ FP8_PEAK = 5.0e15
 D26 = dict(sequence_len=2048, vocab_size=32768, n_layer=26, n_head=13, n_kv_head=13, n_embd=1664, window_pattern="SSSL")
 BATCH = 64
 CONTEXT = 2048
+PROMPT_TOKENS = 1792
+NEW_TOKENS = CONTEXT - PROMPT_TOKENS      # 256
 
 
 class RangeTokenizer:
@@ -105,17 +106,26 @@ def gemm_rates(device, library_gemm=False):
         # 60 untimed launches first: enough back-to-back work for the clocks to settle
         fwd_us = timed(lambda: ops.fp8_gemm(a8, w8, ia, iw, out=res), warm=60, n=100)
         flops = 2.0 * M * N * K
-        # quantize (amax + convert) of the activation, 3 bytes per element algorithmic
+        # quantize (amax + convert) of the activation, 3 bytes per element algorithmic, over a ring of distinct tensors larger
+        # than the 256 MB memory-side cache: every pass reads its tensor from HBM, as a Float8Linear in a model does
+        ring = [a] + [a.clone() for _ in range((320 << 20) // (a.numel() * 2) + 1)]
+        for t in ring:
+            ops.fp8_quantize(t)
+        torch.cuda.synchronize()
         lib.nc_profile_enable(1)
-        for _ in range(20):
-            ops.fp8_quantize(a)
+        for i in range(max(20, 2 * len(ring))):
+            ops.fp8_quantize(ring[i % len(ring)])
         torch.cuda.synchronize()
         qms, qbytes, qn = read_profile(lib, 2)
         lib.nc_profile_enable(0)
+        quantize_ring_mb = len(ring) * a.numel() * 2 >> 20
+        del ring
         tf = flops / (fwd_us * 1e-6) / 1e12
         out[f"K{K}_N{N}"] = {"us": round(fwd_us, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
                              "quantize_us": round(qms / qn * 1e3, 2),
-                             "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1)}
+                             "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1),
+                             "quantize_frac_hbm_peak": round(qbytes / (qms * 1e-3) / HBM_PEAK, 4),
+                             "quantize_distinct_input_mb": quantize_ring_mb}
         # the two backward GEMMs of the same layer (nanochat/fp8.py:156-192): e5m2 gradient x e4m3 saved operands
         go = (torch.randn(M, N, device=device, generator=g) * 1e-3).bfloat16()
 
@@ -178,63 +188,97 @@ def cpu_gemm_baseline(cores, budget_s=6.0):
     return out
 
 
-def cpu_baseline(budget_s=25.0):
-    """One decode step of the CPU oracle at the same shape (d26, 64 rows, context 1792), bf16 with
-    fp8-emulated linears, weights re-quantized on every call as the reference does (fp8.py:136)."""
+def cpu_decode_leg(cfg_kwargs, seed, batch, ctx, max_steps, budget_s, cores):
+    """Decode steps of the CPU oracle at one configuration: bf16 with fp8-emulated linears, weights re-quantized on every call as
+    the reference does (fp8.py:136), on a cache filled with random keys and values (no CPU prefill is paid for)."""
     from oracle import decode_ref, gpt_ref
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    cfg = gpt_ref.GPTConfig(**D26)
+    cfg = gpt_ref.GPTConfig(**cfg_kwargs)
     t0 = time.time()
-    g = torch.Generator().manual_seed(2)
-    E, L, V = cfg.n_embd, cfg.n_layer, cfg.vocab_size
+    g = torch.Generator().manual_seed(seed)
+    E, L, V, H, Hkv = cfg.n_embd, cfg.n_layer, cfg.vocab_size, cfg.n_head, cfg.n_kv_head
     s = 3 ** 0.5 * E ** -0.5
     p = {}
 
     # one random matrix per shape, cloned per layer: distinct memory (no cache reuse across layers) without
-    # paying the host RNG for 1.9e9 elements; timing does not depend on the values
+    # paying the host RNG for every element; timing does not depend on the values
     def u(*shape, a):
         return (torch.rand(*shape, generator=g) * 2 * a - a).bfloat16()
-    w_ee, w_fc, w_pr, w_ve = u(E, E, a=s), u(4 * E, E, a=0.4 * s), u(E, 4 * E, a=0.5 * s), u(V, E, a=s)
+    w_q, w_kv, w_o = u(H * 128, E, a=s), u(Hkv * 128, E, a=s), u(E, H * 128, a=s)
+    w_fc, w_pr, w_ve = u(4 * E, E, a=0.4 * s), u(E, 4 * E, a=0.5 * s), u(V, Hkv * 128, a=s)
     p["transformer.wte.weight"] = torch.randn(V, E, generator=g).bfloat16()
     p["lm_head.weight"] = (torch.randn(V, E, generator=g) * 0.03).bfloat16()
     for i in range(L):
         pre = f"transformer.h.{i}."
-        for nm in ("attn.c_q", "attn.c_k", "attn.c_v", "attn.c_proj"):
-            p[pre + nm + ".weight"] = w_ee.clone()
+        p[pre + "attn.c_q.weight"] = w_q.clone()
+        p[pre + "attn.c_k.weight"] = w_kv.clone()
+        p[pre + "attn.c_v.weight"] = w_kv.clone()
+        p[pre + "attn.c_proj.weight"] = w_o.clone()
         p[pre + "mlp.c_fc.weight"] = w_fc.clone()
         p[pre + "mlp.c_proj.weight"] = w_pr.clone()
         if gpt_ref.has_ve(i, L):
             p[f"value_embeds.{i}.weight"] = w_ve.clone()
-            p[pre + "attn.ve_gate.weight"] = torch.rand(cfg.n_kv_head, 12, generator=g) - 0.5
+            p[pre + "attn.ve_gate.weight"] = torch.rand(Hkv, 12, generator=g) - 0.5
     p["resid_lambdas"] = torch.linspace(1.15, 1.05, L)
     p["x0_lambdas"] = torch.linspace(0.20, 0.05, L)
     p["smear_lambda"] = torch.full((1,), 0.35)
     p["backout_lambda"] = torch.full((1,), 0.2)
     p["smear_gate.weight"] = torch.rand(1, 24, generator=g) - 0.5
     rt = gpt_ref.Runtime(cfg, p, compute_dtype=torch.bfloat16, fp8=True, cache_weights=False)
-    ctx = 1792
-    cache = decode_ref.new_cache(cfg, BATCH, ctx + 8, torch.bfloat16)
-    # a filled cache without paying for a CPU prefill: random keys/values of the right magnitude
-    kblk = (torch.randn(1, 1, ctx, cfg.n_kv_head, 128, generator=g) * 1.2).bfloat16()
-    vblk = (torch.randn(1, 1, ctx, cfg.n_kv_head, 128, generator=g) * 0.5).bfloat16()
+    cache = decode_ref.new_cache(cfg, batch, ctx + max_steps, torch.bfloat16)
+    kblk = (torch.randn(1, 1, ctx, Hkv, 128, generator=g) * 1.2).bfloat16()
+    vblk = (torch.randn(1, 1, ctx, Hkv, 128, generator=g) * 0.5).bfloat16()
     cache.k_cache[:, :, :ctx] = kblk
     cache.v_cache[:, :, :ctx] = vblk
     cache.cache_seqlens.fill_(ctx)
-    cache.prev_embedding = torch.randn(BATCH, 1, E, generator=g).bfloat16()
+    cache.prev_embedding = torch.randn(batch, 1, E, generator=g).bfloat16()
     setup_s = time.time() - t0
-    ids = torch.randint(0, V, (BATCH, 1), generator=g)
+    ids = torch.randint(0, V, (batch, 1), generator=g)
     steps, spent = 0, 0.0
-    while steps < 1 or (spent < budget_s and steps < 4):
+    while steps < 1 or (spent < budget_s and steps < max_steps):
         t1 = time.time()
         logits = gpt_ref.forward(rt, ids, cache)
         ids = logits[:, -1].argmax(-1, keepdim=True)
         spent += time.time() - t1
         steps += 1
-    return {"value": round(BATCH * steps / spent, 3), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{steps} decode step(s) of the CPU oracle at d26, 64 rows, context {ctx} (random-filled cache), bf16 + "
-                      f"fp8-emulated linears with per-call weight quantization as in the reference; setup {setup_s:.0f}s not timed",
-            "s_per_step": round(spent / steps, 3),
+    return {"tokens_per_s": round(batch * steps / spent, 3), "s_per_step": round(spent / steps, 4), "steps_timed": steps,
+            "batch": batch, "context": ctx, "setup_s_not_timed": round(setup_s, 1)}
+
+
+def cpu_config1_leg(cores):
+    """BASELINE configs[0] in full, the way scripts/infer_bench.py:73-79,207-216 times a run: the d4 model in fp32 on the CPU, the
+    repository's init (seed 0), batch 1, a 32-token prompt, 64 greedy tokens; tokens/s over prefill + decode."""
+    from oracle import decode_ref, gpt_ref
+    torch.set_num_threads(cores)
+    cfg = gpt_ref.GPTConfig(sequence_len=2048, vocab_size=32768, n_layer=4, n_head=2, n_kv_head=2, n_embd=256)
+    params = gpt_ref.init_params(cfg, seed=0, compute_dtype=torch.float32)
+    rt = gpt_ref.Runtime(cfg, params, compute_dtype=torch.float32, fp8=False)
+    g = torch.Generator().manual_seed(0)
+    prompt = torch.randint(0, 32768, (32,), generator=g).tolist()
+    decode_ref.generate(rt, prompt, 1, 4, temperature=0.0)            # one short run first (allocator, thread pool)
+    t0 = time.time()
+    out, _ = decode_ref.generate(rt, prompt, 1, 64, temperature=0.0)
+    dt = time.time() - t0
+    return {"tokens_per_s": round(len(out) / dt, 2), "seconds": round(dt, 3), "new_tokens": len(out), "prompt_tokens": 32,
+            "batch": 1, "dtype": "fp32, plain linears"}
+
+
+def cpu_baseline():
+    """The CPU oracle on this box's host cores, bounded samples: the headline configuration (configs[3]: d26, 64 rows, context
+    1792; up to 4 decode steps), configs[2] (d20, 8 rows, context 512; the first 8 decode steps), configs[0] in full (d4 fp32, one
+    row, 32-token prompt + 64 greedy tokens), and row samples of the isolated GEMM shapes (configs[1])."""
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    c4 = cpu_decode_leg(D26 | {"window_pattern": "SSSL"}, 2, BATCH, PROMPT_TOKENS, 4, 12.0, cores)
+    d20 = dict(sequence_len=2048, vocab_size=32768, n_layer=20, n_head=10, n_kv_head=10, n_embd=1280, window_pattern="SSSL")
+    c3 = cpu_decode_leg(d20, 1, 8, 512, 8, 8.0, cores)
+    c1 = cpu_config1_leg(cores)
+    return {"value": c4["tokens_per_s"], "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{c4['steps_timed']} decode step(s) of the CPU oracle at d26, 64 rows, context {PROMPT_TOKENS} (random-filled cache), "
+                      f"bf16 + fp8-emulated linears with per-call weight quantization as in the reference; setup "
+                      f"{c4['setup_s_not_timed']:.0f}s not timed",
+            "s_per_step": c4["s_per_step"],
+            "config3_d20_b8_ctx512": c3 | {"sample": f"first {c3['steps_timed']} decode steps, greedy, random-filled cache"},
+            "config1_d4_fp32_b1": c1 | {"sample": "full: 32-token prompt + 64 greedy tokens through the oracle's generate loop"},
             "fp8_gemm_m8192": cpu_gemm_baseline(cores)}
 
 
@@ -263,57 +307,39 @@ def measured_traffic():
         return None, "no counter summary under profiles/"
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=232)
-    ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-gemm", action="store_true")
-    ap.add_argument("--library-gemm", action="store_true", help="also time torch._scaled_mm on the M=8192 GEMM operands")
-    ap.add_argument("--profile-steps", type=int, default=16)
-    ap.add_argument("--window-pattern", default="SSSL",
-                    help="sliding-window pattern of the layers (the headline number is SSSL; L makes every layer read the whole context)")
-    ap.add_argument("--copy-probe-mib", type=int, default=0,
-                    help="after the decode steps, run an elementwise pass that reads and writes this many MiB "
-                         "(a kernel of known traffic to scale hardware byte counters with)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (decode would shard by batch row, one independent copy per GPU). "
-              "Run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
-    assert torch.cuda.is_available(), "bench.py needs the GPU"
-    from nanochat_amd import _lib
-    from nanochat_amd.engine import Engine
-    lib = _lib.lib()
-    device = torch.device("cuda:0")
-    torch.cuda.set_device(device)
+def set_window_pattern(model, pattern):
+    """Switch the sliding-window pattern of a built model: the weights do not depend on it, the per-layer windows of the plan do."""
+    from nanochat_amd.gpt import compute_window_sizes
+    model.config.window_pattern = pattern
+    model.window_sizes = compute_window_sizes(model.config)
+    model.invalidate_plan()
 
-    D26["window_pattern"] = args.window_pattern
-    K, W, P = args.steps, args.warmup, max(1, args.profile_steps)
-    total_new = W + P + K
-    prompt_len = CONTEXT - total_new          # the last timed step brings the context to 2048
-    assert prompt_len >= 1, "warmup + profile steps + steps must stay below the 2048-token context"
-    model = build_model(device)
+
+def run_decode(model, lib, K, W, P, pattern):
+    """The headline protocol on `model` with the given window pattern: 1792-token prompt, 64 rows, 256 greedy tokens; W warm-up steps,
+    untimed steps, P steps with a HIP event pair around every kernel launch, and the last K steps timed.  Returns the figures."""
+    from nanochat_amd.engine import Engine
+    set_window_pattern(model, pattern)
+    filler = NEW_TOKENS - (W + P + K)
     engine = Engine(model, RangeTokenizer())
     g = torch.Generator().manual_seed(2)
-    prompt = torch.randint(0, D26["vocab_size"], (prompt_len,), generator=g).tolist()
+    prompt = torch.randint(0, D26["vocab_size"], (PROMPT_TOKENS,), generator=g).tolist()
 
     # one-off work (FP8 weight quantization of the plan, workspace allocation) is kept out of the time to first token
     for _ in engine.generate(prompt[:64], num_samples=2, max_tokens=2, temperature=0.0):
         pass
     torch.cuda.synchronize()
-    gen = engine.generate(prompt, num_samples=BATCH, max_tokens=total_new + 1, temperature=0.0)
+    gen = engine.generate(prompt, num_samples=BATCH, max_tokens=NEW_TOKENS + 1, temperature=0.0)
     t_pre = time.perf_counter()
     next(gen)                                  # prefill + cache replication + first sample + first forward
     torch.cuda.synchronize()
     ttft = time.perf_counter() - t_pre
-    for _ in range(W - 1):
+    for _ in range(W - 1 + filler):
         next(gen)
     torch.cuda.synchronize()
+    first_profiled = PROMPT_TOKENS + W + filler         # cache length the first profiled forward starts from
 
-    # ---- kernel-level timing, HIP events on the launch stream, same process and state, inside the configured context:
-    # the forwards of these P steps see contexts prompt_len + W + 1 .. prompt_len + W + P
+    # ---- kernel-level timing, HIP events on the launch stream, same process and state, right in front of the timed steps
     lib.nc_profile_enable(1)
     for _ in range(P):
         next(gen)
@@ -341,8 +367,54 @@ def main():
         step_times.append(time.perf_counter() - t1)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    tok_per_s = BATCH * K / elapsed
     gen.close()
+    del gen, engine
+    att_ms, _, att_n = prof[0]
+    # the P profiled forwards ran at cache lengths first_profiled .. first_profiled + P - 1 (each then sees one more key: itself)
+    launches_per_step = model.config.n_layer
+    att_bytes_step = sum(attention_bytes_per_step(model, BATCH, first_profiled + j + 1) for j in range(P)) / P
+    att_avg_s = att_ms * 1e-3 / att_n
+    att_bytes_launch = att_bytes_step / launches_per_step
+    weight_bytes_step = sum(v["weight_bytes"] * (1 if k == "lm_head" else model.config.n_layer) for k, v in linears.items())
+    return {"tok_per_s": BATCH * K / elapsed, "ms_per_step": elapsed / K * 1e3, "ttft": ttft,
+            "tpot_ms_median": sorted(step_times)[len(step_times) // 2] * 1e3,
+            "att_bytes_launch": att_bytes_launch, "att_avg_s": att_avg_s, "att_n": att_n, "att_bytes_step": att_bytes_step,
+            "kernel_ms_per_step": {name: round(prof[c][0] / P, 3) for c, name in enumerate(["attention", "fp8_gemm", "quantize", "rows", "sampler"])},
+            "linears": linears, "weight_bytes_step": weight_bytes_step,
+            "profiled_steps_context": [first_profiled + 1, first_profiled + P], "filler": filler}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=232)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--no-pattern-l", action="store_true", help="skip the second run with every layer reading the whole context")
+    ap.add_argument("--library-gemm", action="store_true", help="also time torch._scaled_mm on the M=8192 GEMM operands")
+    ap.add_argument("--profile-steps", type=int, default=16)
+    ap.add_argument("--window-pattern", default="SSSL",
+                    help="sliding-window pattern of the layers (the headline number is SSSL; L makes every layer read the whole context)")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="after the decode steps, run an elementwise pass that reads and writes this many MiB "
+                         "(a kernel of known traffic to scale hardware byte counters with)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (decode would shard by batch row, one independent copy per GPU). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    from nanochat_amd import _lib
+    lib = _lib.lib()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    K, W = args.steps, max(1, args.warmup)
+    assert 1 <= K and W + K + 1 <= NEW_TOKENS, f"warmup + steps must leave at least one of the {NEW_TOKENS} new tokens for the profiled steps"
+    P = max(1, min(args.profile_steps, NEW_TOKENS - W - K))       # what the 256 new tokens leave room for
+    model = build_model(device)
+    r = run_decode(model, lib, K, W, P, args.window_pattern)
     if args.copy_probe_mib > 0:
         n = args.copy_probe_mib * (1 << 20) // 2
         src = torch.ones(n, dtype=torch.bfloat16, device=device)
@@ -351,53 +423,63 @@ def main():
             torch.mul(src, 1.0, out=dst)       # reads n*2 bytes, writes n*2 bytes
         torch.cuda.synchronize()
         del src, dst
-    att_ms, _, att_n = prof[0]
-    # the P profiled forwards ran at cache lengths prompt_len + W .. prompt_len + W + P - 1 (each then sees one more key: itself)
-    launches_per_step = model.config.n_layer
-    att_bytes_step = sum(attention_bytes_per_step(model, BATCH, prompt_len + W + j + 1) for j in range(P)) / P
-    att_avg_s = att_ms * 1e-3 / att_n
-    att_bytes_launch = att_bytes_step / launches_per_step
-    achieved = att_bytes_launch / att_avg_s
-    per_step_ms = {name: round(prof[c][0] / P, 3) for c, name in enumerate(["attention", "fp8_gemm", "quantize", "rows", "sampler"])}
+    achieved = r["att_bytes_launch"] / r["att_avg_s"]
     traffic, traffic_note = measured_traffic() if args.window_pattern == "SSSL" else (None, "counter summary exists for window pattern SSSL only")
-    weight_bytes_step = sum(v["weight_bytes"] * (1 if k == "lm_head" else model.config.n_layer) for k, v in linears.items())
 
     result = {
         "metric": "decode tokens/sec @ d26 bs64 ctx2048",
-        "value": round(tok_per_s, 1),
+        "value": round(r["tok_per_s"], 1),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": K,
-        "warmup": W,
-        "ms_per_step": round(elapsed / K * 1e3, 4),
+        "warmup": args.warmup,
+        "ms_per_step": round(r["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "fp8_e4m3 x fp8_e4m3 -> fp32 acc (linears), bf16 (KV cache, activations)",
         "data": "synthetic: random token ids, random-init weights of the d26 architecture (seed 2)",
-        "config": {"workload": f"nanochat d26 decode (BASELINE configs[3]), batch 64, prompt {prompt_len} tokens, {total_new} new tokens, "
-                               f"timed steps at context {CONTEXT - K}->{CONTEXT}, greedy, window pattern {args.window_pattern}, "
+        "config": {"workload": f"nanochat d26 decode (BASELINE configs[3]), batch 64, prompt {PROMPT_TOKENS} tokens, {NEW_TOKENS} new tokens, "
+                               f"timed: the last {K} steps, context {CONTEXT - K}->{CONTEXT}, greedy, window pattern {args.window_pattern}, "
                                "Engine.generate loop (sample + GPT.forward with KV cache per step)",
-                   "batch": BATCH, "context_end": CONTEXT, "prompt_tokens": prompt_len, "new_tokens": total_new,
-                   "profiled_steps_context": [prompt_len + W + 1, prompt_len + W + P]},
-        "tpot_ms_median": round(sorted(step_times)[len(step_times) // 2] * 1e3, 4),
-        "ttft_s": round(ttft, 3),
+                   "batch": BATCH, "context_end": CONTEXT, "prompt_tokens": PROMPT_TOKENS, "new_tokens": NEW_TOKENS,
+                   "untimed_steps_before_the_profiled_ones": W + r["filler"], "profiled_steps": P,
+                   "profiled_steps_context": r["profiled_steps_context"]},
+        "tpot_ms_median": round(r["tpot_ms_median"], 4),
+        "ttft_s": round(r["ttft"], 3),
         "roofline": {"bound": "hbm", "kernel": "attn_partial_kernel (+combine) per layer launch",
                      "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4),
                      "traffic": traffic, "traffic_source": traffic_note,
-                     "bytes_per_launch": int(att_bytes_launch), "avg_launch_us": round(att_avg_s * 1e6, 2),
-                     "launches_timed": att_n},
-        "kernel_ms_per_step": per_step_ms,
+                     "bytes_per_launch": int(r["att_bytes_launch"]), "avg_launch_us": round(r["att_avg_s"] * 1e6, 2),
+                     "launches_timed": r["att_n"]},
+        "kernel_ms_per_step": r["kernel_ms_per_step"],
         # the weight-streaming linears of the decode step against the HBM peak (HIP events around each launch, in-step)
-        "decode_linears": linears,
+        "decode_linears": r["linears"],
         # the reference's MBU numerator with the bytes really streamed: e4m3 weights + KV read at the profiled context
-        "step_bytes": {"weights_e4m3": weight_bytes_step, "kv_read": int(att_bytes_step),
-                       "frac_hbm_peak_whole_step": round((weight_bytes_step + att_bytes_step) / (elapsed / K) / HBM_PEAK, 4)},
+        "step_bytes": {"weights_e4m3": r["weight_bytes_step"], "kv_read": int(r["att_bytes_step"]),
+                       "frac_hbm_peak_whole_step": round((r["weight_bytes_step"] + r["att_bytes_step"]) / (r["ms_per_step"] * 1e-3) / HBM_PEAK, 4)},
     }
+    if args.window_pattern == "SSSL" and not args.no_pattern_l:
+        # the same configuration with every layer reading the whole context (22.7 GB of KV per step at context 2048): the case
+        # that is bound by KV reads alone; a shorter timed window, same prompt, same 256 new tokens
+        KL = min(K, 64)
+        PL = max(1, min(P, 8))
+        torch.cuda.empty_cache()
+        rl = run_decode(model, lib, KL, W, PL, "L")
+        ach_l = rl["att_bytes_launch"] / rl["att_avg_s"]
+        result["window_pattern_L"] = {
+            "value": round(rl["tok_per_s"], 1), "unit": "tokens/s", "ms_per_step": round(rl["ms_per_step"], 4), "steps": KL,
+            "workload": f"same model, prompt and batch with window pattern L; timed: the last {KL} of the {NEW_TOKENS} steps",
+            "roofline": {"bound": "hbm", "achieved": round(ach_l / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                         "frac": round(ach_l / HBM_PEAK, 4), "bytes_per_launch": int(rl["att_bytes_launch"]),
+                         "avg_launch_us": round(rl["att_avg_s"] * 1e6, 2), "launches_timed": rl["att_n"]},
+            "kernel_ms_per_step": rl["kernel_ms_per_step"],
+            "step_bytes": {"weights_e4m3": rl["weight_bytes_step"], "kv_read": int(rl["att_bytes_step"]),
+                           "frac_hbm_peak_whole_step": round((rl["weight_bytes_step"] + rl["att_bytes_step"]) / (rl["ms_per_step"] * 1e-3) / HBM_PEAK, 4)}}
     if not args.no_gemm:
         result["fp8_gemm_m8192"] = gemm_rates(device, args.library_gemm)
-    del gen, engine, model
+    del model
     torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
