@@ -121,7 +121,11 @@ def gemm_rates(device, library_gemm=False):
         quantize_ring_mb = len(ring) * a.numel() * 2 >> 20
         del ring
         tf = flops / (fwd_us * 1e-6) / 1e12
+        # the matrix pipe's own ceiling on this shape's activation bytes: pure MFMA, no memory traffic (power-managed clock)
+        ceil = mfma_ceiling(device, a8.view(torch.uint8), iters=12000)["these_operands"]
         out[f"K{K}_N{N}"] = {"us": round(fwd_us, 2), "tflops": round(tf, 1), "frac_fp8_peak": round(tf * 1e12 / FP8_PEAK, 4),
+                             "mfma_only_pflops_on_these_operands": ceil["pflops"], "mfma_only_clock_ghz": ceil["shader_clock_ghz"],
+                             "frac_of_mfma_only_rate": round(tf / 1e3 / ceil["pflops"], 4),
                              "quantize_us": round(qms / qn * 1e3, 2),
                              "quantize_gbps": round(qbytes / (qms * 1e-3) / 1e9, 1),
                              "quantize_frac_hbm_peak": round(qbytes / (qms * 1e-3) / HBM_PEAK, 4),
@@ -159,6 +163,33 @@ def gemm_rates(device, library_gemm=False):
             out[f"K{K}_N{N}"]["library_us"] = round(us, 2)
             out[f"K{K}_N{N}"]["library_tflops"] = round(2.0 * M * N * K / us / 1e6, 1)
             out[f"K{K}_N{N}"]["rel_l2_vs_library"] = float(((res.float() - ref.float()).norm() / ref.float().norm()).item())
+    return out
+
+
+def mfma_ceiling(device, operands=None, iters=30000):
+    """What the fp8 matrix cores sustain with nothing else running (nc_probe_fp8_mfma_ceiling): PFLOP/s and shader clock on all-zero
+    operands (the published peak) and on the given e4m3 bytes.  Two launches each; the second, on a warm and settled part, counts."""
+    from nanochat_amd import _lib
+    lib = _lib.lib()
+    clocks = torch.zeros(8, dtype=torch.int64, device=device)
+    flops = C.c_double()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for name, buf in (("zero_operands", None), ("these_operands", operands)):
+        if name == "these_operands" and buf is None:
+            continue
+        for _ in range(2):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.nc_probe_fp8_mfma_ceiling(C.c_void_p(buf.data_ptr()) if buf is not None else None,
+                                                     buf.numel() * buf.element_size() if buf is not None else 0, iters,
+                                                     C.c_void_p(clocks.data_ptr()), C.byref(flops), stream))
+            e1.record()
+            torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        ck = clocks.tolist()
+        out[name] = {"pflops": round(flops.value / (ms * 1e-3) / 1e15, 3), "ms": round(ms, 2),
+                     "shader_clock_ghz": round(ck[0] / (ck[1] * 10.0), 3) if ck[1] else None}
     return out
 
 
@@ -479,6 +510,11 @@ def main():
                            "frac_hbm_peak_whole_step": round((rl["weight_bytes_step"] + rl["att_bytes_step"]) / (rl["ms_per_step"] * 1e-3) / HBM_PEAK, 4)}}
     if not args.no_gemm:
         result["fp8_gemm_m8192"] = gemm_rates(device, args.library_gemm)
+        # the published 5.0 PFLOP/s is what all-zero operands sustain; random e4m3 bytes settle at a lower clock
+        rnd = torch.randint(0, 127, (1 << 20,), dtype=torch.uint8, device=device) | (torch.randint(0, 2, (1 << 20,), dtype=torch.uint8, device=device) << 7)
+        result["fp8_mfma_only"] = mfma_ceiling(device, rnd)
+        result["fp8_mfma_only"]["note"] = ("pure v_mfma_f32_16x16x128_f8f6f4 loop on every SIMD, no memory or LDS traffic: the rate the part's "
+                                           "power management sustains; these_operands = uniformly random finite e4m3 bytes")
     del model
     torch.cuda.empty_cache()
     if not args.no_cpu_baseline:

@@ -293,6 +293,16 @@ int nc_profile_read(int cls, double* total_ms /*host*/, double* total_units /*ho
 /* The FP8 GEMM launches (class 1) of one weight shape [N,K] only: the decode step's four linears and lm_head apart. */
 int nc_profile_read_gemm(int N, int K, double* total_ms /*host*/, double* total_units /*host*/, int64_t* count /*host*/);
 
+/* What the fp8 matrix cores of this GPU sustain on given operand bytes, with nothing else running (no counterpart in the
+ * reference; measurement aid): one 8-wave workgroup per CU issues `iters` rounds of 32 independent
+ * v_mfma_f32_16x16x128_f8f6f4 per wave on operands taken once from `operands` (device, e4m3 bytes, 32-byte aligned; NULL =
+ * all-zero operands) -- no memory or LDS traffic inside the loop.  The published peak is what all-zero operands reach; the
+ * part's power management settles at a lower clock on data whose bits toggle, so an FP8 GEMM on such data is bounded by this
+ * figure, not by the published one.  *flops_out (host): flops the launch performs; time it with events.  clocks_out (device,
+ * 8 x uint64 or NULL): for workgroups 0..3, shader-clock ticks and 100 MHz ticks spent in the loop (their ratio x 0.1 = GHz). */
+int nc_probe_fp8_mfma_ceiling(const uint8_t* operands, int64_t operand_bytes, int iters, uint64_t* clocks_out,
+                              double* flops_out /*host*/, nc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

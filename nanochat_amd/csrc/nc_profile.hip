@@ -69,4 +69,51 @@ int nc_profile_read(int cls, double* total_ms, double* total_units, int64_t* cou
 int nc_profile_read_gemm(int N, int K, double* total_ms, double* total_units, int64_t* count) {
     return profile_read_impl(1, true, ((int64_t)N << 32) | (uint32_t)K, total_ms, total_units, count);
 }
+
+// ---- the matrix pipe's own ceiling on given operand bytes -------------------------------------------------
+// One workgroup of 8 waves per CU; every wave issues `iters` rounds of 32 independent v_mfma_f32_16x16x128_f8f6f4 whose operands
+// come from registers (loaded once from `operands`, or all zero): no memory traffic, no LDS, nothing but the matrix pipe.  The
+// rate a long run of this kernel sustains is what the part's power management lets the fp8 matrix cores deliver on that data (the
+// published peak is reached on all-zero operands; random e4m3 bytes settle at a lower clock), i.e. the ceiling an FP8 GEMM on such
+// data is priced against.  clocks_out[2 i], [2 i + 1] (i < 4): shader-clock ticks and 100 MHz ticks that workgroup i spent in the loop.
+typedef int probe_v8i __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(512) void mfma_ceiling_kernel(const probe_v8i* __restrict__ operands, int n_frags, int iters,
+                                                           unsigned long long* __restrict__ clocks_out, float* __restrict__ sink) {
+    probe_v8i a[4], b[2];
+    const probe_v8i zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; i++) a[i] = operands ? operands[(threadIdx.x + 512u * i + 3072u * blockIdx.x) % (unsigned)n_frags] : zero;
+#pragma unroll
+    for (int i = 0; i < 2; i++) b[i] = operands ? operands[(threadIdx.x + 512u * (4 + i) + 3072u * blockIdx.x) % (unsigned)n_frags] : zero;
+    v4f acc[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    unsigned long long r0, r1;
+    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r0));
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 32; i++) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(b[i & 1]), "v"(a[i & 3]));
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r1));
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) t += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    if (t == 123.456f && sink) sink[0] = t;                    // keeps the loop alive; never true for finite sums of this size
+    if (threadIdx.x == 0 && blockIdx.x < 4 && clocks_out) clocks_out[2 * blockIdx.x] = c1 - c0, clocks_out[2 * blockIdx.x + 1] = r1 - r0;
+}
+
+int nc_probe_fp8_mfma_ceiling(const uint8_t* operands, int64_t operand_bytes, int iters, uint64_t* clocks_out, double* flops_out,
+                              nc_stream_t stream) {
+    NC_CHECK_ARG(iters > 0 && iters <= (1 << 22), "probe_fp8_mfma_ceiling: iters must be 1 .. 2^22");
+    NC_CHECK_ARG(!operands || (operand_bytes >= 32 && ((uintptr_t)operands & 31) == 0), "probe_fp8_mfma_ceiling: operands need 32-byte alignment and size");
+    NC_CHECK_ARG(!operands || operand_bytes / 32 < (1LL << 31), "probe_fp8_mfma_ceiling: at most 64 GiB of operand bytes");
+    const int cus = nc_cu_count();
+    hipLaunchKernelGGL(mfma_ceiling_kernel, dim3(cus), dim3(512), 0, (hipStream_t)stream, (const probe_v8i*)operands,
+                       operands ? (int)(operand_bytes / 32) : 1, iters, (unsigned long long*)clocks_out, (float*)nullptr);
+    NC_CHECK_LAUNCH("probe_fp8_mfma_ceiling");
+    if (flops_out) *flops_out = (double)cus * 8.0 * 32.0 * (double)iters * 65536.0;     // 2 * 16 * 16 * 128 per instruction
+    return 0;
+}
 }
