@@ -218,6 +218,133 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Any top_k beyond what the candidate sort above holds in LDS (4096 < top_k < V): the whole row is sorted, by a stable
+// least-significant-digit radix sort of the indices (three digits of 11 / 11 / 10 bits of the inverted order key, so ascending
+// digits are descending logits, and the initial index order makes equal logits come out lowest index first, like
+// torch.sort(descending=True, stable=True)).  The two index arrays (uint16: V <= 32768 ... 65536 entries of 2 bytes) and the three
+// digit histograms fill the LDS of one CU: 2 * 2 * V + 24 KB.  Counting is done by all four waves in one pass over the row;
+// the scatter of a pass must keep the order of equal digits, so one wave walks the sequence 64 entries at a time and ranks the
+// lanes of a round among themselves with ballots.  A rarely used path (the reference accepts any k, nanochat/engine.py:147-152):
+// correctness over speed, a few hundred microseconds per call.
+#define LK_BINS 2048
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_large_k_kernel(const float* __restrict__ logits, int V, int ld, float temperature,
+                                                                        int top_k, const float* __restrict__ noise,
+                                                                        int64_t* __restrict__ out_ids) {
+    extern __shared__ __align__(16) uint8_t lk_lds[];
+    __shared__ float sval[4];
+    __shared__ int sidx[4];
+    __shared__ float fsum[SAMPLE_THREADS];
+    uint32_t* hist = (uint32_t*)lk_lds;                                   // [3][LK_BINS]
+    uint16_t* ord_a = (uint16_t*)(lk_lds + 3 * LK_BINS * 4);
+    uint16_t* ord_b = ord_a + V;
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float* lr = logits + (size_t)row * ld;
+    auto digit_of = [](float v, int pass) -> uint32_t {
+        const uint32_t inv = ~fkey(v);                                    // ascending inv = descending logit
+        return pass == 0 ? (inv & 0x7ffu) : (pass == 1 ? ((inv >> 11) & 0x7ffu) : (inv >> 22));
+    };
+    // ---- digit counts of all three passes in one scan of the row
+    for (int i = tid; i < 3 * LK_BINS; i += SAMPLE_THREADS) hist[i] = 0;
+    __syncthreads();
+    scan_row(lr, V, tid, [&](float v, int) {
+        const uint32_t inv = ~fkey(v);
+        atomicAdd(&hist[inv & 0x7ffu], 1u);
+        atomicAdd(&hist[LK_BINS + ((inv >> 11) & 0x7ffu)], 1u);
+        atomicAdd(&hist[2 * LK_BINS + (inv >> 22)], 1u);
+    });
+    __syncthreads();
+    // ---- exclusive prefix sums, one histogram after the other: thread t owns bins 8t .. 8t+7
+    for (int h = 0; h < 3; h++) {
+        uint32_t* hh = hist + h * LK_BINS;
+        uint32_t local[8], sum = 0;
+#pragma unroll
+        for (int b = 0; b < 8; b++) local[b] = hh[8 * tid + b], sum += local[b];
+        fsum[tid] = __uint_as_float(sum);
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t run = 0;
+            for (int t = 0; t < SAMPLE_THREADS; t++) {
+                const uint32_t c = __float_as_uint(fsum[t]);
+                fsum[t] = __uint_as_float(run);
+                run += c;
+            }
+        }
+        __syncthreads();
+        uint32_t run = __float_as_uint(fsum[tid]);
+#pragma unroll
+        for (int b = 0; b < 8; b++) hh[8 * tid + b] = run, run += local[b];
+        __syncthreads();
+    }
+    // ---- three stable scatters by wave 0; indices travel ord_a -> ord_b -> ord_a -> ord_b (the first pass reads the identity)
+    if (wave == 0) {
+        const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+        for (int pass = 0; pass < 3; pass++) {
+            const uint16_t* src = (pass & 1) ? ord_b : ord_a;
+            uint16_t* dst = (pass & 1) ? ord_a : ord_b;
+            volatile uint32_t* offs = hist + pass * LK_BINS;
+            for (int base = 0; base < V; base += 4 * 64) {
+                // four rounds' worth of indices and logits are asked for at once (the gathers are what a round costs)
+                int idx[4];
+                float val[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int i = base + 64 * u + lane;
+                    idx[u] = i < V ? (pass == 0 ? i : (int)src[i]) : 0;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) val[u] = lr[idx[u]];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int i = base + 64 * u + lane;
+                    const bool valid = i < V;
+                    const uint32_t d = digit_of(val[u], pass);
+                    unsigned long long peers = __ballot(valid);
+#pragma unroll
+                    for (int b = 0; b < 11; b++) {
+                        const bool bit = (d >> b) & 1u;
+                        const unsigned long long bal = __ballot(bit && valid);
+                        peers &= bit ? bal : ~bal;
+                    }
+                    // lanes with the same digit: the lowest of them takes the digit's running offset and moves it on
+                    const int rank = __popcll(peers & lt_mask), cnt = __popcll(peers);
+                    uint32_t start = 0;
+                    if (valid && rank == 0) {
+                        start = offs[d];
+                        offs[d] = start + (uint32_t)cnt;
+                    }
+                    const int leader = valid ? (int)__ffsll((long long)peers) - 1 : lane;
+                    start = (uint32_t)__shfl((int)start, leader);
+                    if (valid) dst[start + rank] = (uint16_t)idx[u];
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");      // the next round reads the offsets this one moved
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const uint16_t* order = ord_b;                       // after three passes
+    const uint32_t k = (uint32_t)top_k;
+    // ---- softmax over the k best / T, then the draw: argmax_j (p_j / denom) / e_j, first j on equal quotients
+    const float vmax = lr[order[0]] / temperature;
+    float part = 0.f;
+    for (uint32_t j = tid; j < k; j += SAMPLE_THREADS) part += expf(lr[order[j]] / temperature - vmax);
+    fsum[tid] = part;
+    __syncthreads();
+    for (int o = SAMPLE_THREADS / 2; o > 0; o >>= 1) {   // a fixed tree: the same sum on every launch
+        if (tid < o) fsum[tid] += fsum[tid + o];
+        __syncthreads();
+    }
+    const float denom = fsum[0];
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (uint32_t j = tid; j < k; j += SAMPLE_THREADS) {
+        const float qv = (expf(lr[order[j]] / temperature - vmax) / denom) / noise[(size_t)row * k + j];
+        if (qv > bv) bv = qv, bi = (int)j;
+    }
+    block_argmax(bv, bi, sval, sidx);
+    if (tid == 0) out_ids[row] = (int64_t)order[(bi == 0x7fffffff) ? 0 : bi];
+}
+
 int nc_launch_softcap(const bf16_t* raw, float* out, int64_t n, float softcap, hipStream_t s) {
     NC_CHECK_ARG(raw && out && n >= 0 && softcap > 0.f, "softcap: bad arguments");
     int64_t g = (n + 255) / 256;
@@ -235,7 +362,24 @@ int nc_launch_sample(const float* logits, int B, int V, int ld, float temperatur
     NC_CHECK_ARG(temperature >= 0.0f, "sample: temperature must be non-negative");
     NC_CHECK_ARG(temperature == 0.0f || noise, "sample: temperature > 0 needs the exponential noise buffer");
     const int k_eff = (top_k > 0 && top_k < V) ? top_k : 0;
-    NC_CHECK_ARG(k_eff <= MAX_TOP_K, "sample: top_k %d exceeds the supported maximum of %d (or pass 0 for none)", top_k, MAX_TOP_K);
+    if (temperature > 0.0f && k_eff > MAX_TOP_K) {
+        // the whole row is sorted in the LDS of one CU
+        NC_CHECK_ARG(V <= 32768, "sample: top_k %d above %d needs the row's indices in LDS, which holds a vocabulary of at most 32768 (got %d)",
+                     top_k, MAX_TOP_K, V);
+        const size_t lds_bytes = 3 * LK_BINS * 4 + 2 * (size_t)V * sizeof(uint16_t);
+        static bool reserved[64];
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        if (dev < 0 || dev >= 64 || !reserved[dev]) {
+            const hipError_t e = hipFuncSetAttribute((const void*)sample_large_k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(3 * LK_BINS * 4 + 4 * 32768));
+            if (e != hipSuccess) NC_FAIL(-2, "sample: cannot reserve LDS for the large top_k path: %s", hipGetErrorString(e));
+            if (dev >= 0 && dev < 64) reserved[dev] = true;
+        }
+        NcProfScope prof(4, 4.0 * B * V, s);
+        hipLaunchKernelGGL(sample_large_k_kernel, dim3(B), dim3(SAMPLE_THREADS), lds_bytes, s, logits, V, ld, temperature, k_eff, noise, out_ids);
+        NC_CHECK_LAUNCH("sample");
+        return 0;
+    }
     NcProfScope prof(4, 4.0 * B * V, s);
     if (k_eff <= 256)
         hipLaunchKernelGGL(sample_kernel<256>, dim3(B), dim3(SAMPLE_THREADS), 0, s, logits, V, ld, temperature, k_eff, noise, out_ids);

@@ -890,12 +890,18 @@ def test_sample_argmax_first_index_on_ties(ops):
 @pytest.mark.parametrize("temperature,top_k,V", [(1.0, 50, 32768), (0.6, 50, 32768), (0.8, 1, 1000), (1.0, 256, 5000),
                                                  (1.3, None, 4096), (1.0, 500, 262),
                                                  # more candidates than threads: the 4096-entry instantiation, sorts of 512 .. 4096
-                                                 (1.0, 257, 32768), (0.9, 1000, 32768), (1.0, 4096, 32768), (0.7, 3000, 5000)])
+                                                 (1.0, 257, 32768), (0.9, 1000, 32768), (1.0, 4096, 32768), (0.7, 3000, 5000),
+                                                 # any k beyond that (the reference takes min(top_k, V), engine.py:147-152): the whole row is
+                                                 # sorted; few distinct values (bf16-rounded logits) make ties by index matter
+                                                 (1.0, 4097, 32768), (0.8, 20000, 32768), (1.0, 32767, 32768), (1.1, 4999, 5000),
+                                                 (0.9, 6000, 8191)])
 def test_sample_matches_oracle_given_the_same_noise(ops, temperature, top_k, V):
     say(f"sample T={temperature} k={top_k} V={V}")
     g = torch.Generator().manual_seed(7)
     B = 64
     logits = 15.0 * torch.tanh(torch.randn(B, V, generator=g) * 2 / 15.0)
+    if top_k is not None and top_k > 4096:
+        logits = logits.bfloat16().float()          # the logits of the model are bf16 values: many exact ties
     width = min(top_k, V) if top_k else V
     noise = torch.empty(B, width).exponential_(1.0, generator=g)
     want = decode_ref.sample_with_noise(logits, temperature, top_k, noise)
