@@ -133,18 +133,35 @@ def gemm_rates(device, library_gemm=False):
         # the two backward GEMMs of the same layer (nanochat/fp8.py:156-192): e5m2 gradient x e4m3 saved operands
         go = (torch.randn(M, N, device=device, generator=g) * 1e-3).bfloat16()
 
-        go8, igo, _ = ops.fp8_quantize(go, fp8_dtype=torch.float8_e5m2)
-        wT, goT, xT = ops.fp8_transpose(w8), ops.fp8_transpose(go8), ops.fp8_transpose(a8)
+        # what Float8Linear does under autograd: the output gradient quantized to e5m2 once, written as [M,N] and [N,M] by the same
+        # pass; the input's transposed payload saved by the forward's quantization; the transposed weight kept with the cached weight
+        go8, goT, igo, _ = ops.fp8_quantize_transposed(go, fp8_dtype=torch.float8_e5m2)
+        _, xT, _, _ = ops.fp8_quantize_transposed(a)
+        wT = ops.fp8_transpose(w8)
         gi = torch.empty(M, K, dtype=torch.bfloat16, device=device)
         gw = torch.empty(N, K, dtype=torch.bfloat16, device=device)
         dx_us = timed(lambda: ops.fp8_gemm_grad(go8, wT, igo, iw, out=gi))
         dw_us = timed(lambda: ops.fp8_gemm_grad(goT, xT, igo, ia, out=gw))
-        prep_us = timed(lambda: (ops.fp8_quantize(go, fp8_dtype=torch.float8_e5m2), ops.fp8_transpose(w8), ops.fp8_transpose(go8),
-                                 ops.fp8_transpose(a8)), warm=10, n=20)
+        # over rings of distinct tensors larger than the memory-side cache, like the forward's quantize figure
+        go_ring = [go] + [go.clone() for _ in range((320 << 20) // (go.numel() * 2) + 1)]
+        a_ring = [a] + [a.clone() for _ in range((320 << 20) // (a.numel() * 2) + 1)]
+        ring_i = [0]
+
+        def next_of(ring):
+            ring_i[0] += 1
+            return ring[ring_i[0] % len(ring)]
+        prep_us = timed(lambda: ops.fp8_quantize_transposed(next_of(go_ring), fp8_dtype=torch.float8_e5m2), warm=len(go_ring), n=2 * len(go_ring))
+        fwd_q_us = timed(lambda: ops.fp8_quantize_transposed(next_of(a_ring)), warm=len(a_ring), n=2 * len(a_ring))
+        old_prep_us = timed(lambda: (ops.fp8_quantize(next_of(go_ring), fp8_dtype=torch.float8_e5m2), ops.fp8_transpose(w8), ops.fp8_transpose(go8),
+                                     ops.fp8_transpose(a8)), warm=len(go_ring), n=2 * len(go_ring))
+        del go_ring, a_ring
         out[f"K{K}_N{N}"]["backward"] = {"grad_input_us": round(dx_us, 2), "grad_weight_us": round(dw_us, 2),
                                          "grad_input_tflops": round(2.0 * M * N * K / dx_us / 1e6, 1),
                                          "grad_weight_tflops": round(2.0 * M * N * K / dw_us / 1e6, 1),
-                                         "quantize_and_transposes_us": round(prep_us, 2)}
+                                         "quantize_and_transposes_us": round(prep_us, 2),
+                                         "quantize_and_transposes_over_gemms": round(prep_us / (dx_us + dw_us), 3),
+                                         "forward_quantize_with_transposed_copy_us": round(fwd_q_us, 2),
+                                         "separate_quantize_and_three_transposes_us": round(old_prep_us, 2)}
         if library_gemm:
             sa, sw = ia.reshape(()).float(), iw.reshape(()).float()
             a8t, w8t = a8.view(torch.float8_e4m3fn), w8.view(torch.float8_e4m3fn).t()

@@ -71,6 +71,14 @@ int nc_fp8_quantize_tensorwise_fused(const void* x, int x_dtype, int64_t n, int 
 int nc_fp8_quantize_tensorwise_fused_bounded(const void* x, int x_dtype, int64_t n, int fp8_format, uint8_t* out, float* scale_out,
                                              float* inv_scale_out, void* state, int encoder, uint32_t spin_limit, nc_stream_t stream);
 
+/* Tensorwise quantization of a bf16 matrix x[rows][cols] that writes the payload twice from one read of x: out[rows][cols] and
+ * out_t[cols][rows].  The backward GEMMs of nanochat/fp8.py:156-192 take the output gradient both ways (grad_output in e5m2 for
+ * grad_input, fp8.py:166-177; its transpose for grad_weight, fp8.py:179-190) and the saved input transposed (_to_col_major,
+ * fp8.py:110-118,181-182): the separate transposes of those payloads drop out.  Scale, inverse scale and payload bits are those of
+ * nc_fp8_quantize_tensorwise_as.  rows and cols multiples of 16, pointers 16-byte aligned; amax_ws: one uint32, cleared by the call. */
+int nc_fp8_quantize_tensorwise_transposed(const uint16_t* x, int rows, int cols, int fp8_format, uint8_t* out, uint8_t* out_t,
+                                          float* scale_out, float* inv_scale_out, uint32_t* amax_ws, nc_stream_t stream);
+
 /* dst[cols][rows] = transpose of the fp8 payload src[rows][cols]: the memory rearrangement of _to_col_major and
  * .t().contiguous() at nanochat/fp8.py:110-118,169,181-182 (the backward GEMMs want the summed index contiguous in
  * both operands).  rows and cols multiples of 16, pointers 16-byte aligned. */

@@ -17,7 +17,7 @@ EXPORTS = [
     "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read", "nc_profile_read_gemm",
     "nc_decode_attention_append", "nc_qkv_rope_append_attention", "nc_decode_attention_plan", "nc_gpt_forward_tapped",
     "nc_decode_attention_static", "nc_decode_attention_static_max_row_heads",
-    "nc_fp8_quantize_state_bytes", "nc_fp8_quantize_tensorwise_fused", "nc_fp8_quantize_tensorwise_fused_bounded", "nc_probe_fp8_mfma_ceiling",
+    "nc_fp8_quantize_state_bytes", "nc_fp8_quantize_tensorwise_fused", "nc_fp8_quantize_tensorwise_fused_bounded", "nc_probe_fp8_mfma_ceiling", "nc_fp8_quantize_tensorwise_transposed",
 ]
 
 
@@ -58,6 +58,7 @@ def _bind(lib):
         "nc_fp8_quantize_tensorwise_fused_bounded": (i, [p, i, i64, i, p, p, p, p, i, C.c_uint32, p]),
         "nc_fp8_encode_with_scale": (i, [p, i64, f, i, p, i, p]),
         "nc_fp8_transpose": (i, [p, i, i, p, p]),
+        "nc_fp8_quantize_tensorwise_transposed": (i, [p, i, i, i, p, p, p, p, p, p]),
         "nc_fp8_gemm_tn_grad": (i, [p, p, p, p, p, i, i, i, i, i, p]),
         "nc_fp8_gemm_tn_relu2": (i, [p, p, p, p, p, p, i, i, i, i, i, p]),
         "nc_fp8_gemm_tn": (i, [p, p, p, p, p, i, p, i, f, i, i, i, i, i, p, sz, p]),

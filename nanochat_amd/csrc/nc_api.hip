@@ -53,6 +53,11 @@ int nc_fp8_encode_with_scale(const uint16_t* x, int64_t n, float scale, int fp8_
     return nc_launch_encode_with_scale(x, n, scale, fp8_format, out, encoder, (hipStream_t)stream);
 }
 
+int nc_fp8_quantize_tensorwise_transposed(const uint16_t* x, int rows, int cols, int fp8_format, uint8_t* out, uint8_t* out_t, float* scale_out,
+                                          float* inv_scale_out, uint32_t* amax_ws, nc_stream_t stream) {
+    return nc_launch_quantize_transposed(x, rows, cols, fp8_format, out, out_t, scale_out, inv_scale_out, amax_ws, (hipStream_t)stream);
+}
+
 int nc_fp8_transpose(const uint8_t* src, int rows, int cols, uint8_t* dst, nc_stream_t stream) {
     return nc_launch_transpose_u8(src, rows, cols, dst, (hipStream_t)stream);
 }

@@ -16,6 +16,8 @@ int nc_launch_quantize(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* 
 int nc_launch_quantize_fused(const void* x, int x_dtype, int64_t n, int fmt, uint8_t* out, float* scale_out, float* inv_out,
                              uint32_t* state, int encoder, hipStream_t s, uint32_t spin_limit = NC_QUANTIZE_DEFAULT_SPINS);
 int nc_launch_transpose_u8(const uint8_t* src, int R, int C, uint8_t* dst, hipStream_t s);
+int nc_launch_quantize_transposed(const bf16_t* x, int R, int C, int fmt, uint8_t* out, uint8_t* out_t, float* scale_out, float* inv_out,
+                                  uint32_t* amax_ws, hipStream_t s);
 int nc_launch_convert_only(const void* x, int64_t n, uint8_t* out, float* inv_out, const uint32_t* amax_ws, hipStream_t s);
 int nc_launch_encode_with_scale(const bf16_t* x, int64_t n, float scale, int fmt, uint8_t* out, int encoder, hipStream_t s);
 

@@ -467,6 +467,86 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t* __rest
     }
 }
 
+// ---------------------------------------------------------------- convert + transpose in one pass
+// out[r][c] = fp8(x[r][c]) and out_t[c][r] = the same byte, from one read of x (amax already reduced into amax_bits): what the
+// backward GEMMs of nanochat/fp8.py:156-192 need of the output gradient (both grad_output in e5m2 and its transpose) and, saved by
+// the forward, of the input (its transpose for grad_weight).  128 x 128 tiles: every thread converts eight 16-byte pieces of bf16
+// (coalesced 256-byte row segments), stores the eight payload bytes row-major straight from registers (16 lanes = one 128-byte
+// line) and into an LDS copy of the tile, which then goes through the 4 x 4 byte transposes of transpose_u8_kernel.
+template <int FMT>
+__global__ __launch_bounds__(256) void convert_transpose_kernel(const bf16_t* __restrict__ x, int R, int C, const uint32_t* __restrict__ amax_bits,
+                                                                uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
+                                                                float* __restrict__ scale_out, float* __restrict__ inv_out) {
+    __shared__ __align__(16) uint8_t ta[128 * TP_PITCH], tb[128 * TP_PITCH];
+    const int r0 = blockIdx.y * 128, c0 = blockIdx.x * 128, t = threadIdx.x;
+    uint4 in[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = t + 256 * i, row = q >> 4, c8 = (q & 15) * 8;
+        in[i] = make_uint4(0, 0, 0, 0);
+        if (r0 + row < R && c0 + c8 < C) in[i] = *(const uint4*)(x + (size_t)(r0 + row) * C + c0 + c8);
+    }
+    const float scale = scale_from_amax(amax_read(amax_bits), fp8_max<FMT>());
+    if (blockIdx.x == 0 && blockIdx.y == 0 && t == 0) {
+        if (scale_out) *scale_out = scale;
+        *inv_out = 1.0f / scale;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = t + 256 * i, row = q >> 4, c8 = (q & 15) * 8;
+        const uint32_t w[4] = {in[i].x, in[i].y, in[i].z, in[i].w};
+        uint32_t o[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            o[j] = fp8_pack4<FMT, true>(fp8_clamp<FMT>(bf16_lo(w[2 * j]) * scale), fp8_clamp<FMT>(bf16_hi(w[2 * j]) * scale),
+                                        fp8_clamp<FMT>(bf16_lo(w[2 * j + 1]) * scale), fp8_clamp<FMT>(bf16_hi(w[2 * j + 1]) * scale));
+        *(uint2*)(ta + row * TP_PITCH + c8) = make_uint2(o[0], o[1]);
+        if (r0 + row < R && c0 + c8 < C) *(uint2*)(out + (size_t)(r0 + row) * C + c0 + c8) = make_uint2(o[0], o[1]);
+    }
+    __syncthreads();
+    const int lrow = t >> 3, lc16 = (t & 7) * 16;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int blk = t + 256 * i, rb = blk >> 5, cb = blk & 31;      // 4x4 block: rows 4 rb.., columns 4 cb..
+        uint32_t d[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) d[k] = *(const uint32_t*)(ta + (4 * rb + k) * TP_PITCH + 4 * cb);
+        const uint32_t t0 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400), t1 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602);
+        const uint32_t u0 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400), u1 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602);
+        const uint32_t o[4] = {__builtin_amdgcn_perm(u0, t0, 0x05040100), __builtin_amdgcn_perm(u0, t0, 0x07060302),
+                               __builtin_amdgcn_perm(u1, t1, 0x05040100), __builtin_amdgcn_perm(u1, t1, 0x07060302)};
+#pragma unroll
+        for (int k = 0; k < 4; k++) *(uint32_t*)(tb + (4 * cb + k) * TP_PITCH + 4 * rb) = o[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = lrow + 32 * i;          // a column of x
+        if (c0 + row < C && r0 + lc16 < R)
+            *(uint4*)(out_t + (size_t)(c0 + row) * R + r0 + lc16) = *(const uint4*)(tb + row * TP_PITCH + lc16);
+    }
+}
+
+int nc_launch_quantize_transposed(const bf16_t* x, int R, int C, int fmt, uint8_t* out, uint8_t* out_t, float* scale_out, float* inv_out,
+                                  uint32_t* amax_ws, hipStream_t s) {
+    NC_CHECK_ARG(R >= 0 && C >= 0, "fp8_quantize_transposed: negative shape");
+    NC_CHECK_ARG(inv_out && amax_ws, "fp8_quantize_transposed: null pointer");
+    NC_CHECK_ARG(fmt == 0 || fmt == 1, "fp8_quantize_transposed: format must be 0 (e4m3fn) or 1 (e5m2)");
+    if (R == 0 || C == 0) return 0;
+    NC_CHECK_ARG(x && out && out_t, "fp8_quantize_transposed: null pointer");
+    NC_CHECK_ARG(R % 16 == 0 && C % 16 == 0, "fp8_quantize_transposed: rows=%d and cols=%d must be multiples of 16", R, C);
+    NC_CHECK_ARG((((uintptr_t)x | (uintptr_t)out | (uintptr_t)out_t) & 15) == 0, "fp8_quantize_transposed: pointers must be 16-byte aligned");
+    const int64_t n = (int64_t)R * C;
+    nc_clear_u32(amax_ws, 1, s);
+    NcProfScope prof(2, 4.0 * n, s);             // 2 bytes read + 2 x 1 byte written per element
+    hipLaunchKernelGGL(amax_kernel<true>, dim3(grid_for(n / 8, 1024, 1024)), dim3(256), 0, s, (const void*)x, n, amax_ws);
+    const dim3 grid((C + 127) / 128, (R + 127) / 128);
+    if (fmt == 0) hipLaunchKernelGGL(convert_transpose_kernel<0>, grid, dim3(256), 0, s, x, R, C, amax_ws, out, out_t, scale_out, inv_out);
+    else hipLaunchKernelGGL(convert_transpose_kernel<1>, grid, dim3(256), 0, s, x, R, C, amax_ws, out, out_t, scale_out, inv_out);
+    NC_CHECK_LAUNCH("fp8_quantize_transposed");
+    return 0;
+}
+
 int nc_launch_transpose_u8(const uint8_t* src, int R, int C, uint8_t* dst, hipStream_t s) {
     NC_CHECK_ARG(R >= 0 && C >= 0, "fp8_transpose: negative shape");
     if (R == 0 || C == 0) return 0;

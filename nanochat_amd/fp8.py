@@ -6,7 +6,8 @@ convert_to_float8_training :243-266).  Differences that do not change results:
     version counter changes; the reference re-quantizes it on every call (fp8.py:136), which for an
     unchanged weight produces the same bytes;
   * without autograd (inference) no tensors are saved and the call is three launches; with autograd the
-    three GEMMs of _Float8Matmul (fp8.py:123-192) run: e4m3 x e4m3 forward, e5m2 x e4m3 for both gradients.
+    three GEMMs of _Float8Matmul (fp8.py:123-192) run: e4m3 x e4m3 forward, e5m2 x e4m3 for both gradients,
+    their transposed operands written by the quantization passes themselves instead of by separate copies.
 """
 import torch
 import torch.nn as nn
@@ -16,29 +17,52 @@ from .common import COMPUTE_DTYPE
 
 
 class _Float8Matmul(torch.autograd.Function):
-    """input_2d [B,K] @ weight[N,K]^T with the reference's three FP8 GEMMs (nanochat/fp8.py:123-192)."""
+    """input_2d [B,K] @ weight[N,K]^T with the reference's three FP8 GEMMs (nanochat/fp8.py:123-192).
+
+    The backward GEMMs want the summed index contiguous in both operands, which the reference gets from _to_col_major /
+    .t().contiguous() copies (fp8.py:110-118,169,181-182).  Here every quantization that feeds the backward writes its payload
+    both ways from one read of the bf16 tensor: the forward saves the input already transposed (when the weight needs a gradient),
+    the output gradient is quantized to e5m2 once into [B,N] and [N,B], and the transposed weight payload is kept with the module's
+    cached e4m3 weight.  Same payload bits and scales as the separate quantize + transpose passes."""
 
     @staticmethod
     def forward(ctx, input_2d, weight, module):
-        a8, inv_a, _ = ops.fp8_quantize(input_2d)
+        rows, _ = input_2d.shape
+        both_ways = weight.requires_grad and rows % 16 == 0
+        if both_ways:
+            a8, a8_t, inv_a, _ = ops.fp8_quantize_transposed(input_2d)
+        else:
+            a8, inv_a, _ = ops.fp8_quantize(input_2d)
+            a8_t = None
         w8, inv_w = module._weight_fp8()
-        ctx.save_for_backward(a8, inv_a, w8, inv_w)
+        ctx.module = module
+        ctx.input_saved_transposed = a8_t is not None
+        ctx.save_for_backward(a8_t if a8_t is not None else a8, inv_a, w8, inv_w)
         return ops.fp8_gemm(a8, w8, inv_a, inv_w)
 
     @staticmethod
     def backward(ctx, grad_output):
-        a8, inv_a, w8, inv_w = ctx.saved_tensors
+        a_saved, inv_a, w8, inv_w = ctx.saved_tensors
         if grad_output.dtype != torch.bfloat16:
             raise ValueError("Float8Linear: the GPU path computes in bf16")
+        grad_output = grad_output.contiguous()
+        need_in, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         # gradients in e5m2 (wider range), saved operands in e4m3 (fp8.py:163-165)
-        go8, inv_go, _ = ops.fp8_quantize(grad_output.contiguous(), fp8_dtype=torch.float8_e5m2)
+        go8_t = None
+        if need_w and grad_output.shape[0] % 16 == 0:
+            go8, go8_t, inv_go, _ = ops.fp8_quantize_transposed(grad_output, fp8_dtype=torch.float8_e5m2)
+        else:
+            go8, inv_go, _ = ops.fp8_quantize(grad_output, fp8_dtype=torch.float8_e5m2)
         grad_input = grad_weight = None
-        if ctx.needs_input_grad[0]:
+        if need_in:
             # grad_input [B,K] = grad_output [B,N] @ weight [N,K]: the summed index N must be contiguous in both (fp8.py:166-177)
-            grad_input = ops.fp8_gemm_grad(go8, ops.fp8_transpose(w8), inv_go, inv_w)
-        if ctx.needs_input_grad[1]:
+            grad_input = ops.fp8_gemm_grad(go8, ctx.module._weight_fp8_transposed(w8), inv_go, inv_w)
+        if need_w:
             # grad_weight [N,K] = grad_output^T [N,B] @ input [B,K]: B contiguous in both (fp8.py:179-190)
-            grad_weight = ops.fp8_gemm_grad(ops.fp8_transpose(go8), ops.fp8_transpose(a8), inv_go, inv_a)
+            if go8_t is None:
+                go8_t = ops.fp8_transpose(go8)
+            a8_t = a_saved if ctx.input_saved_transposed else ops.fp8_transpose(a_saved)
+            grad_weight = ops.fp8_gemm_grad(go8_t, a8_t, inv_go, inv_a)
         return grad_input, grad_weight, None
 
 
@@ -55,6 +79,14 @@ class Float8Linear(nn.Linear):
             cached = (key, payload, inv.reshape(1))
             self._fp8_cache = cached
         return cached[1], cached[2]
+
+    def _weight_fp8_transposed(self, w8):
+        """The [K,N] copy of the cached weight payload `w8` (the operand of grad_input), made once per weight version."""
+        cached = getattr(self, "_fp8_cache_t", None)
+        if cached is None or cached[0] is not w8:
+            cached = (w8, ops.fp8_transpose(w8))
+            self._fp8_cache_t = cached
+        return cached[1]
 
     def forward(self, input):
         if not input.is_cuda:

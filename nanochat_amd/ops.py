@@ -78,6 +78,29 @@ def fp8_quantize(x, encoder=0, fp8_dtype=torch.float8_e4m3fn, spin_limit=None):
     return out.view(fp8_dtype), scales[1], scales[0]
 
 
+def fp8_quantize_transposed(x, fp8_dtype=torch.float8_e4m3fn):
+    """Tensorwise fp8 quantization of a bf16 matrix [R,C] that also writes the transposed payload [C,R] from the same read (what the
+    backward GEMMs of nanochat/fp8.py:156-192 take: grad_output both ways, the saved input transposed).
+
+    Returns (payload [R,C], payload_t [C,R], inv_scale fp32 0-dim, scale fp32 0-dim); the bits are those of fp8_quantize."""
+    _need_cuda(x)
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise ValueError("fp8_quantize_transposed: a 2-D bf16 tensor is required")
+    if fp8_dtype not in _FP8_FORMATS:
+        raise ValueError(f"fp8_quantize_transposed: format {fp8_dtype} not supported (float8_e4m3fn or float8_e5m2)")
+    x = x.contiguous()
+    R, Cc = x.shape
+    out = torch.empty(R, Cc, dtype=torch.uint8, device=x.device)
+    out_t = torch.empty(Cc, R, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(2, dtype=torch.float32, device=x.device)
+    state = _quantize_state(x.device)
+    scratch = C.c_void_p(state.data_ptr() + 4 * 320)          # the state block's scratch word
+    _lib.check(_lib.lib().nc_fp8_quantize_tensorwise_transposed(_ptr(x), R, Cc, _FP8_FORMATS[fp8_dtype], _ptr(out), _ptr(out_t),
+                                                                C.c_void_p(scales.data_ptr()), C.c_void_p(scales.data_ptr() + 4), scratch,
+                                                                _stream()))
+    return out.view(fp8_dtype), out_t.view(fp8_dtype), scales[1], scales[0]
+
+
 def fp8_encode_with_scale(x_bf16, scale, fp8_dtype, encoder=0):
     """The saturating cast alone, with a given scale (nanochat/fp8.py:100-103); returns uint8 payload bytes."""
     _need_cuda(x_bf16)

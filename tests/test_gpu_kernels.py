@@ -511,6 +511,25 @@ def test_fp8_transpose_is_exact(ops, R, C):
         ops.fp8_transpose(torch.zeros(24, 40, dtype=torch.uint8, device=DEV))        # not multiples of 16
 
 
+@pytest.mark.parametrize("R,C", [(128, 128), (16, 16), (48, 144), (8192, 1664), (2048, 6656), (400, 1648), (1664, 208)])
+@pytest.mark.parametrize("fmt", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_quantize_with_transposed_copy_is_the_quantizer_plus_an_exact_transpose(ops, R, C, fmt):
+    """One pass that writes the payload both ways (what the backward GEMMs of nanochat/fp8.py:156-192 read): bit for bit the oracle's
+    payload and scales, and its exact transpose, including partial 128 x 128 tiles."""
+    say(f"quantize + transposed copy {R}x{C} {fmt}")
+    g = torch.Generator().manual_seed(R * 7 + C)
+    x = torch.randn(R, C, generator=g) * (1e-3 if fmt == torch.float8_e5m2 else 1.0)
+    x = torch.where(torch.rand(R, C, generator=g) < 0.001, x * 30, x).bfloat16()
+    want_p, want_inv, want_s = fp8_ref.to_fp8(x, fmt)
+    p, pt, inv, sc = ops.fp8_quantize_transposed(x.to(DEV), fp8_dtype=fmt)
+    assert p.shape == (R, C) and pt.shape == (C, R) and p.dtype == fmt and pt.dtype == fmt
+    assert f32_bits(sc.item()) == f32_bits(want_s.item()) and f32_bits(inv.item()) == f32_bits(want_inv.item())
+    assert torch.equal(p.view(torch.uint8).cpu(), want_p.view(torch.uint8))
+    assert torch.equal(pt.view(torch.uint8).cpu(), want_p.view(torch.uint8).t().contiguous())
+    with pytest.raises((AssertionError, ValueError)):
+        ops.fp8_quantize_transposed(torch.zeros(24, 40, dtype=torch.bfloat16, device=DEV))        # not multiples of 16
+
+
 @pytest.mark.parametrize("M,N,K,kernel", [
     (300, 320, 256, 5), (64, 128, 400, 5), (513, 272, 1664, 5), (2100, 1300, 48, 5),
     (300, 320, 256, 8), (513, 272, 1664, 8), (4100, 2100, 384, 8),
