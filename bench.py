@@ -363,7 +363,7 @@ def set_window_pattern(model, pattern):
     model.invalidate_plan()
 
 
-def run_decode(model, lib, K, W, P, pattern):
+def run_decode(model, lib, K, W, P, pattern, share_prompt_reads=False):
     """The headline protocol on `model` with the given window pattern: 1792-token prompt, 64 rows, 256 greedy tokens; W warm-up steps,
     untimed steps, P steps with a HIP event pair around every kernel launch, and the last K steps timed.  Returns the figures."""
     from nanochat_amd.engine import Engine
@@ -377,7 +377,7 @@ def run_decode(model, lib, K, W, P, pattern):
     for _ in engine.generate(prompt[:64], num_samples=2, max_tokens=2, temperature=0.0):
         pass
     torch.cuda.synchronize()
-    gen = engine.generate(prompt, num_samples=BATCH, max_tokens=NEW_TOKENS + 1, temperature=0.0)
+    gen = engine.generate(prompt, num_samples=BATCH, max_tokens=NEW_TOKENS + 1, temperature=0.0, share_prompt_reads=share_prompt_reads)
     t_pre = time.perf_counter()
     next(gen)                                  # prefill + cache replication + first sample + first forward
     torch.cuda.synchronize()
@@ -440,6 +440,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--no-pattern-l", action="store_true", help="skip the second run with every layer reading the whole context")
+    ap.add_argument("--no-shared-prompt", action="store_true", help="skip the extra run that reads the replicated prompt once for all rows")
     ap.add_argument("--library-gemm", action="store_true", help="also time torch._scaled_mm on the M=8192 GEMM operands")
     ap.add_argument("--profile-steps", type=int, default=16)
     ap.add_argument("--window-pattern", default="SSSL",
@@ -525,6 +526,17 @@ def main():
             "kernel_ms_per_step": rl["kernel_ms_per_step"],
             "step_bytes": {"weights_e4m3": rl["weight_bytes_step"], "kv_read": int(rl["att_bytes_step"]),
                            "frac_hbm_peak_whole_step": round((rl["weight_bytes_step"] + rl["att_bytes_step"]) / (rl["ms_per_step"] * 1e-3) / HBM_PEAK, 4)}}
+    if args.window_pattern == "SSSL" and not args.no_shared_prompt:
+        # Not the headline: the same run with Engine.generate(share_prompt_reads=True).  The 64 rows are copies of one prompt
+        # (that is how Engine.generate builds a batch), so the full-context layers can read the prompt's keys and values once for
+        # all rows on the matrix cores and stream per row only the tokens decoded since; `value` above reads every row's copy.
+        torch.cuda.empty_cache()
+        rs = run_decode(model, lib, K, W, P, "SSSL", share_prompt_reads=True)
+        result["shared_prompt_reads"] = {
+            "value": round(rs["tok_per_s"], 1), "unit": "tokens/s", "ms_per_step": round(rs["ms_per_step"], 4), "steps": K,
+            "workload": "same model, prompt, batch and window pattern; the full-context layers read the replicated prompt once for all rows "
+                        "(Engine.generate(share_prompt_reads=True), off by default)",
+            "kernel_ms_per_step": rs["kernel_ms_per_step"], "tpot_ms_median": round(rs["tpot_ms_median"], 4)}
     if not args.no_gemm:
         result["fp8_gemm_m8192"] = gemm_rates(device, args.library_gemm)
         # the published 5.0 PFLOP/s is what all-zero operands sustain; random e4m3 bytes settle at a lower clock

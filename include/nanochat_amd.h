@@ -194,6 +194,22 @@ int nc_qkv_rope_append_attention(const uint16_t* qkv, int ld_qkv, const uint16_t
                                  int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax, int vocab_rows,
                                  void* workspace, size_t workspace_bytes, uint32_t* amax_ws, int splits, nc_stream_t stream);
 
+/* nc_decode_attention (one new token per row, already appended) for a batch whose rows all begin with the same shared_len cached
+ * tokens and sit at the same position: what Engine.generate builds, one prompt prefilled at batch 1 and its cache copied to every
+ * row (nanochat/engine.py:198-214, KVCache.prefill :123-137).  The caches keep the reference's layout and contents, every row
+ * holding its copy; the call reads positions [0, shared_len) from row 0 only, once for all rows, on the bf16 matrix cores, and
+ * streams per row only the row's own tail [shared_len, p], then merges the two parts of the softmax: the result is that of
+ * nc_decode_attention to rounding (sums in another order; the shared part's weights pass through bf16 like in the
+ * many-queries kernel), the cache bytes read drop from B x n_keys to shared + B x own.  CONTRACT: rows [0, shared_len) of
+ * every batch row hold identical bytes, cache_seqlens[b] is the same for all b and >= shared_len.  workspace:
+ * nc_decode_attention_shared_workspace_bytes() bytes, 16-byte aligned.  Shapes with too few rows for the per-row kernel to run
+ * unsplit are refused (-1): use nc_decode_attention.  No counterpart in the reference's attention seam. */
+size_t nc_decode_attention_shared_workspace_bytes(int B, int H, int Hkv, int shared_len);
+int nc_decode_attention_shared(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int32_t* cache_seqlens,
+                               int shared_len, int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax,
+                               int seqlens_include_new, void* workspace, size_t workspace_bytes, uint32_t* amax_ws,
+                               nc_stream_t stream);
+
 /* nc_decode_attention for callers that cannot allocate device memory and have no workspace to hand over: code under HIP
  * graph capture, tight serving loops, harnesses that forbid allocation.  It has no counterpart in the reference.  Same
  * arguments and results as nc_decode_attention minus the workspace: the split counters and partial results live in a
@@ -270,6 +286,12 @@ typedef struct nc_cache_desc {
     const uint16_t* prev_in;     /* bf16 [B,E] or NULL: KVCache.prev_embedding */
     uint16_t* prev_out;          /* bf16 [B,E]: the value to keep for the next call */
     int batch, max_seq_len;
+    /* Rows that share their first tokens (optional; 0 = every row reads its own cache everywhere).  shared_prefix > 0 promises that
+     * positions [0, shared_prefix) of every batch row hold identical bytes in every layer (KVCache.prefill from a batch-1 cache,
+     * nanochat/engine.py:123-137) and that all rows sit at the same position uniform_pos (= cache_seqlens[b] for all b, a host copy)
+     * >= shared_prefix.  A one-token-per-row forward then reads the shared keys of full-context layers once for all rows
+     * (nc_decode_attention_shared); results equal to rounding, the caches themselves are untouched by the promise. */
+    int shared_prefix, uniform_pos;
 } nc_cache_desc;
 
 size_t nc_gpt_workspace_bytes(const nc_model_desc* model /*host*/, int B, int T);

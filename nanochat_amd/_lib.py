@@ -18,6 +18,7 @@ EXPORTS = [
     "nc_decode_attention_append", "nc_qkv_rope_append_attention", "nc_decode_attention_plan", "nc_gpt_forward_tapped",
     "nc_decode_attention_static", "nc_decode_attention_static_max_row_heads",
     "nc_fp8_quantize_state_bytes", "nc_fp8_quantize_tensorwise_fused", "nc_fp8_quantize_tensorwise_fused_bounded", "nc_probe_fp8_mfma_ceiling", "nc_fp8_quantize_tensorwise_transposed",
+    "nc_decode_attention_shared", "nc_decode_attention_shared_workspace_bytes",
 ]
 
 
@@ -39,7 +40,8 @@ class ModelDesc(C.Structure):
 
 class CacheDesc(C.Structure):
     _fields_ = [("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("cache_seqlens", C.c_void_p),
-                ("prev_in", C.c_void_p), ("prev_out", C.c_void_p), ("batch", C.c_int), ("max_seq_len", C.c_int)]
+                ("prev_in", C.c_void_p), ("prev_out", C.c_void_p), ("batch", C.c_int), ("max_seq_len", C.c_int),
+                ("shared_prefix", C.c_int), ("uniform_pos", C.c_int)]
 
 
 _lib = None
@@ -75,6 +77,8 @@ def _bind(lib):
         "nc_qkv_rope_append_attention": (i, [p, i, p, i, p, p, p, p, p, i, p, p, p, i, p, i, i, i, i, i, p, sz, p, i, p]),
         "nc_decode_attention_static": (i, [p, p, p, p, i, p, i, i, i, i, i, i, p, i, p]),
         "nc_decode_attention_static_max_row_heads": (sz, []),
+        "nc_decode_attention_shared_workspace_bytes": (sz, [i, i, i, i]),
+        "nc_decode_attention_shared": (i, [p, p, p, p, i, i, p, i, i, i, i, i, p, sz, p, p]),
         "nc_decode_attention_plan": (i, [i, i, i, i, i, i, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
         "nc_kv_cache_prefill": (i, [p, p, i, i, i, i, i, i, i, p]),
         "nc_softcap": (i, [p, p, i64, f, p]),

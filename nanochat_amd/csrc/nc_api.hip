@@ -18,7 +18,7 @@ void nc_set_error(const char* fmt, ...) {
 
 extern "C" {
 
-int nc_abi_version(void) { return 1; }
+int nc_abi_version(void) { return 2; }
 const char* nc_last_error(void) { return g_error; }
 
 int nc_fp8_quantize_tensorwise(const void* x, int x_dtype, int64_t n, uint8_t* out, float* scale_out, float* inv_scale_out,
@@ -166,6 +166,21 @@ int nc_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16
     void* parts = counters ? (uint8_t*)workspace + cb : nullptr;
     return nc_launch_attention(q, k_cache, v_cache, cache_seqlens, window_left, out, B, T, H, Hkv, Tmax, seqlens_include_new,
                                counters, parts, counters ? workspace_bytes - cb : 0, amax_ws, splits, 0, (hipStream_t)stream);
+}
+
+size_t nc_decode_attention_shared_workspace_bytes(int B, int H, int Hkv, int shared_len) {
+    if (B <= 0 || H <= 0 || Hkv <= 0 || shared_len <= 0 || H % Hkv != 0) return 0;
+    return nc_attn_shared_partial_bytes(B, H, Hkv, shared_len);
+}
+
+int nc_decode_attention_shared(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int32_t* cache_seqlens,
+                               int shared_len, int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax, int seqlens_include_new,
+                               void* workspace, size_t workspace_bytes, uint32_t* amax_ws, nc_stream_t stream) {
+    NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && out && workspace, "decode_attention_shared: null pointer");
+    const int rc = nc_launch_attention_shared(q, k_cache, v_cache, cache_seqlens, shared_len, window_left, out, B, H, Hkv, Tmax,
+                                              seqlens_include_new, workspace, workspace_bytes, amax_ws, (hipStream_t)stream);
+    if (rc == -3) NC_FAIL(-1, "decode_attention_shared: this shape splits the keys of a row over workgroups (too few rows); use nc_decode_attention");
+    return rc;
 }
 
 static void split_attention_workspace(void* workspace, size_t workspace_bytes, int B, int T, int H, uint32_t** counters, void** parts,

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
                                                            float* __restrict__ partials, uint32_t* __restrict__ counters,
                                                            uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, int nsplit,
-                                                           NcRopeSrc rope) {
+                                                           NcRopeSrc rope, int k_min, const float* __restrict__ extra, int n_extra) {
     constexpr bool FUSED = MODE != 0;                    // the row's own token comes from LDS, not from the cache
     constexpr int KPI = 4 / HP;                          // keys per load instruction
     constexpr int TASKS = (G + 2) * HP;                  // FUSED: per head the G query heads, then the new key and value
@@ -66,6 +66,9 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     if (hi > Tmax - 1) hi = Tmax - 1;
     int lo = (window_left < 0) ? 0 : hi - window_left;
     if (lo < 0) lo = 0;
+    // keys below k_min are somebody else's: the shared start of all rows, whose part of the softmax arrives in `extra`
+    // (attn_shared_prefix_kernel) and is merged in with the four waves' parts below
+    if (lo < k_min) lo = k_min < hi ? k_min : hi;
     // keys streamed from the cache: [lo, k_stop); the fused kernel takes key hi (its own token) from LDS
     const int k_stop = FUSED ? hi : hi + 1;
     const int n_keys = k_stop - lo;
@@ -293,6 +296,10 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         float mm = NEG_BIG;
 #pragma unroll
         for (int w = 0; w < 4; w++) mm = fmaxf(mm, merge[w][hg][0]);
+        const int head = (hp * HP + hg / G) * G + hg % G;
+        const float* ex = extra ? extra + ((size_t)row * H + head) * n_extra * PART_STRIDE : nullptr;
+        if (ex)
+            for (int e = 0; e < n_extra; e++) mm = fmaxf(mm, ex[e * PART_STRIDE]);
         float ls = 0.f, a = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
@@ -300,7 +307,12 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             ls += merge[w][hg][1] * sc;
             a += merge[w][hg][4 + d] * sc;
         }
-        const int head = (hp * HP + hg / G) * G + hg % G;
+        if (ex)
+            for (int e = 0; e < n_extra; e++) {
+                const float sc = exp2f(ex[e * PART_STRIDE] - mm);
+                ls += ex[e * PART_STRIDE + 1] * sc;
+                a += ex[e * PART_STRIDE + 4 + d] * sc;
+            }
         if (nsplit == 1) {
             const bf16_t o = f32_to_bf16(a / ls);
             out[((size_t)row * H + head) * 128 + d] = o;
@@ -373,7 +385,8 @@ int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax) {
 static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, int mode, bf16_t* k_cache, bf16_t* v_cache,
                                  const int32_t* cache_seqlens, int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax,
                                  int seqlens_include_new, uint32_t* counters, void* partials, size_t partial_bytes, uint32_t* amax_ws,
-                                 int force_splits, int counters_are_zero, hipStream_t s) {
+                                 int force_splits, int counters_are_zero, hipStream_t s, int k_min = 0, const float* extra = nullptr,
+                                 int n_extra = 0) {
     NC_CHECK_ARG((q || mode == 1) && k_cache && v_cache && cache_seqlens && out, "decode_attention: null pointer");
     // many queries per row: the matrix-core kernel (a workgroup there covers 128 queries; below 16 queries per row
     // the per-query streaming kernel wastes less)
@@ -406,6 +419,8 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, int mod
         NC_CHECK_ARG(((uintptr_t)partials & 15) == 0, "decode_attention: workspace must be 16-byte aligned");
         if (!counters_are_zero) nc_clear_u32(counters, B * T * Hkv, s);
     }
+    NC_CHECK_ARG(!extra || (nsplit == 1 && mode == 0 && T == 1 && n_extra > 0 && k_min > 0),
+                 "decode_attention: a shared first part goes with one split, one query per row and tokens already appended");
     NcProfScope prof(0, 0.0, s);
     float* parts = (float*)partials;
     const int hp = (force_splits > 0 || nsplit > 1) ? 1 : pick_heads_per_wg(B, T, Hkv);
@@ -414,7 +429,7 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, int mod
     const NcRopeSrc& rs = rope ? *rope : none;
 #define LAUNCH_GMH(GG, MM, HH)                                                                                                \
     hipLaunchKernelGGL((attn_partial_kernel<GG, MM, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens, window_left, \
-                       seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, rs)
+                       seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, rs, k_min, extra, n_extra)
 #define LAUNCH_GH(GG, HH)                          \
     do {                                           \
         if (mode == 1) LAUNCH_GMH(GG, 1, HH);      \
@@ -462,6 +477,28 @@ int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, 
                               uint32_t* amax_ws, int force_splits, int counters_are_zero, hipStream_t s) {
     return launch_attention_impl(nullptr, &rope, 1, k_cache, v_cache, cache_seqlens, window_left, out, B, 1, H, Hkv, Tmax, 0, counters,
                                  partials, partial_bytes, amax_ws, force_splits, counters_are_zero, s);
+}
+
+// Decode attention for rows that share their first `shared_len` cached tokens (one prompt replicated to every row,
+// nanochat/engine.py:198-214) and sit at the same position: the shared keys are read once for all rows on the matrix cores
+// (attn_shared_prefix_kernel, from row 0 of the cache), the per-row kernel streams only each row's own tail [shared_len, p] and merges
+// the two parts.  One new token per row, already appended.  shared_parts: nc_attn_shared_partial_bytes() bytes.  Returns -3 without
+// launching anything when the shape does not take this path (the per-row kernel would split its keys over workgroups): the caller
+// then uses the plain entry.
+int nc_launch_attention_shared(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int shared_len,
+                               int window_left, bf16_t* out, int B, int H, int Hkv, int Tmax, int seqlens_include_new, void* shared_parts,
+                               size_t shared_part_bytes, uint32_t* amax_ws, hipStream_t s) {
+    NC_CHECK_ARG(B > 0 && H > 0 && Hkv > 0 && Tmax > 0 && H % Hkv == 0, "decode_attention_shared: bad shape");
+    NC_CHECK_ARG(shared_len > 0 && shared_len < Tmax, "decode_attention_shared: shared length %d outside (0, %d)", shared_len, Tmax);
+    const int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
+    if (pick_splits(B, 1, Hkv, max_keys) != 1) return -3;       // (what the per-row launch below will decide for itself)
+    int nchunks = 0;
+    int rc = nc_launch_attention_shared_prefix(q, k_cache, v_cache, cache_seqlens, shared_len, window_left, seqlens_include_new,
+                                               (float*)shared_parts, shared_part_bytes, B, H, Hkv, Tmax, &nchunks, s);
+    if (rc) return rc;
+    return launch_attention_impl(q, nullptr, 0, const_cast<bf16_t*>(k_cache), const_cast<bf16_t*>(v_cache), cache_seqlens, window_left, out, B, 1,
+                                 H, Hkv, Tmax, seqlens_include_new, nullptr, nullptr, 0, amax_ws, 0, 1, s, shared_len, (const float*)shared_parts,
+                                 nchunks);
 }
 
 // cache[b, cache_seqlens[b] + t] = new[b, t] for keys and values (nanochat/flash_attention.py:167-170 with per-row positions);

@@ -282,6 +282,250 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The shared part of a decode step whose rows all start with the same tokens (Engine.generate prefills one prompt at batch 1 and
+// replicates its cache to every row, nanochat/engine.py:198-214): positions [0, shared_len) of every row of the cache hold the same
+// keys and values, so the new token of every row attends to ONE copy of them.  The rows play the part that the query positions
+// play in the kernel above: a workgroup takes up to 128 / (GS * KS) rows x GS query heads of one kv head and a chunk of the shared
+// keys, read from row 0 of the cache, once for all of its rows, and multiplies on the matrix cores (the per-row streaming kernel
+// would pull the same bytes through every CU once per row: 64 rows x 1792 keys x 13 heads x 512 B = 763 MB per layer instead of
+// 12 MB).  All rows sit at the same position (cache_seqlens[0], the Engine's loop), every query sees the same keys
+// [max(0, p - window), shared_len), and nothing is masked inside that range.  The result is not normalised: per (row, head, chunk)
+// the running maximum (log2 units), the sum of weights and the weighted value sums, which the per-row kernel merges with what it
+// finds in the row's own tail of the cache (attn_partial_kernel, `extra`).
+#define SP_PART_STRIDE 132     // floats per partial: m, l, pad, pad, acc[128] (the layout of the per-row kernel's split partials)
+template <int GS, int KS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_shared_prefix_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
+    int shared_len, int window_left, int seqlens_include_new, float* __restrict__ partials, int nparts, int chunk_keys, int nqtiles, int rows,
+    int H, int Hkv, int Tmax) {
+    constexpr int QT = 128 / (GS * KS);                        // rows per workgroup
+    __shared__ __align__(16) uint8_t lds[2 * PF_KBYTES + 2 * PF_VBYTES];
+    uint8_t* const lds_k = lds;
+    uint8_t* const lds_v = lds + 2 * PF_KBYTES;
+    const lds_u8_t lds_v3 = (lds_u8_t)lds + 2 * PF_KBYTES;
+    const int G = H / Hkv, parts = G / GS;
+    const int qb0 = ((int)blockIdx.x % nqtiles) * QT, chunk = (int)blockIdx.x / nqtiles, hy = blockIdx.y;
+    const int hk = hy / parts;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = hk * G + (hy % parts) * GS + wave % GS;
+    const int ks = (wave / GS) % KS;
+    const int qw0 = qb0 + (wave / (GS * KS)) * 32;             // first row of this wave
+    const int col = lane & 31, hl = lane >> 5;
+    const int t = qw0 + col;                                   // this lane's row of the batch
+    const bool q_ok = t < rows;
+
+    // keys of this chunk that the step sees: [k_lo, k_hi], the same for every row
+    const int pos = cache_seqlens[0] - (seqlens_include_new ? 1 : 0);
+    int k_lo = window_left < 0 ? 0 : max(0, pos - window_left);
+    k_lo = max(k_lo, chunk * chunk_keys);
+    const int k_hi = min(min(shared_len, pos), (chunk + 1) * chunk_keys) - 1;
+    float* part = partials + (((size_t)(q_ok ? t : 0) * H + h) * nparts + chunk) * SP_PART_STRIDE;
+    if (k_lo > k_hi) {
+        // nothing of this chunk is visible: a partial of weight zero
+        if (q_ok && ks == 0) {
+            if (hl == 0) part[0] = PF_M_FLOOR, part[1] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) *(float4*)(part + 4 + 64 * hl + 4 * i) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        return;
+    }
+    const int kb_first = k_lo & ~63;
+
+    v8bf qf[8];
+    {
+        const bf16_t* qrow = q + ((size_t)(q_ok ? t : rows - 1) * H + h) * 128;
+#pragma unroll
+        for (int c = 0; c < 8; c++) qf[c] = as_v8bf(*(const uint4*)(qrow + 16 * c + 8 * hl));
+    }
+    v16f o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.f;
+    float m_run = PF_M_FLOOR, l_run = 0.f;
+    const float sc = 1.4426950408889634f * 0.08838834764831845f;     // log2(e) / sqrt(128)
+
+    const int ch = tid & 15, kp = tid >> 4;
+    const uint32_t key_stride = (uint32_t)Hkv * 128;
+    const bf16_t* kbase = k_cache + (size_t)hk * 128 + ch * 8;        // row 0 of the cache
+    const bf16_t* vbase = v_cache + (size_t)hk * 128 + ch * 8;
+    uint4 rk[2][2], rv[2][2];
+    auto fetch_one = [&](int kb, int j) {
+        const int sb = j >> 2, i = (j >> 1) & 1;
+        const int key = kb + 32 * sb + 2 * kp + i;
+        const bool ok = key <= k_hi;
+        const uint32_t off = (uint32_t)key * key_stride;
+        if (j & 1) rv[sb][i] = ok ? *(const uint4*)(vbase + off) : make_uint4(0, 0, 0, 0);
+        else rk[sb][i] = ok ? *(const uint4*)(kbase + off) : make_uint4(0, 0, 0, 0);
+    };
+    auto fetch = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) fetch_one(kb, j);
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                *(uint4*)(lds_k + sb * PF_KBYTES + (2 * kp + i) * PF_KPITCH + ch * 16) = rk[sb][i];
+                *(uint4*)(lds_v + sb * PF_VBYTES + (2 * kp + i) * PF_VPITCH + ch * 16) = rv[sb][i];
+            }
+    };
+    const uint32_t vtr_off = (uint32_t)(4 * hl + ((lane & 15) >> 2)) * PF_VPITCH + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+    auto sub_block = [&](int kb, int sb, bool masked) {
+        v16f s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.f;
+        const uint8_t* kt = lds_k + sb * PF_KBYTES;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const v8bf kf = as_v8bf(*(const uint4*)(kt + col * PF_KPITCH + (16 * c + 8 * hl) * 2));
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], s, 0, 0, 0);
+        }
+        if (masked) {                      // wave-uniform: the chunk's first or last sub-block
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int key = kb + 8 * (r >> 2) + 4 * hl + (r & 3);
+                s[r] = (key >= k_lo && key <= k_hi) ? s[r] : PF_MASKED;
+            }
+        }
+        float mx = s[0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx * sc);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run + PF_LAZY) != 0) {      // wave-uniform
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= corr;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] *= corr;
+            m_run = m_new;
+        }
+        float psum = 0.f;
+        v8bf pf[2];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[r], sc, -m_run));
+            psum += p;
+            pf[r >> 3][r & 7] = (__bf16)p;
+        }
+        l_run += psum;
+#pragma unroll
+        for (int c2 = 0; c2 < 2; c2++)
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const lds_u8_t vblk = lds_v3 + sb * PF_VBYTES + vtr_off + 16 * c2 * PF_VPITCH + 32 * dt * 2;
+                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)vblk);
+                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)(vblk + 8 * PF_VPITCH));
+                const v8bf vf = __builtin_bit_cast(v8bf, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[c2], o[dt], 0, 0, 0);
+            }
+    };
+    auto visit = [&](int kb, int sb) {
+        if (kb <= k_hi && kb + 31 >= k_lo) sub_block(kb, sb, !(kb >= k_lo && kb + 31 <= k_hi));
+    };
+
+    fetch(kb_first);
+    for (int kb = kb_first; kb <= k_hi; kb += 64) {
+        __syncthreads();
+        stage();
+        __syncthreads();
+        if (kb + 64 <= k_hi) fetch(kb + 64);
+        if (KS == 1) {
+#pragma unroll 1
+            for (int sb = 0; sb < 2; sb++) visit(kb + 32 * sb, sb);
+        } else {
+            visit(kb + 32 * ks, ks);
+        }
+    }
+    if (KS == 2) {
+        __syncthreads();
+        float* xch = (float*)lds + (wave / (2 * GS) * GS + wave % GS) * (66 * 64);
+        if (ks == 1) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) xch[(16 * dt + r) * 64 + lane] = o[dt][r];
+            xch[64 * 64 + lane] = m_run;
+            xch[65 * 64 + lane] = l_run;
+        }
+        __syncthreads();
+        if (ks == 0) {
+            const float m2 = xch[64 * 64 + lane], l2 = xch[65 * 64 + lane];
+            const float m_new = fmaxf(m_run, m2);
+            const float wa = __builtin_amdgcn_exp2f(m_run - m_new), wb = __builtin_amdgcn_exp2f(m2 - m_new);
+            l_run = l_run * wa + l2 * wb;
+            m_run = m_new;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * wa + xch[(16 * dt + r) * 64 + lane] * wb;
+        }
+    }
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (q_ok && ks == 0) {
+        if (hl == 0) part[0] = m_run, part[1] = l_tot;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++)
+                *(float4*)(part + 4 + 32 * dt + 8 * g4 + 4 * hl) = make_float4(o[dt][4 * g4], o[dt][4 * g4 + 1], o[dt][4 * g4 + 2], o[dt][4 * g4 + 3]);
+    }
+}
+
+// keys per chunk and chunks of the shared part: chunks of at least 128 keys (two staging rounds), as many as give the launch about one
+// workgroup per CU
+void nc_attn_shared_plan(int rows, int H, int Hkv, int shared_len, int* chunk_keys_out, int* nchunks_out) {
+    const int G = H / Hkv;
+    const int GS = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1), KS = GS <= 2 ? 2 : 1, QT = 128 / (GS * KS);
+    const long per_chunk = (long)((rows + QT - 1) / QT) * Hkv * (G / GS);
+    int want = (int)((nc_cu_count() + per_chunk - 1) / per_chunk);
+    if (want < 1) want = 1;
+    int ck = (shared_len + want - 1) / want;
+    ck = (ck + 63) & ~63;
+    if (ck < 128) ck = 128;
+    *chunk_keys_out = ck;
+    *nchunks_out = (shared_len + ck - 1) / ck;
+}
+size_t nc_attn_shared_partial_bytes(int rows, int H, int Hkv, int shared_len) {
+    int ck, nc;
+    nc_attn_shared_plan(rows, H, Hkv, shared_len, &ck, &nc);
+    return (size_t)rows * H * nc * SP_PART_STRIDE * sizeof(float);
+}
+
+int nc_launch_attention_shared_prefix(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int shared_len,
+                                      int window_left, int seqlens_include_new, float* partials, size_t partial_bytes, int rows, int H, int Hkv,
+                                      int Tmax, int* nchunks_out, hipStream_t s) {
+    NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && partials, "shared_prefix_attention: null pointer");
+    NC_CHECK_ARG(rows > 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && shared_len > 0 && shared_len <= Tmax, "shared_prefix_attention: bad shape");
+    NC_CHECK_ARG((long long)Tmax * Hkv * 128 < (1LL << 31), "shared_prefix_attention: one row of the cache must stay below 2^31 elements");
+    NC_CHECK_ARG((((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)partials) & 15) == 0,
+                 "shared_prefix_attention: pointers must be 16-byte aligned");
+    int ck, nchunks;
+    nc_attn_shared_plan(rows, H, Hkv, shared_len, &ck, &nchunks);
+    NC_CHECK_ARG(partial_bytes >= (size_t)rows * H * nchunks * SP_PART_STRIDE * sizeof(float), "shared_prefix_attention: %zu bytes of partial sums needed",
+                 (size_t)rows * H * nchunks * SP_PART_STRIDE * sizeof(float));
+    const int G = H / Hkv;
+    const int GS = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1), KS = GS <= 2 ? 2 : 1, QT = 128 / (GS * KS);
+    const int nqtiles = (rows + QT - 1) / QT;
+    const dim3 grid(nqtiles * nchunks, Hkv * (G / GS));
+    NC_CHECK_ARG(grid.y <= 65535, "shared_prefix_attention: too many heads in one launch");
+    NcProfScope prof(0, 0.0, s);
+#define SP_LAUNCH(GG, KK)                                                                                                          \
+    hipLaunchKernelGGL((attn_shared_prefix_kernel<GG, KK>), grid, dim3(256), 0, s, q, k_cache, v_cache, cache_seqlens, shared_len,  \
+                       window_left, seqlens_include_new, partials, nchunks, ck, nqtiles, rows, H, Hkv, Tmax)
+    if (GS == 4) SP_LAUNCH(4, 1);
+    else if (GS == 2) SP_LAUNCH(2, 2);
+    else SP_LAUNCH(1, 2);
+#undef SP_LAUNCH
+    NC_CHECK_LAUNCH("shared_prefix_attention");
+    if (nchunks_out) *nchunks_out = nchunks;
+    return 0;
+}
+
 int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
                                 int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                                 uint32_t* amax_ws, hipStream_t s) {

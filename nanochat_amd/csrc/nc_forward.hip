@@ -40,6 +40,10 @@
         if (rc__) return rc__; \
     } while (0)
 
+// Reading a shared prompt once for all rows pays from a few rows on and for layers that see a long stretch of it
+#define NC_SHARED_MIN_ROWS 16
+#define NC_SHARED_MIN_KEYS 768
+
 namespace {
 struct Carver {
     uint8_t* base;
@@ -63,8 +67,8 @@ struct Workspace {
     // handle of amax site i (tagged: NC_AMAX_SLOTS words on separate lines, see amax_read / amax_publish)
     uint32_t* site(int i) const { return nc_amax_slotted(amax + (size_t)i * NC_AMAX_SLOTS * NC_AMAX_STRIDE); }
     int zero_words;
-    uint8_t *gemm_parts, *gemm_parts2, *attn_parts;
-    size_t gemm_part_bytes, attn_part_bytes;
+    uint8_t *gemm_parts, *gemm_parts2, *attn_parts, *shared_parts;
+    size_t gemm_part_bytes, attn_part_bytes, shared_part_bytes;
     size_t total;
 };
 
@@ -129,6 +133,10 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     w.gemm_parts2 = c.take<uint8_t>(fused_rows(m, (int)M) ? gneed : 0);
     w.attn_part_bytes = max_splits > 1 ? nc_attn_partial_bytes(B, T, m->n_head) / 16 * max_splits : 0;
     w.attn_parts = c.take<uint8_t>(w.attn_part_bytes);
+    // partial results of the shared first part of the cache (rows that begin with one replicated prompt): whatever the shared length
+    // turns out to be, the launch cuts it into at most as many chunks as a whole cache row would get
+    w.shared_part_bytes = (T == 1 && B >= NC_SHARED_MIN_ROWS) ? nc_attn_shared_partial_bytes(B, m->n_head, m->n_kv_head, 1 << 20) : 0;
+    w.shared_parts = c.take<uint8_t>(w.shared_part_bytes);
     w.total = (c.off + 255) & ~(size_t)255;
     return w;
 }
@@ -299,7 +307,29 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
         site++;
         bf16_t* kc = kv->k_cache + (size_t)i * layer_elems;
         bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
-        if (T == 1) {
+        // rows that begin with one replicated prompt: a layer that sees a long stretch of it reads that stretch once for all rows
+        bool shared_done = false;
+        if (T == 1 && B >= NC_SHARED_MIN_ROWS && kv->shared_prefix > 0 && kv->uniform_pos >= kv->shared_prefix && w.shared_parts) {
+            const int first_visible = ly.window_left < 0 ? 0 : (kv->uniform_pos - ly.window_left > 0 ? kv->uniform_pos - ly.window_left : 0);
+            if (kv->shared_prefix - first_visible >= NC_SHARED_MIN_KEYS && kv->shared_prefix < kv->max_seq_len) {
+                if (qsrc.parts)
+                    TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
+                                                    kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
+                else
+                    TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
+                                                  kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
+                int rc = nc_launch_attention_shared(w.qh, kc, vc, kv->cache_seqlens, kv->shared_prefix, ly.window_left, w.y, B, H, Hkv,
+                                                    kv->max_seq_len, 0, w.shared_parts, w.shared_part_bytes, w.site(site), s);
+                if (rc == -3)      // (the per-row kernel would split its keys: the plain entry, on the q and the cache rows just written)
+                    rc = nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
+                                             w.attn_counters, w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s);
+                if (rc) return rc;
+                shared_done = true;
+            }
+        }
+        if (shared_done) {
+            // (q, the new cache rows and the attention output are already written)
+        } else if (T == 1) {
             // decode: the attention workgroups finish their own q|k|v heads and append to the cache themselves
             const NcRopeSrc rope{qsrc.parts ? nullptr : w.qkv, qkv_w, qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin,
                                  m->rope_len, m->padded_vocab, nullptr, nullptr};

@@ -119,6 +119,15 @@ int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf
                                 int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                                 uint32_t* amax_ws, hipStream_t s);
 int nc_attn_splits(int B, int T, int Hkv, int window_left, int Tmax);
+// rows that share their first cached tokens (nc_attention_prefill.hip, nc_attention.hip)
+void nc_attn_shared_plan(int rows, int H, int Hkv, int shared_len, int* chunk_keys_out, int* nchunks_out);
+size_t nc_attn_shared_partial_bytes(int rows, int H, int Hkv, int shared_len);
+int nc_launch_attention_shared_prefix(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int shared_len,
+                                      int window_left, int seqlens_include_new, float* partials, size_t partial_bytes, int rows, int H, int Hkv,
+                                      int Tmax, int* nchunks_out, hipStream_t s);
+int nc_launch_attention_shared(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int shared_len,
+                               int window_left, bf16_t* out, int B, int H, int Hkv, int Tmax, int seqlens_include_new, void* shared_parts,
+                               size_t shared_part_bytes, uint32_t* amax_ws, hipStream_t s);
 void nc_attention_plan(int B, int T, int Hkv, int window_left, int Tmax, int force_splits, int* splits_out, int* heads_per_wg_out);
 int nc_launch_attention_append(const bf16_t* q, const bf16_t* k_new, const bf16_t* v_new, bf16_t* k_cache, bf16_t* v_cache,
                                const int32_t* cache_seqlens, int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax,

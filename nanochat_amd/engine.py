@@ -73,11 +73,17 @@ class KVCache:
     back every decode step; it is exact as long as positions change only through advance/reset/prefill
     (or set_seqlens for ragged batches, where it tracks row 0 like the reference's get_pos)."""
 
-    def __init__(self, batch_size, num_heads, seq_len, head_dim, num_layers, device, dtype, prefill_from=None):
+    def __init__(self, batch_size, num_heads, seq_len, head_dim, num_layers, device, dtype, prefill_from=None, share_prompt_reads=False):
         """prefill_from (not in the reference's signature): another cache whose tokens this one starts with, i.e.
         KVCache(...) followed by .prefill(prefill_from) in one step.  On the GPU the tensors then never get the zero fill that the
         copy would overwrite anyway (at d26 / 64 rows / 1792 prompt tokens that fill is 20 of the 22.7 GB, 4 ms of the time to the
-        first token): only the positions past the prompt are cleared, and the end state is the same."""
+        first token): only the positions past the prompt are cleared, and the end state is the same.
+
+        share_prompt_reads (not in the reference's signature, off by default): after a prefill from a batch-1 cache every row holds a
+        copy of the same prompt.  With this set the cache remembers how long that shared start is (`shared_prefix_len`) and a one-token
+        forward reads it once for all rows in the layers that see most of it, instead of once per row; the tensors keep the reference's
+        layout and contents.  The promise that goes with it: nobody writes into positions [0, shared_prefix_len) of k_cache / v_cache
+        by hand (set shared_prefix_len = 0 first)."""
         self.batch_size = batch_size
         self.max_seq_len = seq_len
         self.n_layers = num_layers
@@ -92,6 +98,8 @@ class KVCache:
         self.prev_embedding = None
         self._pos0 = 0          # host mirror of cache_seqlens[0]
         self._pos_max = 0       # host mirror of cache_seqlens.max()
+        self.share_prompt_reads = bool(share_prompt_reads)
+        self.shared_prefix_len = 0      # positions [0, this) hold the same bytes in every row (set by prefill from a batch-1 cache)
         if prefill_from is not None:
             if lazy:
                 n = prefill_from.get_pos()
@@ -104,6 +112,7 @@ class KVCache:
         self.cache_seqlens.zero_()
         self.prev_embedding = None
         self._pos0 = self._pos_max = 0
+        self.shared_prefix_len = 0
 
     def get_pos(self):
         return self._pos0
@@ -124,6 +133,8 @@ class KVCache:
         self._pos0 -= num_tokens
         self._pos_max -= num_tokens
         self.prev_embedding = prev_embedding
+        if self._pos0 < self.shared_prefix_len:         # the next append would land inside the shared start
+            self.shared_prefix_len = 0
 
     def set_seqlens(self, seqlens):
         """Ragged rows: install per-row lengths (host list or tensor)."""
@@ -132,6 +143,7 @@ class KVCache:
         self._pos0, self._pos_max = int(t[0]), int(t.max())
         assert 0 <= int(t.min()) and self._pos_max <= self.max_seq_len
         self.cache_seqlens.copy_(t)
+        self.shared_prefix_len = 0
 
     def prefill(self, other):
         """Copy another cache's first pos tokens into every row of this one (engine.py:123-137)."""
@@ -148,6 +160,7 @@ class KVCache:
             self.v_cache[:, :, :n, :, :] = other.v_cache[:, :, :n, :, :]
         self.cache_seqlens.fill_(n)
         self._pos0 = self._pos_max = n
+        self.shared_prefix_len = n if (other.batch_size == 1 and self.batch_size > 1) else 0
         if other.prev_embedding is not None:
             self.prev_embedding = other.prev_embedding.expand(self.batch_size, -1, -1).clone()
 
@@ -235,9 +248,12 @@ class Engine:
         return self.model.forward(ids, kv_cache=kv_cache)[:, -1, :]
 
     @torch.inference_mode()
-    def generate(self, tokens, num_samples=1, max_tokens=None, temperature=1.0, top_k=None, seed=42):
+    def generate(self, tokens, num_samples=1, max_tokens=None, temperature=1.0, top_k=None, seed=42, share_prompt_reads=False):
         """One batch-1 prefill, cache replicated to num_samples rows, then streamed decoding.
-        Yields (token_column, token_masks) per step (engine.py:175-275)."""
+        Yields (token_column, token_masks) per step (engine.py:175-275).
+
+        share_prompt_reads (not in the reference's signature, off by default): every row's cache starts with a copy of the same
+        prompt; with this set, the decode steps read that prompt once for all rows in the full-context layers (see KVCache)."""
         assert isinstance(tokens, list) and isinstance(tokens[0], int), "expecting list of ints"
         device = self.model.get_device()
         dtype = torch.bfloat16 if torch.device(device).type == "cuda" else COMPUTE_DTYPE
@@ -252,7 +268,8 @@ class Engine:
         logits = self._last_logits(ids, kv_prefill).expand(num_samples, -1)
 
         hint = (len(tokens) + max_tokens) if max_tokens is not None else cfg.sequence_len
-        kv_decode = KVCache(batch_size=num_samples, seq_len=hint, device=device, dtype=dtype, prefill_from=kv_prefill, **geometry)
+        kv_decode = KVCache(batch_size=num_samples, seq_len=hint, device=device, dtype=dtype, prefill_from=kv_prefill,
+                            share_prompt_reads=share_prompt_reads, **geometry)
         del kv_prefill
 
         rows = [RowState(tokens.copy()) for _ in range(num_samples)]

@@ -356,6 +356,12 @@ class GPT(nn.Module):
         cd.prev_in = prev_in.data_ptr() if prev_in is not None else None
         cd.prev_out = prev_out.data_ptr()
         cd.batch, cd.max_seq_len = B, kv_cache.max_seq_len
+        # rows that begin with one replicated prompt and sit at one position (what Engine.generate builds): the cache may ask for the
+        # shared start to be read once for all rows
+        pos0 = getattr(kv_cache, "_pos0", None)
+        shared = getattr(kv_cache, "shared_prefix_len", 0) if getattr(kv_cache, "share_prompt_reads", False) else 0
+        uniform = T == 1 and pos0 is not None and pos0 == pos_hi and shared > 0 and pos0 >= shared
+        cd.shared_prefix, cd.uniform_pos = (shared, pos0) if uniform else (0, 0)
         ws_ptr, ws_bytes = self._workspace(md, B, T, idx.device)
         if taps is None:
             rc = _lib.lib().nc_gpt_forward(C.byref(md), C.byref(cd), idx.data_ptr(), B, T, logits.data_ptr(), 1 if last_only else 0,

@@ -336,6 +336,35 @@ def decode_attention(q, k_cache, v_cache, cache_seqlens, window_left=-1, seqlens
     return out
 
 
+def decode_attention_shared(q, k_cache, v_cache, cache_seqlens, shared_len, window_left=-1, seqlens_include_new=False):
+    """decode_attention for a batch whose rows all begin with the same `shared_len` cached tokens and sit at the same position (one
+    prompt replicated by KVCache.prefill): the shared keys are read once for all rows, each row streams only its own tail."""
+    _need_cuda(q, k_cache, v_cache, cache_seqlens)
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise ValueError("decode_attention_shared: bf16 only")
+    if cache_seqlens.dtype != torch.int32:
+        raise ValueError("decode_attention_shared: cache_seqlens must be int32")
+    B, T, H, D = q.shape
+    Tmax, Hkv = k_cache.shape[1], k_cache.shape[2]
+    if T != 1 or D != 128 or k_cache.shape[-1] != 128:
+        raise ValueError("decode_attention_shared: one new token per row, head_dim 128")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("decode_attention_shared: caches must be contiguous (B,Tmax,Hkv,128)")
+    q = q.contiguous()
+    out = torch.empty_like(q)
+    lib = _lib.lib()
+    ws_bytes = lib.nc_decode_attention_shared_workspace_bytes(B, H, Hkv, int(shared_len))
+    key = (q.device.index, torch.cuda.current_stream().cuda_stream, "shared")
+    ws = _ATTN_WS.get(key)
+    if ws is None or ws.numel() < ws_bytes:
+        ws = torch.empty(max(ws_bytes, 1 << 20), dtype=torch.uint8, device=q.device)
+        _ATTN_WS[key] = ws
+    rc = lib.nc_decode_attention_shared(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cache_seqlens), int(shared_len), int(window_left), _ptr(out),
+                                        B, H, Hkv, Tmax, 1 if seqlens_include_new else 0, _ptr(ws), ws.numel(), C.c_void_p(0), _stream())
+    _lib.check(rc)
+    return out
+
+
 _ATTN_WS = {}
 
 

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_binding_and_error_channel():
     lib = _lib.lib()
-    assert lib.nc_abi_version() == 1
+    assert lib.nc_abi_version() == 2
     # argument validation happens before any GPU call, so it can be exercised without a device
     rc = lib.nc_fp8_quantize_tensorwise(None, 0, 16, None, None, None, None, 0, None)
     assert rc == -1 and b"null pointer" in lib.nc_last_error()
@@ -39,7 +39,7 @@ def test_struct_layout_matches_header():
     # pointer-sized fields + ints: sizes as a C compiler lays them out on LP64
     assert ctypes.sizeof(_lib.LayerDesc) == 10 * 8 + 2 * 4
     assert ctypes.sizeof(_lib.ModelDesc) == 8 * 4 + 2 * 4 + 11 * 8
-    assert ctypes.sizeof(_lib.CacheDesc) == 5 * 8 + 2 * 4
+    assert ctypes.sizeof(_lib.CacheDesc) == 5 * 8 + 4 * 4
 
 
 def test_library_was_built_from_these_sources():

@@ -705,6 +705,67 @@ def test_weight_changes_are_noticed_by_the_next_forward():
     assert torch.equal(logits(), doubled)
 
 
+def test_engine_generate_reading_the_shared_prompt_once():
+    """Engine.generate(share_prompt_reads=True): every row's cache starts with a copy of the one prompt, and the full-context layers
+    read that copy once for all rows.  On the repository init (attention contributes nothing to the logits there) the token stream is
+    that of the plain loop; on a trained-like model the logits of a decode step agree with the per-row path to the distance at which
+    the oracle's own two attention forms agree, and with the oracle."""
+    say("shared prompt: Engine.generate with share_prompt_reads")
+    from nanochat_amd.engine import Engine, KVCache
+    from test_engine_host import ByteTokenizer
+
+    class Tok(ByteTokenizer):
+        def __init__(self):
+            self._special = {"<|python_start|>": 2040, "<|python_end|>": 2041, "<|output_start|>": 2042,
+                             "<|output_end|>": 2043, "<|assistant_end|>": 2044, "<|bos|>": 2045}
+
+        def get_bos_token_id(self):
+            return 2045
+    # 64 rows x 8 kv heads: the per-row kernel runs unsplit, which the shared form needs; three of four layers are full-context
+    cfg = dict(sequence_len=2048, vocab_size=2048, n_layer=4, n_head=8, n_kv_head=8, n_embd=1024, window_pattern="LLSL")
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, 2000, (900,), generator=g).tolist()
+    rt, model = build_pair(cfg, seed=31, trained_like=False)
+    runs = []
+    for share in (False, True):
+        cols = [c for c, _ in Engine(model, Tok()).generate(prompt, num_samples=64, max_tokens=24, temperature=1.0, top_k=50, seed=7,
+                                                           share_prompt_reads=share)]
+        runs.append(cols)
+    assert runs[0] == runs[1] and len(runs[0]) == 24
+    # trained-like weights: one decode step, both ways, and the oracle on a few rows
+    rt, model = build_pair(cfg, seed=32, trained_like=True)
+    B, P = 64, 900
+    ids = torch.tensor([prompt])
+    pre = KVCache(1, 8, P, 128, 4, DEV, torch.bfloat16)
+    model.forward_last(ids.to(DEV), kv_cache=pre)
+    nxt = torch.randint(0, 2000, (B, 1), generator=g)
+    outs = {}
+    for share in (False, True):
+        dec = KVCache(B, 8, P + 8, 128, 4, DEV, torch.bfloat16, prefill_from=pre, share_prompt_reads=share)
+        assert dec.shared_prefix_len == P
+        a = model.forward_last(nxt.to(DEV), kv_cache=dec).cpu()
+        b = model.forward_last(nxt.roll(1, 0).to(DEV), kv_cache=dec).cpu()      # a second step: the rows' own tails now hold two tokens
+        outs[share] = torch.stack([a, b])
+    rows = [0, 13, 63]
+    ref = decode_ref.new_cache(rt.cfg, 1, P + 8, torch.bfloat16)
+    gpt_ref.forward(rt, ids, ref)
+    big = decode_ref.new_cache(rt.cfg, len(rows), P + 8, torch.bfloat16)
+    big.prefill(ref)
+    rt_def = gpt_ref.Runtime(rt.cfg, rt.p, compute_dtype=torch.bfloat16, fp8=True, uniform_sdpa=False)
+    big_def = decode_ref.new_cache(rt.cfg, len(rows), P + 8, torch.bfloat16)
+    big_def.prefill(ref)
+    want = torch.stack([gpt_ref.forward(rt, nxt[rows], big)[:, -1], gpt_ref.forward(rt, nxt.roll(1, 0)[rows], big)[:, -1]])
+    want_def = torch.stack([gpt_ref.forward(rt_def, nxt[rows], big_def)[:, -1], gpt_ref.forward(rt_def, nxt.roll(1, 0)[rows], big_def)[:, -1]])
+    floor_rel, floor_max = rel_l2(want_def, want), (want - want_def).abs().max().item()
+    # (the oracle quantizes with the amax of 3 rows, the GPU with that of 64: the floor criterion covers both differences)
+    print(f"shared prompt vs per-row path: rel_l2 {rel_l2(outs[True], outs[False]):.4f} max {(outs[True] - outs[False]).abs().max().item():.4f}")
+    assert_within_floor(outs[True][:, rows], want, want_def, max(floor_rel, rel_l2(outs[False][:, rows], want)), floor_max, "shared-prompt decode")
+    assert rel_l2(outs[True], outs[False]) <= 1.5 * max(floor_rel, rel_l2(outs[False][:, rows], want)) + 1e-3
+    # (the two paths sum in different orders and the shared part's weights pass through bf16: equal bits would mean that the
+    # shared form had not run at all)
+    assert not torch.equal(outs[True], outs[False]), "the shared-prompt path was meant to run for this shape"
+
+
 @pytest.mark.parametrize("B", [4, 1])
 def test_decode_step_captured_in_a_graph_replays_like_the_eager_step(B):
     """The decode forward makes no allocation of its own, clears its counters with a kernel and reads positions from device memory,

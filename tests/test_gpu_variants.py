@@ -189,6 +189,50 @@ def test_decode_attention_headline_launch_against_the_oracle(ops, window):
     assert ulp_k <= 2 and ulp_v <= 1 and frac_k < 0.01 and frac_v < 0.01, (frac_k, ulp_k, frac_v, ulp_v)
 
 
+# (B, H, Hkv, Tmax, shared, pos, window)
+SHARED_SHAPES = [
+    (64, 13, 13, 2048, 1792, 1920, -1),      # the headline batch in a full-context layer, mid-run
+    (64, 13, 13, 2048, 1792, 2047, -1),      # ... at its last step
+    (64, 13, 13, 2048, 1792, 1792, -1),      # ... at its first decode step: the row's own tail is its new token alone
+    (64, 13, 13, 2048, 1792, 2000, 512),     # a window layer: the window reaches 304 keys into the shared part
+    (64, 13, 13, 2048, 1792, 2047, 200),     # the window no longer reaches the shared part at all
+    (128, 16, 4, 1024, 700, 830, -1),        # four query heads per kv head (the d32 width), a shared length that is no multiple of 64
+    (96, 12, 6, 512, 130, 140, -1),          # two query heads per kv head, one chunk
+    (70, 8, 8, 640, 600, 601, 300),          # rows that do not fill the last block of 32
+]
+
+
+@pytest.mark.parametrize("B,H,Hkv,Tmax,shared,pos,window", SHARED_SHAPES)
+def test_decode_attention_with_a_shared_prompt_against_the_oracle(ops, B, H, Hkv, Tmax, shared, pos, window):
+    """Rows whose first `shared` cached tokens are one prompt replicated to every row (Engine.generate): the shared keys are read once
+    for all rows on the matrix cores, each row streams its own tail, and the two parts of the softmax are merged.  Against the CPU
+    oracle on rows 0, 1, B/2 and B-1 (whole caches, nothing shared there), and against the per-row kernel on every row."""
+    say(f"decode attention with a shared prompt: B={B} H={H} Hkv={Hkv} Tmax={Tmax} shared={shared} pos={pos} window={window}")
+    g = torch.Generator(device=DEV).manual_seed(shared + pos)
+    kd = torch.randn(B, Tmax, Hkv, 128, device=DEV, generator=g).bfloat16()
+    vd = torch.randn(B, Tmax, Hkv, 128, device=DEV, generator=g).bfloat16()
+    kd[:, :shared] = kd[0:1, :shared]                      # what KVCache.prefill leaves: every row holds the prompt's keys and values
+    vd[:, :shared] = vd[0:1, :shared]
+    kd[:, pos + 1:] = float("nan")                         # nothing past the new token may be read
+    vd[:, pos + 1:] = float("nan")
+    qd = (torch.randn(B, 1, H, 128, device=DEV, generator=g) * 1.5).bfloat16()
+    seq = torch.full((B,), pos, dtype=torch.int32, device=DEV)
+    got = ops.decode_attention_shared(qd, kd, vd, seq, shared, window_left=window)
+    assert torch.isfinite(got.float()).all()
+    plain = ops.decode_attention(qd, kd, vd, seq, window_left=window)
+    d_plain = (got.float() - plain.float()).abs().max().item()
+    rows = sorted({0, 1, B // 2, B - 1})
+    # the oracle appends nothing here (the new token is in the cache): it reads keys [lo, pos] of each row
+    kc, vc = kd[rows].cpu(), vd[rows].cpu()
+    kc[:, pos + 1:] = 0
+    vc[:, pos + 1:] = 0
+    want = attention_with_kvcache(qd[rows].cpu(), kc, vc, kc[:, pos:pos + 1].clone(), vc[:, pos:pos + 1].clone(), seq[rows].cpu(), (window, 0))
+    d_oracle = (got[rows].cpu().float() - want.float()).abs().max().item()
+    print(f"shared-prompt attention: max |d| vs the per-row kernel {d_plain:.5f}, vs the oracle {d_oracle:.5f}")
+    assert torch.allclose(got[rows].cpu().float(), want.float(), atol=1e-2, rtol=1e-2), d_oracle
+    assert torch.allclose(got.float(), plain.float(), atol=1e-2, rtol=1e-2), d_plain
+
+
 @pytest.mark.parametrize("splits", [0, 1, 2, 4, 16])
 @pytest.mark.parametrize("H,Hkv", [(4, 2), (13, 13)])
 def test_decode_attention_in_kernel_append_with_key_splits(ops, splits, H, Hkv):
