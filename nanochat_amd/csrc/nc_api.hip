@@ -110,8 +110,12 @@ int nc_fp8_linear_small_m(const uint16_t* a_bf16, const uint32_t* a_amax, const 
     if (int rc = segs_from(seg_ends, nseg, N, &segs)) return rc;
     NC_CHECK_ARG(out && inv_b, "fp8_linear_small_m: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    int ks = ksplits > 0 ? ksplits : nc_gemm_decode_splits(N, K);
-    if (ksplits <= 0 && ks > 1 && (!workspace || workspace_bytes < (size_t)ks * M * N * sizeof(float))) ks = 1;
+    // left to choose (ksplits <= 0), the launch picks the form; without room for the partial sums it would need, one split
+    int ks = ksplits > 0 ? ksplits : 0;
+    if (ksplits <= 0) {
+        const int want = nc_gemm_decode_splits(N, K);
+        if (want > 1 && (!workspace || workspace_bytes < (size_t)want * M * N * sizeof(float))) ks = 1;
+    }
     int used = 1;
     if (int rc = nc_launch_gemm_decode(a_bf16, 1, a_amax, nullptr, b, inv_b, segs, out, out_kind, softcap, out_amax, M, N, K, ldc,
                                        (float*)workspace, workspace_bytes, ks, &used, s))

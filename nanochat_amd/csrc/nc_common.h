@@ -256,7 +256,10 @@ __device__ __forceinline__ float amax_from_lanes(uint32_t loaded) {
 // so the words can be asked for first and looked at last without the compiler having to count vector loads in between.
 struct AmaxWords { uint32_t w[NC_AMAX_SLOTS]; };
 __device__ __forceinline__ AmaxWords amax_load_scalar(const uint32_t* h) {
-    const uint32_t* p = (const uint32_t*)((uintptr_t)h & ~(uintptr_t)3);
+    // (the constant address space is what makes these scalar loads: a generic pointer built from an integer gets flat loads, which
+    // count against both counters and force the vector loads around them to drain)
+    typedef const __attribute__((address_space(4))) uint32_t* cptr;
+    cptr p = (cptr)((uintptr_t)h & ~(uintptr_t)3);
     const int stride = ((uintptr_t)h & 1u) ? NC_AMAX_STRIDE : 0;
     AmaxWords a;
 #pragma unroll

@@ -11,10 +11,20 @@
 // separate convert pass of the quantizer disappears.
 //
 // A dependent trip to memory costs a couple of microseconds here, which is more than the arithmetic of one of
-// these GEMMs, so the kernel is built to make exactly one: all loads of a workgroup's K range are issued
-// at once, and with split-K the raw fp32 partial tiles are simply stored ([split][M][N]) -- the kernel that
-// consumes the linear's output (residual/norm, rotary/append, or nc_finish_partials) adds the splits in a
-// fixed order, applies inv_a * inv_w and rounds to bf16 while it reads them, which it had to read anyway.
+// these GEMMs, so the kernels are built to make as few as they can, and with split-K the raw fp32 partial tiles
+// are simply stored ([split][M][N]) -- the kernel that consumes the linear's output (residual/norm,
+// rotary/append, or nc_finish_partials) adds the splits in a fixed order, applies inv_a * inv_w and rounds to
+// bf16 while it reads them, which it had to read anyway.  Three forms:
+//   gemm_decode_onetrip_kernel  a K range of at most 8 steps per workgroup (every split linear of a decode step):
+//                               the whole range asked for through buffer descriptors before the first wait
+//                               (9.0 / 6.7 / 9.9 / 9.7 us -> 8.2 / 5.0 / 8.3 / 8.5 us for the four linears of a
+//                               d26 layer at 64 rows; about 3.4 us of each is the weight fetch itself, 2.3 us the
+//                               launch, 1.5 us the partial sums leaving the chip);
+//   gemm_decode_full_kernel     17 .. 64 rows, K <= 2048, relu^2 epilogue: unsplit, 32 columns per workgroup,
+//                               the result leaves finished and the MLP activation needs no pass of its own
+//                               (10.6 us against 8.3 + 4.4 us for the split linear and its finishing pass);
+//   gemm_decode_kernel          everything else (longer K ranges walked in 512-wide chunks, more than 64 rows,
+//                               activation rows made inside the kernel from a recipe).
 //
 // Epilogues: 0 bf16;  1 fp32 softcap*tanh(bf16(v)/softcap) (lm_head, nanochat/gpt.py:512-515);
 //            2 bf16 relu(bf16(v))^2 plus atomic amax of the result (MLP activation, gpt.py:139).
@@ -414,6 +424,381 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// The same work when a workgroup's K range is at most 8 steps (every split linear of a decode step): one trip to memory.  All loads
+// go through buffer descriptors, whose range check returns zeros for rows past M / N and for whatever lies beyond the K range, so no
+// load sits under a branch and the whole range -- activation rows first (they come from the L2 and are converted into LDS while the
+// weight rows are still on their way), then the weight rows -- is asked for before anything is waited for.  The tensorwise amax comes
+// through the scalar cache, which has a counter of its own.
+#define NC_DG_OOB 0x80000000u
+typedef int dg_v4i __attribute__((ext_vector_type(4)));
+template <int MB, bool A_BF16, int NSET>
+__global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs g) {
+    constexpr int ROWS = MB * 16;
+    constexpr int A_CH = ROWS * 32 / 256;          // 16-byte e4m3 chunks per thread per 512-wide half of the range
+    constexpr int A_LD = A_BF16 ? 2 : 1;
+    __shared__ __align__(16) uint8_t lds[NSET][ROWS * 512];
+    __shared__ float red[4];
+
+    NC_ARG_NOW(g.A); NC_ARG_NOW(g.a_amax); NC_ARG_NOW(g.inv_a); NC_ARG_NOW(g.B); NC_ARG_NOW(g.partial_out); NC_ARG_NOW(g.ksplits);
+    NC_ARG_NOW(g.ksteps_per_split); NC_ARG_NOW(g.M); NC_ARG_NOW(g.N); NC_ARG_NOW(g.K);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int frow = lane & 15, kb = lane >> 4;
+    const int split = blockIdx.y;
+    const int M = g.M, N = g.N, K = g.K;
+    const int n0 = blockIdx.x * 64 + wave * 16;
+    const int brow = n0 + frow;
+
+    const int nksteps = (K + 127) >> 7;
+    const int ks_begin = split * g.ksteps_per_split;
+    int ks_end = ks_begin + g.ksteps_per_split;
+    if (ks_end > nksteps) ks_end = nksteps;
+    const int nk = ks_end - ks_begin;                              // 1 .. 4 * NSET
+    const int kbase = ks_begin << 7;
+    const int k_hi = (ks_end << 7) < K ? (ks_end << 7) : K;       // exclusive K bound of this split
+
+    AmaxWords aw = {};
+    float inv_a = 0.f;
+    if (A_BF16) aw = amax_load_scalar(g.a_amax);
+    else inv_a = *g.inv_a;
+
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, M * K * (A_BF16 ? 2 : 1), 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, N * K, 0x00020000);
+
+    // (measured: handing the conversion to waves of their own, so that the weight requests go out first, is slower, 9.9 against
+    // 8.3 us at N = 6656, K = 1664)
+    dg_v4i ra[NSET][A_CH][A_LD], rb[NSET][4][2];
+#pragma unroll
+    for (int set = 0; set < NSET; set++)
+#pragma unroll
+        for (int c = 0; c < A_CH; c++) {
+            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+            const int gk = kbase + set * 512 + ch * 16;
+            const uint32_t vo = (row < M && gk < k_hi) ? ((uint32_t)row * (uint32_t)K + (uint32_t)gk) * (A_BF16 ? 2u : 1u) : NC_DG_OOB;
+#pragma unroll
+            for (int h = 0; h < A_LD; h++) ra[set][c][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, vo, h * 16, 0);
+        }
+#pragma unroll
+    for (int set = 0; set < NSET; set++)
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const int gk = kbase + set * 512 + kk * 128 + kb * 32;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint32_t vo = (brow < N && gk + h * 16 < k_hi) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
+                rb[set][kk][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 16, 0);
+            }
+        }
+
+    float scale = 1.f;
+    if (A_BF16) {
+        scale = scale_from_amax(amax_from_words(aw));
+        inv_a = 1.0f / scale;
+    }
+#pragma unroll
+    for (int set = 0; set < NSET; set++)
+#pragma unroll
+        for (int c = 0; c < A_CH; c++) {
+            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+            dg_v4i v;
+            if (A_BF16) {
+                const uint32_t w[8] = {(uint32_t)ra[set][c][0][0], (uint32_t)ra[set][c][0][1], (uint32_t)ra[set][c][0][2], (uint32_t)ra[set][c][0][3],
+                                       (uint32_t)ra[set][c][A_LD - 1][0], (uint32_t)ra[set][c][A_LD - 1][1], (uint32_t)ra[set][c][A_LD - 1][2],
+                                       (uint32_t)ra[set][c][A_LD - 1][3]};
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    // no clamp needed: |x| <= amax gives |x*scale| <= 448*(1+2^-23), which rounds to 448 like the clamped value
+                    v[j] = (int)e4m3_pack4_hw(bf16_lo(w[2 * j]) * scale, bf16_hi(w[2 * j]) * scale, bf16_lo(w[2 * j + 1]) * scale,
+                                              bf16_hi(w[2 * j + 1]) * scale);
+            } else {
+                v = ra[set][c][0];
+            }
+            *(dg_v4i*)(&lds[set][row * 512 + ((ch ^ (row & 15)) << 4)]) = v;
+        }
+    __syncthreads();
+
+    v4f acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+    // K-steps in pairs; the steps past the range hold zeros on both sides, so only whole pairs are skipped
+#pragma unroll
+    for (int pr = 0; pr < 2 * NSET; pr++) {
+        if (2 * pr < nk) {
+            dg_v4i alo[2][MB], ahi[2][MB];
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const int kk = (2 * pr + q) & 3;
+#pragma unroll
+                for (int i = 0; i < MB; i++) {
+                    const int row = i * 16 + frow;
+                    const int c0 = kk * 8 + 2 * kb;
+                    alo[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + ((c0 ^ (row & 15)) << 4)]);
+                    ahi[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + (((c0 + 1) ^ (row & 15)) << 4)]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const int kk = (2 * pr + q) & 3;
+                const dg_v4i lo = rb[pr >> 1][kk][0], hi = rb[pr >> 1][kk][1];
+                v8i bf;
+                bf[0] = lo[0], bf[1] = lo[1], bf[2] = lo[2], bf[3] = lo[3], bf[4] = hi[0], bf[5] = hi[1], bf[6] = hi[2], bf[7] = hi[3];
+#pragma unroll
+                for (int i = 0; i < MB; i++) {
+                    v8i af;
+                    af[0] = alo[q][i][0], af[1] = alo[q][i][1], af[2] = alo[q][i][2], af[3] = alo[q][i][3];
+                    af[4] = ahi[q][i][0], af[5] = ahi[q][i][1], af[6] = ahi[q][i][2], af[7] = ahi[q][i][3];
+                    acc[i] = MFMA_F8(acc[i], bf, af);
+                }
+            }
+        }
+    }
+
+    const int n = n0 + 4 * kb;
+    if (g.ksplits > 1) {
+        // split-K: the raw partial tile; the consumer adds the splits
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const int m = i * 16 + frow;
+            if (m < M && n < N)
+                *(float4*)(g.partial_out + ((size_t)split * M + m) * N + n) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+        }
+        return;
+    }
+    // one split (K <= 1024): the epilogue of gemm_decode_kernel
+    float am = 0.f;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+        const int m = i * 16 + frow;
+        if (m < M && n < N) {
+            const float inv_b = dg_seg_scale(g, n);
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] = (acc[i][r] * inv_a) * inv_b;
+            if (g.out_kind == 1) {
+                float* o = (float*)g.out + (size_t)m * g.ldc + n;
+                for (int r = 0; r < 4 && n + r < N; r++) o[r] = g.softcap * tanhf(rbf(v[r]) / g.softcap);
+            } else {
+                if (g.out_kind == 2) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const float t = relu_keep_nan(rbf(v[r]));
+                        v[r] = rbf(t * t);
+                        if (n + r < N) am = amax_join(am, v[r]);
+                    }
+                }
+                bf16_t* o = (bf16_t*)g.out + (size_t)m * g.ldc + n;
+                if (n + 3 < N) *(uint2*)o = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                else
+                    for (int r = 0; r < 4 && n + r < N; r++) o[r] = f32_to_bf16(v[r]);
+            }
+        }
+    }
+    if (g.out_kind == 2 && g.out_amax) {
+        am = wave_amax(am);
+        if (lane == 0) red[wave] = am;
+        __syncthreads();
+        if (tid == 0) {
+            am = amax_join(amax_join(red[0], red[1]), amax_join(red[2], red[3]));
+            amax_publish(g.out_amax, am);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Unsplit form for 17 .. 64 rows and K <= 2048 (the q|k|v and c_fc linears of a decode step): a workgroup of 8 waves owns 32 output
+// columns over the whole of K, so the result leaves the kernel finished (bf16, relu^2 and its amax included) instead of as fp32
+// partial sums that cost more to write and to read back than the weights did, and the MLP activation needs no pass of its own.
+// The whole activation panel is converted into LDS once per workgroup ([K-step][64 rows][128 bytes] tiles); wave (cb, rh, kh) then
+// multiplies rows 32*rh .. +31 with columns 16*cb .. +15 over half of the K-steps, and the two K halves meet through LDS.
+// Still one trip to memory: activation rows first, then the weight rows, everything asked for before the first wait.
+#define NC_DGF_MAX_K 2048
+template <bool A_BF16, int NKS>
+__global__ __launch_bounds__(1024) void gemm_decode_full_kernel(DecodeGemmArgs g) {
+    constexpr int A_LD = A_BF16 ? 2 : 1;
+    constexpr int NKQ = (NKS + 3) / 4;              // K-steps per quarter
+    extern __shared__ __align__(16) uint8_t dgf_lds[];            // NKS tiles of 8 KB, then 6 x 4 KB for the meeting of the quarters
+    float* const meet = (float*)(dgf_lds + NKS * 8192);
+    __shared__ float red[2];
+
+    NC_ARG_NOW(g.A); NC_ARG_NOW(g.a_amax); NC_ARG_NOW(g.inv_a); NC_ARG_NOW(g.B); NC_ARG_NOW(g.inv_b); NC_ARG_NOW(g.out); NC_ARG_NOW(g.out_kind);
+    NC_ARG_NOW(g.out_amax); NC_ARG_NOW(g.ldc); NC_ARG_NOW(g.M); NC_ARG_NOW(g.N); NC_ARG_NOW(g.K);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int M = g.M, N = g.N, K = g.K;
+    const int nksteps = (K + 127) >> 7;                            // <= NKS
+
+    AmaxWords aw = {};
+    float inv_a = 0.f;
+    if (A_BF16) aw = amax_load_scalar(g.a_amax);
+    else inv_a = *g.inv_a;
+
+    if (wave >= 8) {
+        // ---- the converting waves: thread t converts chunk (row t >> 3, 16-byte piece t & 7) of every K-step tile.  Their loads
+        // come from the L2; they are asked for after the scale is known, which lets the weight requests of the other waves, the
+        // long trip, through the address units first.
+        float scale = 1.f;
+        if (A_BF16) {
+            scale = scale_from_amax(amax_from_words(aw));
+            asm volatile("" : "+v"(scale));
+        }
+        const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, M * K * (A_BF16 ? 2 : 1), 0x00020000);
+        const int ct = tid - 512;
+        const int arow = ct >> 3, ach = ct & 7;
+        dg_v4i ra[NKS][A_LD];
+#pragma unroll
+        for (int j = 0; j < NKS; j++) {
+            const int gk = j * 128 + ach * 16;
+            const uint32_t vo = (arow < M && gk < K) ? ((uint32_t)arow * (uint32_t)K + (uint32_t)gk) * (A_BF16 ? 2u : 1u) : NC_DG_OOB;
+#pragma unroll
+            for (int h = 0; h < A_LD; h++) ra[j][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, vo, h * 16, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < NKS; j++) {
+            dg_v4i v;
+            if (A_BF16) {
+                const uint32_t w[8] = {(uint32_t)ra[j][0][0], (uint32_t)ra[j][0][1], (uint32_t)ra[j][0][2], (uint32_t)ra[j][0][3],
+                                       (uint32_t)ra[j][A_LD - 1][0], (uint32_t)ra[j][A_LD - 1][1], (uint32_t)ra[j][A_LD - 1][2],
+                                       (uint32_t)ra[j][A_LD - 1][3]};
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    // no clamp needed: |x| <= amax gives |x*scale| <= 448*(1+2^-23), which rounds to 448 like the clamped value
+                    v[q] = (int)e4m3_pack4_hw(bf16_lo(w[2 * q]) * scale, bf16_hi(w[2 * q]) * scale, bf16_lo(w[2 * q + 1]) * scale,
+                                              bf16_hi(w[2 * q + 1]) * scale);
+            } else {
+                v = ra[j][0];
+            }
+            if (j < nksteps) *(dg_v4i*)(&dgf_lds[j * 8192 + arow * 128 + ((ach ^ (arow & 7)) << 4)]) = v;
+        }
+        __syncthreads();                  // the panel is complete
+        __syncthreads();                  // (the meeting of the K quarters)
+        if (g.out_kind == 2 && g.out_amax) __syncthreads();
+        return;
+    }
+
+    // ---- the multiplying waves: wave (cb, kq) asks for its weight rows at once and waits for the panel
+    const int frow = lane & 15, kb = lane >> 4;
+    const int cb = wave & 1, kq = wave >> 1;
+    const int n0 = blockIdx.x * 32 + cb * 16;
+    const int brow = n0 + frow;
+    const int nq = (nksteps + 3) >> 2;                             // K-steps [kq * nq, (kq + 1) * nq) belong to quarter kq
+    const int ks0 = kq * nq;
+    const int nk = ks0 + nq <= nksteps ? nq : (nksteps > ks0 ? nksteps - ks0 : 0);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, N * K, 0x00020000);
+    dg_v4i rb[NKQ][2];
+#pragma unroll
+    for (int j = 0; j < NKQ; j++) {
+        const int gk = (ks0 + j) * 128 + kb * 32;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t vo = (brow < N && j < nk && gk + h * 16 < K) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
+            rb[j][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 16, 0);
+        }
+    }
+    if (A_BF16) inv_a = 1.0f / scale_from_amax(amax_from_words(aw));
+    __syncthreads();
+
+    v4f acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < NKQ; j++) {
+        if (j < nk) {
+            const uint8_t* tile = dgf_lds + (ks0 + j) * 8192;
+            v8i bf;
+            bf[0] = rb[j][0][0], bf[1] = rb[j][0][1], bf[2] = rb[j][0][2], bf[3] = rb[j][0][3];
+            bf[4] = rb[j][1][0], bf[5] = rb[j][1][1], bf[6] = rb[j][1][2], bf[7] = rb[j][1][3];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = i * 16 + frow;
+                const dg_v4i alo = *(const dg_v4i*)(tile + row * 128 + (((2 * kb) ^ (row & 7)) << 4));
+                const dg_v4i ahi = *(const dg_v4i*)(tile + row * 128 + (((2 * kb + 1) ^ (row & 7)) << 4));
+                v8i af;
+                af[0] = alo[0], af[1] = alo[1], af[2] = alo[2], af[3] = alo[3], af[4] = ahi[0], af[5] = ahi[1], af[6] = ahi[2], af[7] = ahi[3];
+                acc[i] = MFMA_F8(acc[i], bf, af);
+            }
+        }
+    }
+
+    // the later K quarters hand their sums to the first one (always added in the order 1, 2, 3)
+    if (kq) {
+        float* mp = meet + (((kq - 1) * 2 + cb) * 64 + lane) * 16;
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(float4*)(mp + 4 * i) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+    }
+    __syncthreads();
+    float am = 0.f;
+    if (!kq) {
+#pragma unroll
+        for (int q = 0; q < 3; q++) {
+            const float* mp = meet + ((q * 2 + cb) * 64 + lane) * 16;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float4 u = *(const float4*)(mp + 4 * i);
+                acc[i][0] += u.x, acc[i][1] += u.y, acc[i][2] += u.z, acc[i][3] += u.w;
+            }
+        }
+        // lane holds rows 16*i + frow, columns n0 + 4*kb .. +3
+        const int n = n0 + 4 * kb;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int m = i * 16 + frow;
+            if (m < M && n < N) {
+                const float inv_b = dg_seg_scale(g, n);
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] = (acc[i][r] * inv_a) * inv_b;
+                if (g.out_kind == 1) {
+                    float* o = (float*)g.out + (size_t)m * g.ldc + n;
+                    for (int r = 0; r < 4 && n + r < N; r++) o[r] = g.softcap * tanhf(rbf(v[r]) / g.softcap);
+                } else {
+                    if (g.out_kind == 2) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const float t = relu_keep_nan(rbf(v[r]));
+                            v[r] = rbf(t * t);
+                            if (n + r < N) am = amax_join(am, v[r]);
+                        }
+                    }
+                    bf16_t* o = (bf16_t*)g.out + (size_t)m * g.ldc + n;
+                    if (n + 3 < N) *(uint2*)o = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                    else
+                        for (int r = 0; r < 4 && n + r < N; r++) o[r] = f32_to_bf16(v[r]);
+                }
+            }
+        }
+    }
+    if (g.out_kind == 2 && g.out_amax) {
+        am = wave_amax(am);
+        if (!kq && lane == 0) red[cb] = am;
+        __syncthreads();
+        if (tid == 0) amax_publish(g.out_amax, amax_join(red[0], red[1]));
+    }
+}
+
+namespace {
+template <bool A_BF16, int NKS>
+int launch_full(const DecodeGemmArgs& g, int nblk32, hipStream_t s) {
+    static bool reserved[64];
+    constexpr int lds_bytes = NKS * 8192 + 6 * 4096;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev < 0 || dev >= 64 || !reserved[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)gemm_decode_full_kernel<A_BF16, NKS>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm(decode): cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+        if (dev >= 0 && dev < 64) reserved[dev] = true;
+    }
+    hipLaunchKernelGGL((gemm_decode_full_kernel<A_BF16, NKS>), dim3(nblk32), dim3(1024), lds_bytes, s, g);
+    return 0;
+}
+}  // namespace
+
+// Whether nc_launch_gemm_decode, left to choose (ksplits 0), runs the unsplit form: enough 32-column blocks to occupy half the chip
+// and few enough to run in one round.
+static bool dg_full_form(int M, int N, int K, bool made, int out_kind) {
+    const int nblk32 = (N + 31) / 32;
+    return out_kind == 2 && !made && M > 16 && M <= 64 && K <= NC_DGF_MAX_K && nblk32 >= 128 && nblk32 <= 256 && (int64_t)N * K < ((int64_t)1 << 31);
+}
+
+// ------------------------------------------------------------------------------------------------
 // out = epilogue((sum over splits of partials) * inv_a * inv_w[segment]) -- the finishing pass for callers that
 // need the linear's output materialised (the MLP activation, and the stand-alone API).
 __global__ __launch_bounds__(256) void finish_partials_kernel(const float* __restrict__ parts, int nsplit, size_t split_stride,
@@ -545,6 +930,8 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     NC_CHECK_ARG(K % 16 == 0, "fp8_gemm: K=%d must be a multiple of 16", K);
     NC_CHECK_ARG(((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0, "fp8_gemm: operands must be 16-byte aligned");
     const int nksteps = (K + 127) / 128;
+    const bool full = ksplits <= 0 && dg_full_form(M, N, K, made, out_kind);
+    if (full) ksplits = 1;
     if (ksplits <= 0) ksplits = nc_gemm_decode_splits(N, K);
     NC_CHECK_ARG(ksplits <= 16, "fp8_gemm(decode): at most 16 K splits, got %d", ksplits);
     if (ksplits > nksteps) ksplits = nksteps;
@@ -576,8 +963,38 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
     g.recipe = made ? *recipe : NcRowRecipe{};
     NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
+    if (full) {
+        const int nblk32 = (N + 31) / 32;
+        int rc;
+        if (nksteps <= 10) rc = a_is_bf16 ? launch_full<true, 10>(g, nblk32, s) : launch_full<false, 10>(g, nblk32, s);
+        else if (nksteps <= 13) rc = a_is_bf16 ? launch_full<true, 13>(g, nblk32, s) : launch_full<false, 13>(g, nblk32, s);
+        else rc = a_is_bf16 ? launch_full<true, 16>(g, nblk32, s) : launch_full<false, 16>(g, nblk32, s);
+        if (rc) return rc;
+        NC_CHECK_LAUNCH("fp8_gemm(decode)");
+        return 0;
+    }
     dim3 grid(nblk, ksplits), block(256);
-    if (MB == 1) {
+    const bool onetrip = !made && MB <= 4 && kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
+#define OT_LAUNCH(MB_, AB_)                                                                                            \
+    do {                                                                                                               \
+        if (kps <= 4) hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, AB_, 1>), grid, block, 0, s, g);             \
+        else hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, AB_, 2>), grid, block, 0, s, g);                     \
+    } while (0)
+    if (onetrip) {
+        if (MB == 1) {
+            if (a_is_bf16) OT_LAUNCH(1, true);
+            else OT_LAUNCH(1, false);
+        } else if (MB == 2) {
+            if (a_is_bf16) OT_LAUNCH(2, true);
+            else OT_LAUNCH(2, false);
+        } else if (MB == 3) {
+            if (a_is_bf16) OT_LAUNCH(3, true);
+            else OT_LAUNCH(3, false);
+        } else {
+            if (a_is_bf16) OT_LAUNCH(4, true);
+            else OT_LAUNCH(4, false);
+        }
+    } else if (MB == 1) {
         if (made && recipe->kind == 1) hipLaunchKernelGGL((gemm_decode_kernel<1, 2>), grid, block, 0, s, g);
         else if (made) hipLaunchKernelGGL((gemm_decode_kernel<1, 3>), grid, block, 0, s, g);
         else if (a_is_bf16) hipLaunchKernelGGL((gemm_decode_kernel<1, 1>), grid, block, 0, s, g);

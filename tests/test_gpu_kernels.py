@@ -357,7 +357,10 @@ def test_gemm_softcap_epilogue(ops):
 @pytest.mark.parametrize("M,N,K,ksplits", [(64, 1664, 1664, 0), (64, 4992, 1664, 0), (64, 6656, 1664, 0), (64, 1664, 6656, 0),
                                            (64, 32768, 1664, 0), (64, 1664, 1664, 1), (64, 1664, 1664, 13), (64, 1664, 6656, 5),
                                            (8, 256, 1024, 0), (1, 1024, 256, 2), (100, 2048, 2048, 0), (128, 512, 8192, 7),
-                                           (37, 208, 400, 3)])
+                                           (37, 208, 400, 3),
+                                           # the unsplit form (17 .. 64 rows, K <= 2048, 128 .. 256 blocks of 32 columns), ragged edges included
+                                           (33, 6656, 1664, 0), (64, 4096, 1280, 0), (48, 8192, 2048, 0), (17, 4100, 1664, 0),
+                                           (64, 5000, 1040, 0)])
 def test_fused_small_m_linear(ops, M, N, K, ksplits):
     """Quantize-inside-the-GEMM decode linear: same bytes as quantize + GEMM, whatever the K split."""
     say(f"fused small-M linear M={M} N={N} K={K} ksplits={ksplits}")
