@@ -481,11 +481,13 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
     for (int set = 0; set < NSET; set++)
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
-            const int gk = kbase + set * 512 + kk * 128 + kb * 32;
+            // a lane's 32 K-bytes of a step are pieces kb and 4 + kb of its 128 (the activation side reads the same pieces): the four
+            // lanes of a row then ask for 64 contiguous bytes per instruction
+            const int gk = kbase + set * 512 + kk * 128 + kb * 16;
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                const uint32_t vo = (brow < N && gk + h * 16 < k_hi) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
-                rb[set][kk][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 16, 0);
+                const uint32_t vo = (brow < N && gk + h * 64 < k_hi) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
+                rb[set][kk][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 64, 0);
             }
         }
 
@@ -530,9 +532,9 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
 #pragma unroll
                 for (int i = 0; i < MB; i++) {
                     const int row = i * 16 + frow;
-                    const int c0 = kk * 8 + 2 * kb;
+                    const int c0 = kk * 8 + kb;
                     alo[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + ((c0 ^ (row & 15)) << 4)]);
-                    ahi[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + (((c0 + 1) ^ (row & 15)) << 4)]);
+                    ahi[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + (((c0 + 4) ^ (row & 15)) << 4)]);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -613,7 +615,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
 // Still one trip to memory: activation rows first, then the weight rows, everything asked for before the first wait.
 #define NC_DGF_MAX_K 2048
 template <bool A_BF16, int NKS>
-__global__ __launch_bounds__(1024) void gemm_decode_full_kernel(DecodeGemmArgs g) {
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_decode_full_kernel(DecodeGemmArgs g) {
     constexpr int A_LD = A_BF16 ? 2 : 1;
     constexpr int NKQ = (NKS + 3) / 4;              // K-steps per quarter
     extern __shared__ __align__(16) uint8_t dgf_lds[];            // NKS tiles of 8 KB, then 6 x 4 KB for the meeting of the quarters
@@ -666,7 +668,7 @@ __global__ __launch_bounds__(1024) void gemm_decode_full_kernel(DecodeGemmArgs g
             } else {
                 v = ra[j][0];
             }
-            if (j < nksteps) *(dg_v4i*)(&dgf_lds[j * 8192 + arow * 128 + ((ach ^ (arow & 7)) << 4)]) = v;
+            *(dg_v4i*)(&dgf_lds[j * 8192 + arow * 128 + ((ach ^ (arow & 7)) << 4)]) = v;      // (tiles past K hold zeros)
         }
         __syncthreads();                  // the panel is complete
         __syncthreads();                  // (the meeting of the K quarters)
@@ -686,11 +688,12 @@ __global__ __launch_bounds__(1024) void gemm_decode_full_kernel(DecodeGemmArgs g
     dg_v4i rb[NKQ][2];
 #pragma unroll
     for (int j = 0; j < NKQ; j++) {
-        const int gk = (ks0 + j) * 128 + kb * 32;
+        // (a lane's 32 K-bytes of a step are pieces kb and 4 + kb of its 128, on both sides: 64 contiguous bytes per row and instruction)
+        const int gk = (ks0 + j) * 128 + kb * 16;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            const uint32_t vo = (brow < N && j < nk && gk + h * 16 < K) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
-            rb[j][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 16, 0);
+            const uint32_t vo = (brow < N && j < nk && gk + h * 64 < K) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
+            rb[j][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 64, 0);
         }
     }
     if (A_BF16) inv_a = 1.0f / scale_from_amax(amax_from_words(aw));
@@ -699,22 +702,21 @@ __global__ __launch_bounds__(1024) void gemm_decode_full_kernel(DecodeGemmArgs g
     v4f acc[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+    // no branch per K-step (the waits then count loads): a step past this quarter multiplies zero weight rows with some tile of the panel
 #pragma unroll
     for (int j = 0; j < NKQ; j++) {
-        if (j < nk) {
-            const uint8_t* tile = dgf_lds + (ks0 + j) * 8192;
-            v8i bf;
-            bf[0] = rb[j][0][0], bf[1] = rb[j][0][1], bf[2] = rb[j][0][2], bf[3] = rb[j][0][3];
-            bf[4] = rb[j][1][0], bf[5] = rb[j][1][1], bf[6] = rb[j][1][2], bf[7] = rb[j][1][3];
+        const uint8_t* tile = dgf_lds + (j < nk ? ks0 + j : 0) * 8192;
+        v8i bf;
+        bf[0] = rb[j][0][0], bf[1] = rb[j][0][1], bf[2] = rb[j][0][2], bf[3] = rb[j][0][3];
+        bf[4] = rb[j][1][0], bf[5] = rb[j][1][1], bf[6] = rb[j][1][2], bf[7] = rb[j][1][3];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int row = i * 16 + frow;
-                const dg_v4i alo = *(const dg_v4i*)(tile + row * 128 + (((2 * kb) ^ (row & 7)) << 4));
-                const dg_v4i ahi = *(const dg_v4i*)(tile + row * 128 + (((2 * kb + 1) ^ (row & 7)) << 4));
-                v8i af;
-                af[0] = alo[0], af[1] = alo[1], af[2] = alo[2], af[3] = alo[3], af[4] = ahi[0], af[5] = ahi[1], af[6] = ahi[2], af[7] = ahi[3];
-                acc[i] = MFMA_F8(acc[i], bf, af);
-            }
+        for (int i = 0; i < 4; i++) {
+            const int row = i * 16 + frow;
+            const dg_v4i alo = *(const dg_v4i*)(tile + row * 128 + ((kb ^ (row & 7)) << 4));
+            const dg_v4i ahi = *(const dg_v4i*)(tile + row * 128 + (((4 + kb) ^ (row & 7)) << 4));
+            v8i af;
+            af[0] = alo[0], af[1] = alo[1], af[2] = alo[2], af[3] = alo[3], af[4] = ahi[0], af[5] = ahi[1], af[6] = ahi[2], af[7] = ahi[3];
+            acc[i] = MFMA_F8(acc[i], bf, af);
         }
     }
 
@@ -774,6 +776,156 @@ __global__ __launch_bounds__(1024) void gemm_decode_full_kernel(DecodeGemmArgs g
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Unsplit form for a wide output (lm_head): 17 .. 64 rows, K <= 2048, thousands of columns.  A workgroup of 8 waves converts the
+// activation panel into LDS once and then owns 128 columns at a time (16 per wave, the whole of K, no meeting between waves), taking
+// further blocks of 128 while there are any, so the panel is read and converted by at most as many workgroups as the chip has CUs
+// instead of once per 64 columns.  Each wave asks for all weight rows of its block at once and multiplies K-step by K-step as they
+// arrive.
+template <bool A_BF16, int NKS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_decode_wide_kernel(DecodeGemmArgs g) {
+    constexpr int A_LD = A_BF16 ? 2 : 1;
+    extern __shared__ __align__(16) uint8_t dgw_lds[];            // NKS tiles of 8 KB
+    __shared__ float red[8];
+
+    NC_ARG_NOW(g.A); NC_ARG_NOW(g.a_amax); NC_ARG_NOW(g.inv_a); NC_ARG_NOW(g.B); NC_ARG_NOW(g.inv_b); NC_ARG_NOW(g.out); NC_ARG_NOW(g.out_kind);
+    NC_ARG_NOW(g.out_amax); NC_ARG_NOW(g.ldc); NC_ARG_NOW(g.M); NC_ARG_NOW(g.N); NC_ARG_NOW(g.K);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int frow = lane & 15, kb = lane >> 4;
+    const int M = g.M, N = g.N, K = g.K;
+    const int nblk = (N + 127) >> 7;
+
+    AmaxWords aw = {};
+    float inv_a = 0.f;
+    if (A_BF16) aw = amax_load_scalar(g.a_amax);
+    else inv_a = *g.inv_a;
+
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, M * K * (A_BF16 ? 2 : 1), 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, N * K, 0x00020000);
+
+    // activation panel: thread t converts chunk (row t >> 3, 16-byte piece t & 7) of every K-step tile
+    const int arow = tid >> 3, ach = tid & 7;
+    dg_v4i ra[NKS][A_LD], rb[NKS][2];
+#pragma unroll
+    for (int j = 0; j < NKS; j++) {
+        const int gk = j * 128 + ach * 16;
+        const uint32_t vo = (arow < M && gk < K) ? ((uint32_t)arow * (uint32_t)K + (uint32_t)gk) * (A_BF16 ? 2u : 1u) : NC_DG_OOB;
+#pragma unroll
+        for (int h = 0; h < A_LD; h++) ra[j][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, vo, h * 16, 0);
+    }
+    auto load_b = [&](int blk) {
+        const int brow = blk * 128 + wave * 16 + frow;
+#pragma unroll
+        for (int j = 0; j < NKS; j++) {
+            // (a lane's 32 K-bytes of a step are pieces kb and 4 + kb of its 128, on both sides: 64 contiguous bytes per row and instruction)
+            const int gk = j * 128 + kb * 16;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint32_t vo = (brow < N && gk + h * 64 < K) ? (uint32_t)brow * (uint32_t)K + (uint32_t)gk : NC_DG_OOB;
+                rb[j][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_b, vo, h * 64, 0);
+            }
+        }
+    };
+    load_b(blockIdx.x);
+
+    float scale = 1.f;
+    if (A_BF16) {
+        scale = scale_from_amax(amax_from_words(aw));
+        inv_a = 1.0f / scale;
+    }
+#pragma unroll
+    for (int j = 0; j < NKS; j++) {
+        dg_v4i v;
+        if (A_BF16) {
+            const uint32_t w[8] = {(uint32_t)ra[j][0][0], (uint32_t)ra[j][0][1], (uint32_t)ra[j][0][2], (uint32_t)ra[j][0][3],
+                                   (uint32_t)ra[j][A_LD - 1][0], (uint32_t)ra[j][A_LD - 1][1], (uint32_t)ra[j][A_LD - 1][2],
+                                   (uint32_t)ra[j][A_LD - 1][3]};
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                // no clamp needed: |x| <= amax gives |x*scale| <= 448*(1+2^-23), which rounds to 448 like the clamped value
+                v[q] = (int)e4m3_pack4_hw(bf16_lo(w[2 * q]) * scale, bf16_hi(w[2 * q]) * scale, bf16_lo(w[2 * q + 1]) * scale,
+                                          bf16_hi(w[2 * q + 1]) * scale);
+        } else {
+            v = ra[j][0];
+        }
+        *(dg_v4i*)(&dgw_lds[j * 8192 + arow * 128 + ((ach ^ (arow & 7)) << 4)]) = v;      // (tiles past K hold zeros)
+    }
+    __syncthreads();
+
+    float am = 0.f;
+    for (int blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        v4f acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
+        // every tile of the panel, the ones past K included (zeros on both sides): no branch, so the waits count loads
+#pragma unroll
+        for (int j = 0; j < NKS; j++) {
+            const uint8_t* tile = dgw_lds + j * 8192;
+            v8i bf;
+            bf[0] = rb[j][0][0], bf[1] = rb[j][0][1], bf[2] = rb[j][0][2], bf[3] = rb[j][0][3];
+            bf[4] = rb[j][1][0], bf[5] = rb[j][1][1], bf[6] = rb[j][1][2], bf[7] = rb[j][1][3];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = i * 16 + frow;
+                const dg_v4i alo = *(const dg_v4i*)(tile + row * 128 + ((kb ^ (row & 7)) << 4));
+                const dg_v4i ahi = *(const dg_v4i*)(tile + row * 128 + (((4 + kb) ^ (row & 7)) << 4));
+                v8i af;
+                af[0] = alo[0], af[1] = alo[1], af[2] = alo[2], af[3] = alo[3], af[4] = ahi[0], af[5] = ahi[1], af[6] = ahi[2], af[7] = ahi[3];
+                acc[i] = MFMA_F8(acc[i], bf, af);
+            }
+            __builtin_amdgcn_sched_barrier(0);          // (keeps the panel reads of later steps from being hoisted over this one)
+        }
+        // the next block's weight rows are on their way while this one's results leave
+        if (blk + (int)gridDim.x < nblk) load_b(blk + gridDim.x);
+        // lane holds rows 16*i + frow, columns n .. n + 3
+        const int n = blk * 128 + wave * 16 + 4 * kb;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int m = i * 16 + frow;
+            if (m < M && n < N) {
+                const float inv_b = dg_seg_scale(g, n);
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] = (acc[i][r] * inv_a) * inv_b;
+                if (g.out_kind == 1) {
+                    float* o = (float*)g.out + (size_t)m * g.ldc + n;
+                    if (n + 3 < N && (g.ldc & 3) == 0 && ((uintptr_t)g.out & 15) == 0) {
+                        float4 t;
+                        t.x = g.softcap * tanhf(rbf(v[0]) / g.softcap), t.y = g.softcap * tanhf(rbf(v[1]) / g.softcap);
+                        t.z = g.softcap * tanhf(rbf(v[2]) / g.softcap), t.w = g.softcap * tanhf(rbf(v[3]) / g.softcap);
+                        *(float4*)o = t;
+                    } else {
+                        for (int r = 0; r < 4 && n + r < N; r++) o[r] = g.softcap * tanhf(rbf(v[r]) / g.softcap);
+                    }
+                } else {
+                    if (g.out_kind == 2) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const float t = relu_keep_nan(rbf(v[r]));
+                            v[r] = rbf(t * t);
+                            if (n + r < N) am = amax_join(am, v[r]);
+                        }
+                    }
+                    bf16_t* o = (bf16_t*)g.out + (size_t)m * g.ldc + n;
+                    if (n + 3 < N) *(uint2*)o = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                    else
+                        for (int r = 0; r < 4 && n + r < N; r++) o[r] = f32_to_bf16(v[r]);
+                }
+            }
+        }
+    }
+    if (g.out_kind == 2 && g.out_amax) {
+        am = wave_amax(am);
+        if (lane == 0) red[wave] = am;
+        __syncthreads();
+        if (tid == 0) {
+#pragma unroll
+            for (int i = 1; i < 8; i++) am = amax_join(am, red[i]);
+            amax_publish(g.out_amax, amax_join(am, red[0]));
+        }
+    }
+}
+
 namespace {
 template <bool A_BF16, int NKS>
 int launch_full(const DecodeGemmArgs& g, int nblk32, hipStream_t s) {
@@ -790,6 +942,28 @@ int launch_full(const DecodeGemmArgs& g, int nblk32, hipStream_t s) {
     return 0;
 }
 }  // namespace
+
+namespace {
+template <bool A_BF16, int NKS>
+int launch_wide(const DecodeGemmArgs& g, int grid, hipStream_t s) {
+    static bool reserved[64];
+    constexpr int lds_bytes = NKS * 8192;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev < 0 || dev >= 64 || !reserved[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)gemm_decode_wide_kernel<A_BF16, NKS>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm(decode): cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+        if (dev >= 0 && dev < 64) reserved[dev] = true;
+    }
+    hipLaunchKernelGGL((gemm_decode_wide_kernel<A_BF16, NKS>), dim3(grid), dim3(512), lds_bytes, s, g);
+    return 0;
+}
+}  // namespace
+
+// Whether a single-split launch runs the wide form: at least one block of 128 columns per CU.
+static bool dg_wide_form(int M, int N, int K, bool made) {
+    return !made && M > 16 && M <= 64 && K <= NC_DGF_MAX_K && (N + 127) / 128 >= 256 && (int64_t)N * K < ((int64_t)1 << 31);
+}
 
 // Whether nc_launch_gemm_decode, left to choose (ksplits 0), runs the unsplit form: enough 32-column blocks to occupy half the chip
 // and few enough to run in one round.
@@ -963,6 +1137,17 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
     g.recipe = made ? *recipe : NcRowRecipe{};
     NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
+    if (ksplits == 1 && !full && dg_wide_form(M, N, K, made)) {
+        const int nblk128 = (N + 127) / 128, cus = nc_cu_count();
+        const int grid = nblk128 < cus ? nblk128 : cus;
+        int rc;
+        if (nksteps <= 10) rc = a_is_bf16 ? launch_wide<true, 10>(g, grid, s) : launch_wide<false, 10>(g, grid, s);
+        else if (nksteps <= 13) rc = a_is_bf16 ? launch_wide<true, 13>(g, grid, s) : launch_wide<false, 13>(g, grid, s);
+        else rc = a_is_bf16 ? launch_wide<true, 16>(g, grid, s) : launch_wide<false, 16>(g, grid, s);
+        if (rc) return rc;
+        NC_CHECK_LAUNCH("fp8_gemm(decode)");
+        return 0;
+    }
     if (full) {
         const int nblk32 = (N + 31) / 32;
         int rc;

@@ -360,7 +360,9 @@ def test_gemm_softcap_epilogue(ops):
                                            (37, 208, 400, 3),
                                            # the unsplit form (17 .. 64 rows, K <= 2048, 128 .. 256 blocks of 32 columns), ragged edges included
                                            (33, 6656, 1664, 0), (64, 4096, 1280, 0), (48, 8192, 2048, 0), (17, 4100, 1664, 0),
-                                           (64, 5000, 1040, 0)])
+                                           (64, 5000, 1040, 0),
+                                           # the wide unsplit form (at least 256 blocks of 128 columns): two blocks per workgroup, ragged edges
+                                           (33, 65536, 1280, 0), (64, 32804, 2048, 0), (20, 32768, 400, 1)])
 def test_fused_small_m_linear(ops, M, N, K, ksplits):
     """Quantize-inside-the-GEMM decode linear: same bytes as quantize + GEMM, whatever the K split."""
     say(f"fused small-M linear M={M} N={N} K={K} ksplits={ksplits}")
@@ -383,6 +385,10 @@ def test_fused_small_m_linear(ops, M, N, K, ksplits):
     want_h2 = torch.relu(got).square()
     assert torch.equal(h2, want_h2)
     assert am.view(torch.float32).item() == want_h2.float().max().item()
+    # softcap epilogue (fp32 out): the same sums through 15 * tanh(bf16(v) / 15)
+    capped = ops.fp8_linear_small_m(ad, bits, w8d, iwd, softcap=15.0, ksplits=ksplits)
+    assert capped.dtype == torch.float32
+    assert (capped - 15.0 * torch.tanh(got.float() / 15.0)).abs().max().item() < 1e-5
 
 
 def test_split_hand_off_never_reads_stale_partials(ops):
