@@ -282,7 +282,7 @@ typedef struct nc_model_desc {
 typedef struct nc_cache_desc {
     uint16_t* k_cache;           /* bf16 [L, B, Tmax, Hkv, 128]  (engine.py:98-99) */
     uint16_t* v_cache;
-    const int32_t* cache_seqlens;/* int32 [B], tokens cached before this call; the caller advances it */
+    const int32_t* cache_seqlens;/* int32 [B], tokens cached before this call; the caller advances it (but see `advance`) */
     const uint16_t* prev_in;     /* bf16 [B,E] or NULL: KVCache.prev_embedding */
     uint16_t* prev_out;          /* bf16 [B,E]: the value to keep for the next call */
     int batch, max_seq_len;
@@ -292,6 +292,10 @@ typedef struct nc_cache_desc {
      * >= shared_prefix.  A one-token-per-row forward then reads the shared keys of full-context layers once for all rows
      * (nc_decode_attention_shared); results equal to rounding, the caches themselves are untouched by the promise. */
     int shared_prefix, uniform_pos;
+    /* advance != 0 (one-token forwards only, T = 1): nc_gpt_forward adds it to every row's cache_seqlens itself, inside its last row
+     * kernel, once every layer has read the positions; the caller then must not advance them again (saves the caller's own launch,
+     * ~5 us of a decode step).  0: the caller advances, as nanochat/gpt.py:122-123 does. */
+    int advance;
 } nc_cache_desc;
 
 size_t nc_gpt_workspace_bytes(const nc_model_desc* model /*host*/, int B, int T);

@@ -41,7 +41,7 @@ class ModelDesc(C.Structure):
 class CacheDesc(C.Structure):
     _fields_ = [("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("cache_seqlens", C.c_void_p),
                 ("prev_in", C.c_void_p), ("prev_out", C.c_void_p), ("batch", C.c_int), ("max_seq_len", C.c_int),
-                ("shared_prefix", C.c_int), ("uniform_pos", C.c_int)]
+                ("shared_prefix", C.c_int), ("uniform_pos", C.c_int), ("advance", C.c_int)]
 
 
 _lib = None

@@ -190,7 +190,8 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
                                                            const bf16_t* __restrict__ x0, const float* __restrict__ resid_lambda,
                                                            const float* __restrict__ x0_lambda, const float* __restrict__ backout_lambda,
                                                            const bf16_t* __restrict__ backout_src, bf16_t* __restrict__ backout_save,
-                                                           bf16_t* __restrict__ xn_out, int cols, uint32_t* __restrict__ amax_ws) {
+                                                           bf16_t* __restrict__ xn_out, int cols, uint32_t* __restrict__ amax_ws,
+                                                           int32_t* __restrict__ bump, int bump_by) {
     NC_ARG_NOW(x); NC_ARG_NOW(add); NC_ARG_NOW(padd.parts); NC_ARG_NOW(padd.nsplit); NC_ARG_NOW(padd.ld); NC_ARG_NOW(padd.split_stride);
     NC_ARG_NOW(padd.a_amax); NC_ARG_NOW(padd.inv_b); NC_ARG_NOW(x0); NC_ARG_NOW(resid_lambda); NC_ARG_NOW(x0_lambda);
     NC_ARG_NOW(backout_lambda); NC_ARG_NOW(backout_src); NC_ARG_NOW(backout_save); NC_ARG_NOW(xn_out); NC_ARG_NOW(cols); NC_ARG_NOW(amax_ws);
@@ -321,6 +322,8 @@ __global__ __launch_bounds__(256) void mix_norm_vec_kernel(bf16_t* __restrict__ 
         }
     }
     block_amax_commit(am, amax_ws, red);
+    // the row's cache position, advanced here when this is the last kernel of a decode step that reads no positions any more
+    if (bump && threadIdx.x == 0) bump[blockIdx.x] += bump_by;
 }
 
 // out = relu(h)^2, elementwise bf16, plus amax (gpt.py:139)
@@ -537,7 +540,7 @@ int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const floa
 
 static int launch_mix_norm_impl(bf16_t* x, const bf16_t* add, NcPartialSrc padd, const bf16_t* x0, const float* resid_lambda,
                                 const float* x0_lambda, const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save,
-                                bf16_t* xn_out, int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+                                bf16_t* xn_out, int rows, int cols, uint32_t* amax_ws, hipStream_t s, int32_t* bump, int bump_by) {
     NC_CHECK_ARG(x && xn_out, "mix_norm: null pointer");
     NC_CHECK_ARG(row_args_ok(rows, cols), "mix_norm: bad shape rows=%d cols=%d", rows, cols);
     NC_CHECK_ARG(!resid_lambda || (x0 && x0_lambda), "mix_norm: the residual mix needs x0 and x0_lambda");
@@ -549,7 +552,7 @@ static int launch_mix_norm_impl(bf16_t* x, const bf16_t* add, NcPartialSrc padd,
     const bool aligned = cols % 8 == 0 && (((uintptr_t)x | (uintptr_t)xn_out | (uintptr_t)add | (uintptr_t)x0 | (uintptr_t)backout_src |
                                             (uintptr_t)backout_save | (uintptr_t)padd.parts) & 15) == 0 && padd.ld % 4 == 0 &&
                          padd.split_stride % 4 == 0;
-#define MIX_ARGS x, add, padd, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws
+#define MIX_ARGS x, add, padd, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws, bump, bump_by
 #define MIX_LAUNCH(NVV)                                                                                                  \
     do {                                                                                                                 \
         if (padd.parts) hipLaunchKernelGGL((mix_norm_vec_kernel<NVV, true>), dim3(rows), dim3(256), 0, s, MIX_ARGS);      \
@@ -559,7 +562,7 @@ static int launch_mix_norm_impl(bf16_t* x, const bf16_t* add, NcPartialSrc padd,
     else if (aligned && cols <= 4096) MIX_LAUNCH(2);
     else if (aligned && cols <= 8192) MIX_LAUNCH(4);
     else {
-        NC_CHECK_ARG(!padd.parts, "mix_norm: partial-sum input needs cols %% 8 == 0, cols <= 8192 and 16-byte alignment");
+        NC_CHECK_ARG(!padd.parts && !bump, "mix_norm: partial-sum input and the position advance need cols %% 8 == 0, cols <= 8192 and 16-byte alignment");
         hipLaunchKernelGGL(mix_norm_kernel, dim3(rows), dim3(256), cols * sizeof(float), s, x, add, x0, resid_lambda, x0_lambda,
                            backout_lambda, backout_src, backout_save, xn_out, cols, amax_ws);
     }
@@ -571,18 +574,18 @@ static int launch_mix_norm_impl(bf16_t* x, const bf16_t* add, NcPartialSrc padd,
 
 int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
                        const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
-                       int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+                       int rows, int cols, uint32_t* amax_ws, hipStream_t s, int32_t* bump, int bump_by) {
     NcPartialSrc none{nullptr, 0, 0, 0, nullptr, nullptr, 0, 0};
     return launch_mix_norm_impl(x, add, none, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, rows,
-                                cols, amax_ws, s);
+                                cols, amax_ws, s, bump, bump_by);
 }
 
 int nc_launch_mix_norm_p(bf16_t* x, NcPartialSrc add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
                          const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
-                         int rows, int cols, uint32_t* amax_ws, hipStream_t s) {
+                         int rows, int cols, uint32_t* amax_ws, hipStream_t s, int32_t* bump, int bump_by) {
     NC_CHECK_ARG(!add.parts || (add.nsplit >= 1 && add.a_amax && add.inv_b && add.ld >= cols), "mix_norm: bad partial-sum source");
     return launch_mix_norm_impl(x, nullptr, add, x0, resid_lambda, x0_lambda, backout_lambda, backout_src, backout_save, xn_out, rows,
-                                cols, amax_ws, s);
+                                cols, amax_ws, s, bump, bump_by);
 }
 
 int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, hipStream_t s) {

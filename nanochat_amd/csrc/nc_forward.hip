@@ -238,9 +238,11 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
     // output of the previous MLP projection, still to be added into the residual stream: bf16 rows or split partials
     const bf16_t* pending_add = nullptr;
     NcPartialSrc pending_parts = NO_PARTIALS;
-    auto mix = [&](const float* rl, const float* xl, const float* bl, const bf16_t* bsrc, bf16_t* save, uint32_t* amax) -> int {
-        if (pending_parts.parts) return nc_launch_mix_norm_p(w.x, pending_parts, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
-        return nc_launch_mix_norm(w.x, pending_add, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s);
+    auto mix = [&](const float* rl, const float* xl, const float* bl, const bf16_t* bsrc, bf16_t* save, uint32_t* amax,
+                   int32_t* bump = nullptr, int bump_by = 0) -> int {
+        if (pending_parts.parts)
+            return nc_launch_mix_norm_p(w.x, pending_parts, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s, bump, bump_by);
+        return nc_launch_mix_norm(w.x, pending_add, w.x0, rl, xl, bl, bsrc, save, w.xn, M, E, amax, s, bump, bump_by);
     };
     // (measured at d26, steps without a synchronisation in between: one row 1.30 -> 1.13 ms, two rows 1.37 -> 1.27 ms)
     const bool fused = T == 1 && fused_rows(m, M);
@@ -367,7 +369,10 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
             pending_add = nullptr;
             pending_parts = NO_PARTIALS;
         }
-        TRY(mix(nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.site(site)));
+        // every layer has read the positions by now: a one-token step may have them advanced here instead of by a launch of the caller's
+        const bool bump = kv->advance != 0 && T == 1 && E % 8 == 0 && E <= 8192;
+        NC_CHECK_ARG(kv->advance == 0 || bump, "gpt_forward: cache_desc.advance needs T == 1 (and n_embd %% 8 == 0, <= 8192)");
+        TRY(mix(nullptr, nullptr, m->backout_lambda, w.xb, nullptr, w.site(site), bump ? (int32_t*)kv->cache_seqlens : nullptr, kv->advance));
         if (tap_x) TRY(tap_copy(tap_x + (size_t)L * M * E, w.xn, (size_t)M * E, s));
     }
     // lm_head.  Its activation scale is tensorwise over all M rows (that is what the reference quantizes),

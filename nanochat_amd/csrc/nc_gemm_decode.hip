@@ -1065,6 +1065,9 @@ int nc_gemm_decode_splits(int N, int K) {
     int ks = 256 / nblk;
     if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;
+    // a short K (at most 16 steps) is cut in four at most: each workgroup still makes one trip (four steps), and the consumer reads
+    // four partial sums per output instead of seven (measured equal to slightly faster, and 1.3 MB less to write and read back)
+    if (nksteps <= 16 && ks > 4) ks = 4;
     const int kps = (nksteps + ks - 1) / ks;
     return (nksteps + kps - 1) / kps;
 }

@@ -86,11 +86,12 @@ int nc_launch_embed_norm_smear(const int64_t* idx, const bf16_t* wte, const floa
                                int vocab_rows, uint32_t* clear_words, int n_clear, hipStream_t s);
 int nc_launch_mix_norm(bf16_t* x, const bf16_t* add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
                        const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
-                       int rows, int cols, uint32_t* amax_ws, hipStream_t s);
+                       int rows, int cols, uint32_t* amax_ws, hipStream_t s, int32_t* bump = nullptr, int bump_by = 0);
+// (bump: int32 [rows] or null; row r's workgroup adds bump_by to bump[r] when it is done -- the cache positions of a decode step)
 // same, with the added tensor given as split partials of the linear that produced it (decode path)
 int nc_launch_mix_norm_p(bf16_t* x, NcPartialSrc add, const bf16_t* x0, const float* resid_lambda, const float* x0_lambda,
                          const float* backout_lambda, const bf16_t* backout_src, bf16_t* backout_save, bf16_t* xn_out,
-                         int rows, int cols, uint32_t* amax_ws, hipStream_t s);
+                         int rows, int cols, uint32_t* amax_ws, hipStream_t s, int32_t* bump = nullptr, int bump_by = 0);
 int nc_launch_relu2(const bf16_t* h, bf16_t* out, int64_t n, uint32_t* amax_ws, hipStream_t s);
 int nc_launch_qkv_rope_append_p(NcPartialSrc qkv_parts, const bf16_t* xn, int ld_xn, const int64_t* idx,
                                 const bf16_t* ve_table, const float* ve_gate_w, const bf16_t* cos, const bf16_t* sin,

@@ -125,6 +125,11 @@ class KVCache:
         self._pos0 += num_tokens
         self._pos_max += num_tokens
 
+    def note_advanced(self, num_tokens):
+        """The forward call advanced `cache_seqlens` on the device itself (nc_cache_desc.advance): only the host mirrors follow."""
+        self._pos0 += num_tokens
+        self._pos_max += num_tokens
+
     def rewind(self, num_tokens, prev_embedding):
         """Take back the last advance (the appended rows stay in the tensors and are overwritten by the next
         append at the same positions); `prev_embedding` is the smear state from before that forward."""
@@ -292,6 +297,8 @@ class Engine:
             # time to the first token ends before the first decode forward)
             run_ahead = ahead and produced > 0 and not (max_tokens is not None and produced + 1 >= max_tokens)
             if run_ahead:
+                # (on the launch stream: handing this copy to a stream of its own costs 90 us per step -- with a second queue
+                # active every one of the step's ~190 launches starts ~0.5 us later)
                 host_ids.copy_(sampled_dev[:, 0], non_blocking=True)
                 ids_ready.record()
                 prev_before = kv_decode.prev_embedding

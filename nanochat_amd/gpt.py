@@ -362,6 +362,9 @@ class GPT(nn.Module):
         shared = getattr(kv_cache, "shared_prefix_len", 0) if getattr(kv_cache, "share_prompt_reads", False) else 0
         uniform = T == 1 and pos0 is not None and pos0 == pos_hi and shared > 0 and pos0 >= shared
         cd.shared_prefix, cd.uniform_pos = (shared, pos0) if uniform else (0, 0)
+        # a one-token step: the library advances the positions inside its last row kernel (one launch less per step)
+        advance_inside = T == 1 and hasattr(kv_cache, "note_advanced") and cfg.n_embd % 8 == 0 and cfg.n_embd <= 8192
+        cd.advance = T if advance_inside else 0
         ws_ptr, ws_bytes = self._workspace(md, B, T, idx.device)
         if taps is None:
             rc = _lib.lib().nc_gpt_forward(C.byref(md), C.byref(cd), idx.data_ptr(), B, T, logits.data_ptr(), 1 if last_only else 0,
@@ -374,7 +377,10 @@ class GPT(nn.Module):
                                                   torch.cuda.current_stream().cuda_stream)
         _lib.check(rc)
         kv_cache.prev_embedding = prev_out
-        kv_cache.advance(T)
+        if advance_inside:
+            kv_cache.note_advanced(T)
+        else:
+            kv_cache.advance(T)
         return logits if last_only else logits.view(B, T, cfg.vocab_size)
 
     def forward(self, idx, targets=None, kv_cache=None, loss_reduction='mean'):

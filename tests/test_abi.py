@@ -39,7 +39,7 @@ def test_struct_layout_matches_header():
     # pointer-sized fields + ints: sizes as a C compiler lays them out on LP64
     assert ctypes.sizeof(_lib.LayerDesc) == 10 * 8 + 2 * 4
     assert ctypes.sizeof(_lib.ModelDesc) == 8 * 4 + 2 * 4 + 11 * 8
-    assert ctypes.sizeof(_lib.CacheDesc) == 5 * 8 + 4 * 4
+    assert ctypes.sizeof(_lib.CacheDesc) == 5 * 8 + 5 * 4 + 4
 
 
 def test_library_was_built_from_these_sources():
