@@ -298,8 +298,22 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         for (int w = 0; w < 4; w++) mm = fmaxf(mm, merge[w][hg][0]);
         const int head = (hp * HP + hg / G) * G + hg % G;
         const float* ex = extra ? extra + ((size_t)row * H + head) * n_extra * PART_STRIDE : nullptr;
-        if (ex)
+        // up to 16 partial results of the shared start: all of their words asked for at once (one trip to memory at the end of the
+        // kernel instead of one per partial), added in chunk order like the loop below
+        const bool few = ex && n_extra <= 16;
+        float em[16], el[16], ea[16];
+        if (few) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const float* q = ex + (e < n_extra ? e : 0) * PART_STRIDE;
+                em[e] = q[0], el[e] = q[1], ea[e] = q[4 + d];
+            }
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                if (e < n_extra) mm = fmaxf(mm, em[e]);
+        } else if (ex) {
             for (int e = 0; e < n_extra; e++) mm = fmaxf(mm, ex[e * PART_STRIDE]);
+        }
         float ls = 0.f, a = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
@@ -307,12 +321,21 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
             ls += merge[w][hg][1] * sc;
             a += merge[w][hg][4 + d] * sc;
         }
-        if (ex)
+        if (few) {
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                if (e < n_extra) {
+                    const float sc = exp2f(em[e] - mm);
+                    ls += el[e] * sc;
+                    a += ea[e] * sc;
+                }
+        } else if (ex) {
             for (int e = 0; e < n_extra; e++) {
                 const float sc = exp2f(ex[e * PART_STRIDE] - mm);
                 ls += ex[e * PART_STRIDE + 1] * sc;
                 a += ex[e * PART_STRIDE + 4 + d] * sc;
             }
+        }
         if (nsplit == 1) {
             const bf16_t o = f32_to_bf16(a / ls);
             out[((size_t)row * H + head) * 128 + d] = o;

@@ -391,6 +391,26 @@ def test_fused_small_m_linear(ops, M, N, K, ksplits):
     assert (capped - 15.0 * torch.tanh(got.float() / 15.0)).abs().max().item() < 1e-5
 
 
+@pytest.mark.parametrize("M,N,K,forms", [(64, 6656, 1664, (0, 1, 2, 4)),      # unsplit (32 columns per workgroup) / chunk-walking / one trip
+                                         (64, 4992, 1664, (0, 1, 3)), (64, 1664, 6656, (0, 1, 13)), (64, 1664, 1664, (0, 1, 7)),
+                                         (64, 32768, 1664, (0, 2, 4)),           # wide unsplit form / one trip
+                                         (40, 6656, 1280, (0, 2, 5))])
+def test_decode_linear_forms_agree_bit_for_bit(ops, M, N, K, forms):
+    """The small-M linear has several kernels (one trip per split, unsplit with the activation in the GEMM, wide unsplit, chunk-walking);
+    which one runs depends on the shape and on the split count asked for.  On the same operands they must give the same bf16 bits --
+    the fp32 sums of e4m3 products are formed in another order, which must not show -- and the same relu^2 + amax."""
+    say(f"decode linear forms M={M} N={N} K={K} splits {forms}")
+    a, w = make_operands(M, N, K, seed=3 * M + N + K)
+    w8, iw, _ = fp8_ref.to_fp8(w)
+    ad, w8d, iwd = a.to(DEV), w8.to(DEV), iw.reshape(1).to(DEV)
+    bits = ops.amax_bits(ad)
+    outs = [ops.fp8_linear_small_m(ad, bits, w8d, iwd, ksplits=ks) for ks in forms]
+    acts = [ops.fp8_linear_small_m(ad, bits, w8d, iwd, relu2=True, ksplits=ks) for ks in forms]
+    for ks, o, (h2, am) in zip(forms[1:], outs[1:], acts[1:]):
+        assert torch.equal(o, outs[0]), f"ksplits={ks}: {(o.float() - outs[0].float()).abs().max().item()}"
+        assert torch.equal(h2, acts[0][0]) and torch.equal(am, acts[0][1]), f"relu^2 form, ksplits={ks}"
+
+
 def test_split_hand_off_never_reads_stale_partials(ops):
     """The split-K GEMM and the split attention pass partial results between workgroups through a scratch
     buffer that is reused by every call.  Alternate two different inputs many times: a stale partial from
