@@ -431,13 +431,17 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
 // through the scalar cache, which has a counter of its own.
 #define NC_DG_OOB 0x80000000u
 typedef int dg_v4i __attribute__((ext_vector_type(4)));
-template <int MB, bool A_BF16, int NSET>
+// A_MODE as in gemm_decode_kernel: 0 e4m3 activations, 1 bf16 + the producer's amax, 2 / 3 rows made here from a recipe of kind 1 / 2
+// (one or two rows; the weight rows are on their way while the rows are made).
+template <int MB, int A_MODE, int NSET>
 __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs g) {
+    constexpr bool A_BF16 = A_MODE != 0;
     constexpr int ROWS = MB * 16;
     constexpr int A_CH = ROWS * 32 / 256;          // 16-byte e4m3 chunks per thread per 512-wide half of the range
     constexpr int A_LD = A_BF16 ? 2 : 1;
     __shared__ __align__(16) uint8_t lds[NSET][ROWS * 512];
-    __shared__ float red[4];
+    __shared__ float red[8];
+    __shared__ __align__(16) bf16_t rowbuf[A_MODE == 2 ? NC_RECIPE_MAX_ROWS * 2048 : (A_MODE == 3 ? NC_RECIPE_MAX_ROWS * NC_RECIPE_MAX_K : 8)];
 
     NC_ARG_NOW(g.A); NC_ARG_NOW(g.a_amax); NC_ARG_NOW(g.inv_a); NC_ARG_NOW(g.B); NC_ARG_NOW(g.partial_out); NC_ARG_NOW(g.ksplits);
     NC_ARG_NOW(g.ksteps_per_split); NC_ARG_NOW(g.M); NC_ARG_NOW(g.N); NC_ARG_NOW(g.K);
@@ -458,8 +462,8 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
 
     AmaxWords aw = {};
     float inv_a = 0.f;
-    if (A_BF16) aw = amax_load_scalar(g.a_amax);
-    else inv_a = *g.inv_a;
+    if (A_MODE == 1) aw = amax_load_scalar(g.a_amax);
+    else if (A_MODE == 0) inv_a = *g.inv_a;
 
     const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, M * K * (A_BF16 ? 2 : 1), 0x00020000);
     const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, N * K, 0x00020000);
@@ -467,16 +471,18 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
     // (measured: handing the conversion to waves of their own, so that the weight requests go out first, is slower, 9.9 against
     // 8.3 us at N = 6656, K = 1664)
     dg_v4i ra[NSET][A_CH][A_LD], rb[NSET][4][2];
+    if (A_MODE < 2) {
 #pragma unroll
-    for (int set = 0; set < NSET; set++)
+        for (int set = 0; set < NSET; set++)
 #pragma unroll
-        for (int c = 0; c < A_CH; c++) {
-            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
-            const int gk = kbase + set * 512 + ch * 16;
-            const uint32_t vo = (row < M && gk < k_hi) ? ((uint32_t)row * (uint32_t)K + (uint32_t)gk) * (A_BF16 ? 2u : 1u) : NC_DG_OOB;
+            for (int c = 0; c < A_CH; c++) {
+                const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+                const int gk = kbase + set * 512 + ch * 16;
+                const uint32_t vo = (row < M && gk < k_hi) ? ((uint32_t)row * (uint32_t)K + (uint32_t)gk) * (A_BF16 ? 2u : 1u) : NC_DG_OOB;
 #pragma unroll
-            for (int h = 0; h < A_LD; h++) ra[set][c][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, vo, h * 16, 0);
-        }
+                for (int h = 0; h < A_LD; h++) ra[set][c][h] = __builtin_amdgcn_raw_buffer_load_b128(desc_a, vo, h * 16, 0);
+            }
+    }
 #pragma unroll
     for (int set = 0; set < NSET; set++)
 #pragma unroll
@@ -492,9 +498,26 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
         }
 
     float scale = 1.f;
-    if (A_BF16) {
+    if (A_MODE == 1) {
         scale = scale_from_amax(amax_from_words(aw));
         inv_a = 1.0f / scale;
+    }
+    if (A_MODE >= 2) {
+        // the rows from their recipe, as bf16 in LDS, then this workgroup's K range of them into the staging registers
+        scale = scale_from_amax(recipe_rows<A_MODE - 1>(g.recipe, rowbuf, red, M, K, blockIdx.x == 0 && blockIdx.y == 0));
+        inv_a = 1.0f / scale;
+#pragma unroll
+        for (int set = 0; set < NSET; set++)
+#pragma unroll
+            for (int c = 0; c < A_CH; c++) {
+                const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+                const int gk = kbase + set * 512 + ch * 16;
+                const bool ok = row < M && gk < k_hi;
+                const dg_v4i* p = (const dg_v4i*)(rowbuf + (ok ? (size_t)row * K + gk : 0));
+                const dg_v4i z = {0, 0, 0, 0};
+                ra[set][c][0] = ok ? p[0] : z;
+                ra[set][c][A_LD - 1] = ok ? p[1] : z;
+            }
     }
 #pragma unroll
     for (int set = 0; set < NSET; set++)
@@ -1162,25 +1185,28 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
         return 0;
     }
     dim3 grid(nblk, ksplits), block(256);
-    const bool onetrip = !made && MB <= 4 && kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
-#define OT_LAUNCH(MB_, AB_)                                                                                            \
+    const bool onetrip = MB <= 4 && kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
+#define OT_LAUNCH(MB_, MODE_)                                                                                          \
     do {                                                                                                               \
-        if (kps <= 4) hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, AB_, 1>), grid, block, 0, s, g);             \
-        else hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, AB_, 2>), grid, block, 0, s, g);                     \
+        if (kps <= 4) hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 1>), grid, block, 0, s, g);           \
+        else hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 2>), grid, block, 0, s, g);                   \
     } while (0)
     if (onetrip) {
-        if (MB == 1) {
-            if (a_is_bf16) OT_LAUNCH(1, true);
-            else OT_LAUNCH(1, false);
+        if (made) {
+            if (recipe->kind == 1) OT_LAUNCH(1, 2);
+            else OT_LAUNCH(1, 3);
+        } else if (MB == 1) {
+            if (a_is_bf16) OT_LAUNCH(1, 1);
+            else OT_LAUNCH(1, 0);
         } else if (MB == 2) {
-            if (a_is_bf16) OT_LAUNCH(2, true);
-            else OT_LAUNCH(2, false);
+            if (a_is_bf16) OT_LAUNCH(2, 1);
+            else OT_LAUNCH(2, 0);
         } else if (MB == 3) {
-            if (a_is_bf16) OT_LAUNCH(3, true);
-            else OT_LAUNCH(3, false);
+            if (a_is_bf16) OT_LAUNCH(3, 1);
+            else OT_LAUNCH(3, 0);
         } else {
-            if (a_is_bf16) OT_LAUNCH(4, true);
-            else OT_LAUNCH(4, false);
+            if (a_is_bf16) OT_LAUNCH(4, 1);
+            else OT_LAUNCH(4, 0);
         }
     } else if (MB == 1) {
         if (made && recipe->kind == 1) hipLaunchKernelGGL((gemm_decode_kernel<1, 2>), grid, block, 0, s, g);
