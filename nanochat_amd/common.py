@@ -24,10 +24,13 @@ PEAK_HBM_BYTES_PER_S = 8.0e12
 
 
 def get_peak_flops(device_name=None):
+    """Dense bf16 peak (common.py:228-270).  The library's kernels exist for gfx950 only, so there is one answer whatever the driver
+    calls the device (some report an empty or generic name); the argument is kept for the reference's signature."""
     return PEAK_BF16_FLOPS
 
 
 def get_peak_bandwidth(device_name=None):
+    """HBM peak (common.py:300-328); one answer, as for get_peak_flops."""
     return PEAK_HBM_BYTES_PER_S
 
 
