@@ -17,6 +17,7 @@
 //
 // HBM traffic per (row, kv head): 2 * n_keys * 256 bytes, the algorithmic minimum.
 #include <type_traits>
+#include <hip/hip_ext.h>
 #include "nc_common.h"
 #include "nc_kernels.h"
 #include "nc_rope.h"
@@ -444,15 +445,25 @@ static int launch_attention_impl(const bf16_t* q, const NcRopeSrc* rope, int mod
     }
     NC_CHECK_ARG(!extra || (nsplit == 1 && mode == 0 && T == 1 && n_extra > 0 && k_min > 0),
                  "decode_attention: a shared first part goes with one split, one query per row and tokens already appended");
-    NcProfScope prof(0, 0.0, s);
+    // when the profiler is on, the launch carries its own event pair (kernel begin / end, no marker packets around it)
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    const bool timed = nc_prof_take(0, 0.0, 0, &ev0, &ev1);
     float* parts = (float*)partials;
     const int hp = (force_splits > 0 || nsplit > 1) ? 1 : pick_heads_per_wg(B, T, Hkv);
     dim3 grid(nsplit, hp == 2 ? (Hkv + 1) / 2 : Hkv, B * T), block(256);
     const NcRopeSrc none{};
     const NcRopeSrc& rs = rope ? *rope : none;
-#define LAUNCH_GMH(GG, MM, HH)                                                                                                \
-    hipLaunchKernelGGL((attn_partial_kernel<GG, MM, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens, window_left, \
-                       seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, rs, k_min, extra, n_extra)
+#define LAUNCH_GMH(GG, MM, HH)                                                                                                     \
+    do {                                                                                                                           \
+        if (timed)                                                                                                                 \
+            hipExtLaunchKernelGGL((attn_partial_kernel<GG, MM, HH>), grid, block, 0, s, ev0, ev1, 0, q, k_cache, v_cache,         \
+                                  cache_seqlens, window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, \
+                                  nsplit, rs, k_min, extra, n_extra);                                                              \
+        else                                                                                                                       \
+            hipLaunchKernelGGL((attn_partial_kernel<GG, MM, HH>), grid, block, 0, s, q, k_cache, v_cache, cache_seqlens,           \
+                               window_left, seqlens_include_new, out, parts, counters, amax_ws, T, H, Hkv, Tmax, nsplit, rs,       \
+                               k_min, extra, n_extra);                                                                             \
+    } while (0)
 #define LAUNCH_GH(GG, HH)                          \
     do {                                           \
         if (mode == 1) LAUNCH_GMH(GG, 1, HH);      \

@@ -28,6 +28,7 @@
 //
 // Epilogues: 0 bf16;  1 fp32 softcap*tanh(bf16(v)/softcap) (lm_head, nanochat/gpt.py:512-515);
 //            2 bf16 relu(bf16(v))^2 plus atomic amax of the result (MLP activation, gpt.py:139).
+#include <hip/hip_ext.h>
 #include "nc_common.h"
 #include "nc_kernels.h"
 #include "nc_rope.h"
@@ -951,7 +952,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 namespace {
 template <bool A_BF16, int NKS>
-int launch_full(const DecodeGemmArgs& g, int nblk32, hipStream_t s) {
+int launch_full(const DecodeGemmArgs& g, int nblk32, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
     static bool reserved[64];
     constexpr int lds_bytes = NKS * 8192 + 6 * 4096;
     int dev = 0;
@@ -961,14 +962,15 @@ int launch_full(const DecodeGemmArgs& g, int nblk32, hipStream_t s) {
         if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm(decode): cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
         if (dev >= 0 && dev < 64) reserved[dev] = true;
     }
-    hipLaunchKernelGGL((gemm_decode_full_kernel<A_BF16, NKS>), dim3(nblk32), dim3(1024), lds_bytes, s, g);
+    if (ev0) hipExtLaunchKernelGGL((gemm_decode_full_kernel<A_BF16, NKS>), dim3(nblk32), dim3(1024), lds_bytes, s, ev0, ev1, 0, g);
+    else hipLaunchKernelGGL((gemm_decode_full_kernel<A_BF16, NKS>), dim3(nblk32), dim3(1024), lds_bytes, s, g);
     return 0;
 }
 }  // namespace
 
 namespace {
 template <bool A_BF16, int NKS>
-int launch_wide(const DecodeGemmArgs& g, int grid, hipStream_t s) {
+int launch_wide(const DecodeGemmArgs& g, int grid, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
     static bool reserved[64];
     constexpr int lds_bytes = NKS * 8192;
     int dev = 0;
@@ -978,7 +980,8 @@ int launch_wide(const DecodeGemmArgs& g, int grid, hipStream_t s) {
         if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm(decode): cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
         if (dev >= 0 && dev < 64) reserved[dev] = true;
     }
-    hipLaunchKernelGGL((gemm_decode_wide_kernel<A_BF16, NKS>), dim3(grid), dim3(512), lds_bytes, s, g);
+    if (ev0) hipExtLaunchKernelGGL((gemm_decode_wide_kernel<A_BF16, NKS>), dim3(grid), dim3(512), lds_bytes, s, ev0, ev1, 0, g);
+    else hipLaunchKernelGGL((gemm_decode_wide_kernel<A_BF16, NKS>), dim3(grid), dim3(512), lds_bytes, s, g);
     return 0;
 }
 }  // namespace
@@ -1153,23 +1156,30 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     }
     if (ksplits_out) *ksplits_out = ksplits;
 
-    // rows of the MFMA block: the A panel in LDS (and its staging, zero rows included) is sized by it, so a small batch takes a small
-    // block (batch 8: 1.50 -> 1.35 ms per d26 step with 16 rows instead of 64)
-    const int MB = (made || M <= 16) ? 1 : (M <= 32 ? 2 : (M <= 48 ? 3 : (M <= 64 ? 4 : 8)));
     const int nblk = (N + 63) / 64;
     DecodeGemmArgs g;
     g.A = a, g.a_amax = a_amax, g.inv_a = inv_a, g.B = b, g.inv_b = inv_b, g.segs = segs, g.out = out, g.out_kind = out_kind;
     g.softcap = softcap, g.ldc = ldc, g.out_amax = out_amax, g.partial_out = partials;
     g.ksplits = ksplits, g.ksteps_per_split = kps, g.M = M, g.N = N, g.K = K;
     g.recipe = made ? *recipe : NcRowRecipe{};
-    NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
-    if (ksplits == 1 && !full && dg_wide_form(M, N, K, made)) {
+    // rows of the MFMA block: the A panel in LDS (and its staging, zero rows included) is sized by it, so a small batch takes a small
+    // block (batch 8: 1.50 -> 1.35 ms per d26 step with 16 rows instead of 64)
+    const int MB = (made || M <= 16) ? 1 : (M <= 32 ? 2 : (M <= 48 ? 3 : (M <= 64 ? 4 : 8)));
+    const bool wide = ksplits == 1 && !full && dg_wide_form(M, N, K, made);
+    const bool onetrip = MB <= 4 && kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
+    // the one-trip, unsplit and wide forms hand their event pair to the launch itself when the profiler is on (the kernel's own begin and end,
+    // no marker packets around it); the chunk-walking kernel keeps the bracketing pair
+    const bool own_events = wide || full || onetrip;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    if (own_events && !nc_prof_take(1, 2.0 * M * N * K, ((int64_t)N << 32) | (uint32_t)K, &ev0, &ev1)) ev0 = ev1 = nullptr;
+    NcProfScope prof(own_events ? -1 : 1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
+    if (wide) {
         const int nblk128 = (N + 127) / 128, cus = nc_cu_count();
         const int grid = nblk128 < cus ? nblk128 : cus;
         int rc;
-        if (nksteps <= 10) rc = a_is_bf16 ? launch_wide<true, 10>(g, grid, s) : launch_wide<false, 10>(g, grid, s);
-        else if (nksteps <= 13) rc = a_is_bf16 ? launch_wide<true, 13>(g, grid, s) : launch_wide<false, 13>(g, grid, s);
-        else rc = a_is_bf16 ? launch_wide<true, 16>(g, grid, s) : launch_wide<false, 16>(g, grid, s);
+        if (nksteps <= 10) rc = a_is_bf16 ? launch_wide<true, 10>(g, grid, s, ev0, ev1) : launch_wide<false, 10>(g, grid, s, ev0, ev1);
+        else if (nksteps <= 13) rc = a_is_bf16 ? launch_wide<true, 13>(g, grid, s, ev0, ev1) : launch_wide<false, 13>(g, grid, s, ev0, ev1);
+        else rc = a_is_bf16 ? launch_wide<true, 16>(g, grid, s, ev0, ev1) : launch_wide<false, 16>(g, grid, s, ev0, ev1);
         if (rc) return rc;
         NC_CHECK_LAUNCH("fp8_gemm(decode)");
         return 0;
@@ -1177,18 +1187,19 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     if (full) {
         const int nblk32 = (N + 31) / 32;
         int rc;
-        if (nksteps <= 10) rc = a_is_bf16 ? launch_full<true, 10>(g, nblk32, s) : launch_full<false, 10>(g, nblk32, s);
-        else if (nksteps <= 13) rc = a_is_bf16 ? launch_full<true, 13>(g, nblk32, s) : launch_full<false, 13>(g, nblk32, s);
-        else rc = a_is_bf16 ? launch_full<true, 16>(g, nblk32, s) : launch_full<false, 16>(g, nblk32, s);
+        if (nksteps <= 10) rc = a_is_bf16 ? launch_full<true, 10>(g, nblk32, s, ev0, ev1) : launch_full<false, 10>(g, nblk32, s, ev0, ev1);
+        else if (nksteps <= 13) rc = a_is_bf16 ? launch_full<true, 13>(g, nblk32, s, ev0, ev1) : launch_full<false, 13>(g, nblk32, s, ev0, ev1);
+        else rc = a_is_bf16 ? launch_full<true, 16>(g, nblk32, s, ev0, ev1) : launch_full<false, 16>(g, nblk32, s, ev0, ev1);
         if (rc) return rc;
         NC_CHECK_LAUNCH("fp8_gemm(decode)");
         return 0;
     }
     dim3 grid(nblk, ksplits), block(256);
-    const bool onetrip = MB <= 4 && kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
 #define OT_LAUNCH(MB_, MODE_)                                                                                          \
     do {                                                                                                               \
-        if (kps <= 4) hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 1>), grid, block, 0, s, g);           \
+        if (kps <= 4 && ev0) hipExtLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 1>), grid, block, 0, s, ev0, ev1, 0, g); \
+        else if (kps <= 4) hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 1>), grid, block, 0, s, g);      \
+        else if (ev0) hipExtLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 2>), grid, block, 0, s, ev0, ev1, 0, g); \
         else hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 2>), grid, block, 0, s, g);                   \
     } while (0)
     if (onetrip) {

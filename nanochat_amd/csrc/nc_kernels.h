@@ -151,6 +151,7 @@ int nc_launch_sample(const float* logits, int B, int V, int ld, float temperatur
 // ---- optional event timing (nc_profile.hip)
 int nc_prof_begin(int cls, double units, hipStream_t s, int64_t tag = 0);
 void nc_prof_end(int slot, hipStream_t s);
+bool nc_prof_take(int cls, double units, int64_t tag, hipEvent_t* start, hipEvent_t* stop);
 struct NcProfScope {
     int slot;
     hipStream_t s;

@@ -1,6 +1,7 @@
 // Optional per-kernel-class timing with HIP events on the launch stream.  Off by default (zero cost
 // beyond one branch); when on, every nc_launch_* brackets its launches with a start/stop event pair
-// taken from a fixed pool.  nc_profile_read() waits for the events and sums the elapsed times.
+// taken from a fixed pool (the decode attention launch, whose duration the roofline figure is made of, gives its pair to the launch
+// itself instead, see nc_prof_take).  nc_profile_read() waits for the events and sums the elapsed times.
 #include "../../include/nanochat_amd.h"
 #include "nc_common.h"
 #include "nc_kernels.h"
@@ -31,6 +32,21 @@ int nc_prof_begin(int cls, double units, hipStream_t s, int64_t tag) {
     r.tag = tag;
     (void)hipEventRecord(r.start, s);
     return g_used++;
+}
+
+// A record whose two events the caller hands to the launch itself (hipExtLaunchKernelGGL): they then hold the kernel's own begin and end
+// timestamps, without the marker packets that hipEventRecord puts around a launch.  Returns false when profiling is off.
+bool nc_prof_take(int cls, double units, int64_t tag, hipEvent_t* start, hipEvent_t* stop) {
+    if (!g_on || cls < 0 || g_used >= POOL) return false;
+    if (g_used >= g_created) {
+        if (hipEventCreate(&g_recs[g_created].start) != hipSuccess) return false;
+        if (hipEventCreate(&g_recs[g_created].stop) != hipSuccess) return false;
+        g_created++;
+    }
+    Rec& r = g_recs[g_used++];
+    r.cls = cls, r.units = units, r.tag = tag;
+    *start = r.start, *stop = r.stop;
+    return true;
 }
 
 void nc_prof_end(int slot, hipStream_t s) {
