@@ -661,6 +661,43 @@ def test_full_size_d32_gqa_batch128_ragged_rows():
     assert rel < 0.1
 
 
+@pytest.mark.parametrize("B", [1, 3, 40])
+def test_positions_advanced_inside_the_step_or_by_the_caller(B):
+    """A one-token forward may advance cache_seqlens inside its last row kernel (nc_cache_desc.advance) instead of leaving it to the
+    caller: same logits, same positions, same cache, for the fused small-batch step (1 row), the split linears (3) and the unsplit
+    c_fc (40 rows)."""
+    say(f"positions advanced inside the step, {B} row(s)")
+    from nanochat_amd.engine import KVCache
+
+    class CallerAdvances(KVCache):
+        """A cache without note_advanced(): GPT.forward then leaves advance = 0 and calls advance() itself."""
+        def __getattribute__(self, name):
+            if name == "note_advanced":
+                raise AttributeError(name)
+            return super().__getattribute__(name)
+
+    cfg_kwargs = dict(sequence_len=64, vocab_size=1024, n_layer=3, n_head=4, n_kv_head=2, n_embd=512, window_pattern="SL")
+    _, model = build_pair(cfg_kwargs, seed=43)
+    g = torch.Generator().manual_seed(44)
+    P, steps = 7, 4
+    prompt = torch.randint(0, 1024, (B, P), generator=g).to(DEV)
+    toks = [torch.randint(0, 1024, (B, 1), generator=g).to(DEV) for _ in range(steps)]
+    caches = [cls(B, 2, P + steps + 1, 128, 3, DEV, torch.bfloat16) for cls in (KVCache, CallerAdvances)]
+    assert hasattr(caches[0], "note_advanced") and not hasattr(caches[1], "note_advanced")
+    outs = []
+    for c in caches:
+        got = [model.forward_last(prompt, kv_cache=c).clone()]
+        for t in toks:
+            got.append(model.forward_last(t, kv_cache=c).clone())
+            assert c.get_pos() == int(c.cache_seqlens[0])                 # the host mirror follows either way
+        outs.append(got)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert torch.equal(caches[0].cache_seqlens, caches[1].cache_seqlens)
+    assert int(caches[0].cache_seqlens[B - 1]) == P + steps
+    assert torch.equal(caches[0].k_cache, caches[1].k_cache) and torch.equal(caches[0].v_cache, caches[1].v_cache)
+
+
 def test_weight_changes_are_noticed_by_the_next_forward():
     """The quantized copies of the FP8 weights are cached between calls; every way of changing a weight that the module API offers
     must refresh them: an in-place update, load_state_dict (copying and assigning), a cast of a child module, and the explicit call
