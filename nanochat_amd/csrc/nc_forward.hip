@@ -40,9 +40,11 @@
         if (rc__) return rc__; \
     } while (0)
 
-// Reading a shared prompt once for all rows pays from a few rows on and for layers that see a long stretch of it
+// Reading a shared prompt once for all rows pays from a few rows on, and for a layer whose visible keys are at least half shared ones
+// (a full-context layer for as long as the rows have decoded fewer tokens than the prompt holds; a windowed layer until its window
+// has moved halfway out of the prompt): the shared launch and the separate rotary launch cost what ~250 keys per row cost to stream
 #define NC_SHARED_MIN_ROWS 16
-#define NC_SHARED_MIN_KEYS 768
+#define NC_SHARED_MIN_KEYS 256
 
 namespace {
 struct Carver {
@@ -313,7 +315,8 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
         bool shared_done = false;
         if (T == 1 && B >= NC_SHARED_MIN_ROWS && kv->shared_prefix > 0 && kv->uniform_pos >= kv->shared_prefix && w.shared_parts) {
             const int first_visible = ly.window_left < 0 ? 0 : (kv->uniform_pos - ly.window_left > 0 ? kv->uniform_pos - ly.window_left : 0);
-            if (kv->shared_prefix - first_visible >= NC_SHARED_MIN_KEYS && kv->shared_prefix < kv->max_seq_len) {
+            const int shared_visible = kv->shared_prefix - first_visible, own_visible = kv->uniform_pos + 1 - kv->shared_prefix;
+            if (shared_visible >= NC_SHARED_MIN_KEYS && shared_visible >= own_visible && kv->shared_prefix < kv->max_seq_len) {
                 if (qsrc.parts)
                     TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
                                                     kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
