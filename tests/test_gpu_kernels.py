@@ -411,6 +411,37 @@ def test_decode_linear_forms_agree_bit_for_bit(ops, M, N, K, forms):
         assert torch.equal(h2, acts[0][0]) and torch.equal(am, acts[0][1]), f"relu^2 form, ksplits={ks}"
 
 
+def test_fused_small_m_linear_seeded_shape_sweep(ops):
+    """Forty seeded shapes around the borders between the decode linear's forms (rows 1 .. 128 across the 16-row blocks, widths that
+    are no multiple of the 32 / 64 / 128-column blocks, K that ends inside a 128-wide step, every split count the caller may ask
+    for): the result against the oracle's emulated product, and the relu^2 form against the plain one."""
+    say("fused small-M linear: seeded shape sweep")
+    import random
+    rnd = random.Random(20)
+    shapes = []
+    for _ in range(40):
+        M = rnd.choice([1, 2, 3, 15, 16, 17, 31, 33, 47, 49, 63, 64, 65, 100, 128])
+        N = 4 * rnd.choice([1, 7, 16, 33, 250, 416, 1025, 1248, 1664, 2049, 8200])
+        K = 16 * rnd.choice([1, 5, 8, 9, 26, 63, 64, 65, 104, 128, 129, 250])
+        nks = (K + 127) // 128
+        ks = rnd.choice([0, 0, 1, 2, min(nks, rnd.randint(1, 16))])
+        shapes.append((M, N, K, ks))
+    for M, N, K, ks in shapes:
+        a, w = make_operands(M, N, K, seed=M * 7 + N * 3 + K)
+        a8, ia, _ = fp8_ref.to_fp8(a)
+        w8, iw, _ = fp8_ref.to_fp8(w)
+        want = fp8_ref.scaled_mm_emulated(a8, w8, ia, iw)
+        ad, w8d, iwd = a.to(DEV), w8.to(DEV), iw.reshape(1).to(DEV)
+        bits = ops.amax_bits(ad)
+        got = ops.fp8_linear_small_m(ad, bits, w8d, iwd, ksplits=ks)
+        err = rel_l2(got.cpu(), want)
+        assert err <= 2e-3, (M, N, K, ks, err)
+        h2, am = ops.fp8_linear_small_m(ad, bits, w8d, iwd, relu2=True, ksplits=ks)
+        want_h2 = torch.relu(got).square()
+        assert torch.equal(h2, want_h2), (M, N, K, ks)
+        assert am.view(torch.float32).item() == want_h2.float().max().item(), (M, N, K, ks)
+
+
 def test_split_hand_off_never_reads_stale_partials(ops):
     """The split-K GEMM and the split attention pass partial results between workgroups through a scratch
     buffer that is reused by every call.  Alternate two different inputs many times: a stale partial from
