@@ -40,11 +40,15 @@
         if (rc__) return rc__; \
     } while (0)
 
-// Reading a shared prompt once for all rows pays from a few rows on, and for a layer whose visible keys are at least half shared ones
-// (a full-context layer for as long as the rows have decoded fewer tokens than the prompt holds; a windowed layer until its window
-// has moved halfway out of the prompt): the shared launch and the separate rotary launch cost what ~250 keys per row cost to stream
-#define NC_SHARED_MIN_ROWS 16
-#define NC_SHARED_MIN_KEYS 256
+// Reading a shared prompt once for all rows costs two more launches per layer (the stand-alone rotary kernel and the shared-keys kernel,
+// ~12-14 us together with the merge) and saves the per-row streaming of the shared keys the layer sees: rows x kv heads x keys x 512
+// bytes at ~6 TB/s.  It is taken when that is at least ~14 us: 164 000 (row, kv head, key) units -- 197 shared keys at 64 rows of 13
+// heads (a full-context layer always; a 512-key window until it has moved most of the way out of the prompt), 394 at 32 rows.
+// (and only for batches whose per-row launches never split a row's keys over workgroups, rows x kv heads >= 512: below that the
+// per-row launch is short and the three launches of the shared form were measured 2-8 % slower per step)
+#define NC_SHARED_MIN_ROW_HEADS 512
+#define NC_SHARED_MIN_KEYS 128
+#define NC_SHARED_MIN_UNITS 164000L
 
 namespace {
 struct Carver {
@@ -137,7 +141,7 @@ Workspace carve(const nc_model_desc* m, int B, int T, void* base) {
     w.attn_parts = c.take<uint8_t>(w.attn_part_bytes);
     // partial results of the shared first part of the cache (rows that begin with one replicated prompt): whatever the shared length
     // turns out to be, the launch cuts it into at most as many chunks as a whole cache row would get
-    w.shared_part_bytes = (T == 1 && B >= NC_SHARED_MIN_ROWS) ? nc_attn_shared_partial_bytes(B, m->n_head, m->n_kv_head, 1 << 20) : 0;
+    w.shared_part_bytes = (T == 1 && (long)B * m->n_kv_head >= NC_SHARED_MIN_ROW_HEADS) ? nc_attn_shared_partial_bytes(B, m->n_head, m->n_kv_head, 1 << 20) : 0;
     w.shared_parts = c.take<uint8_t>(w.shared_part_bytes);
     w.total = (c.off + 255) & ~(size_t)255;
     return w;
@@ -313,10 +317,10 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
         bf16_t* vc = kv->v_cache + (size_t)i * layer_elems;
         // rows that begin with one replicated prompt: a layer that sees a long stretch of it reads that stretch once for all rows
         bool shared_done = false;
-        if (T == 1 && B >= NC_SHARED_MIN_ROWS && kv->shared_prefix > 0 && kv->uniform_pos >= kv->shared_prefix && w.shared_parts) {
+        if (T == 1 && (long)B * Hkv >= NC_SHARED_MIN_ROW_HEADS && kv->shared_prefix > 0 && kv->uniform_pos >= kv->shared_prefix && w.shared_parts) {
             const int first_visible = ly.window_left < 0 ? 0 : (kv->uniform_pos - ly.window_left > 0 ? kv->uniform_pos - ly.window_left : 0);
-            const int shared_visible = kv->shared_prefix - first_visible, own_visible = kv->uniform_pos + 1 - kv->shared_prefix;
-            if (shared_visible >= NC_SHARED_MIN_KEYS && shared_visible >= own_visible && kv->shared_prefix < kv->max_seq_len) {
+            const int shared_visible = kv->shared_prefix - first_visible;
+            if (shared_visible >= NC_SHARED_MIN_KEYS && (long)shared_visible * B * Hkv >= NC_SHARED_MIN_UNITS && kv->shared_prefix < kv->max_seq_len) {
                 if (qsrc.parts)
                     TRY(nc_launch_qkv_rope_append_p(qsrc, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
                                                     kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));

@@ -68,14 +68,15 @@ def static_card(model, prompt_len, decode_tokens, total_vram, peak_bw):
     }
 
 
-def bench_generate(engine, prompt_tokens, batch_size, decode_tokens, temperature):
+def bench_generate(engine, prompt_tokens, batch_size, decode_tokens, temperature, share_prompt_reads=False):
     """One timed generation with the reference's protocol: the first next() is the time to first token (batch-1
     prefill, cache replication, first sample, first forward), every further next() is one decode step, each
     followed by a device synchronisation."""
     device = engine.model.get_device()
     torch.cuda.reset_peak_memory_stats(device)
     torch.cuda.synchronize(device)
-    gen = engine.generate(prompt_tokens, num_samples=batch_size, max_tokens=decode_tokens, temperature=temperature)
+    gen = engine.generate(prompt_tokens, num_samples=batch_size, max_tokens=decode_tokens, temperature=temperature,
+                          share_prompt_reads=share_prompt_reads)
     t0 = time.perf_counter()
     next(gen)
     torch.cuda.synchronize(device)
@@ -104,6 +105,8 @@ def main(argv=None):
     ap.add_argument("--batch-sizes", type=str, default="1,8,32,128")
     ap.add_argument("-t", "--temperature", type=float, default=0.0)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--share-prompt-reads", action="store_true",
+                    help="not in the reference: read the prompt that Engine.generate replicates into every row once for all rows")
     args = ap.parse_args(argv)
     assert torch.cuda.is_available(), "infer_bench needs the GPU"
     device = torch.device("cuda:0")
@@ -149,7 +152,8 @@ def main(argv=None):
         "source": source, "step": step, "model_config": model_config, "gpu": device_name,
         "peak_bandwidth_bytes_per_sec": peak_bw, "total_vram_bytes": total_vram, **card,
         "peak_flops_per_sec": peak_flops, "peak_fp8_flops_per_sec": PEAK_FP8_FLOPS,
-        "prompt_tokens": prompt_len, "decode_tokens": args.decode_tokens, "temperature": args.temperature, "sweep": [],
+        "prompt_tokens": prompt_len, "decode_tokens": args.decode_tokens, "temperature": args.temperature,
+        "share_prompt_reads": bool(args.share_prompt_reads), "sweep": [],
     }
 
     bench_generate(engine, prompt, 1, 2, args.temperature)                  # warm-up (weight plan, workspaces)
@@ -163,8 +167,8 @@ def main(argv=None):
     print(header)
     print("-" * len(header))
     for batch_size in [int(b) for b in args.batch_sizes.split(",")]:
-        bench_generate(engine, prompt, batch_size, 8, args.temperature)     # warm-up at this batch size
-        res = bench_generate(engine, prompt, batch_size, args.decode_tokens, args.temperature)
+        bench_generate(engine, prompt, batch_size, 8, args.temperature, args.share_prompt_reads)     # warm-up at this batch size
+        res = bench_generate(engine, prompt, batch_size, args.decode_tokens, args.temperature, args.share_prompt_reads)
         steps = res["step_times"]
         if not steps:
             print(f"{batch_size:>6}  no decode steps")
