@@ -202,8 +202,8 @@ int nc_qkv_rope_append_attention(const uint16_t* qkv, int ld_qkv, const uint16_t
  * nc_decode_attention to rounding (sums in another order; the shared part's weights pass through bf16 like in the
  * many-queries kernel), the cache bytes read drop from B x n_keys to shared + B x own.  CONTRACT: rows [0, shared_len) of
  * every batch row hold identical bytes, cache_seqlens[b] is the same for all b and >= shared_len.  workspace:
- * nc_decode_attention_shared_workspace_bytes() bytes, 16-byte aligned.  Shapes with too few rows for the per-row kernel to run
- * unsplit are refused (-1): use nc_decode_attention.  No counterpart in the reference's attention seam. */
+ * nc_decode_attention_shared_workspace_bytes() bytes, 16-byte aligned.  Any batch size (each row's own tail is read by one workgroup
+ * per kv head or head pair).  No counterpart in the reference's attention seam. */
 size_t nc_decode_attention_shared_workspace_bytes(int B, int H, int Hkv, int shared_len);
 int nc_decode_attention_shared(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int32_t* cache_seqlens,
                                int shared_len, int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax,

@@ -181,10 +181,8 @@ int nc_decode_attention_shared(const uint16_t* q, const uint16_t* k_cache, const
                                int shared_len, int window_left, uint16_t* out, int B, int H, int Hkv, int Tmax, int seqlens_include_new,
                                void* workspace, size_t workspace_bytes, uint32_t* amax_ws, nc_stream_t stream) {
     NC_CHECK_ARG(q && k_cache && v_cache && cache_seqlens && out && workspace, "decode_attention_shared: null pointer");
-    const int rc = nc_launch_attention_shared(q, k_cache, v_cache, cache_seqlens, shared_len, window_left, out, B, H, Hkv, Tmax,
-                                              seqlens_include_new, workspace, workspace_bytes, amax_ws, (hipStream_t)stream);
-    if (rc == -3) NC_FAIL(-1, "decode_attention_shared: this shape splits the keys of a row over workgroups (too few rows); use nc_decode_attention");
-    return rc;
+    return nc_launch_attention_shared(q, k_cache, v_cache, cache_seqlens, shared_len, window_left, out, B, H, Hkv, Tmax, seqlens_include_new,
+                                      workspace, workspace_bytes, amax_ws, (hipStream_t)stream);
 }
 
 static void split_attention_workspace(void* workspace, size_t workspace_bytes, int B, int T, int H, uint32_t** counters, void** parts,

@@ -516,22 +516,21 @@ int nc_launch_attention_fused(NcRopeSrc rope, bf16_t* k_cache, bf16_t* v_cache, 
 // Decode attention for rows that share their first `shared_len` cached tokens (one prompt replicated to every row,
 // nanochat/engine.py:198-214) and sit at the same position: the shared keys are read once for all rows on the matrix cores
 // (attn_shared_prefix_kernel, from row 0 of the cache), the per-row kernel streams only each row's own tail [shared_len, p] and merges
-// the two parts.  One new token per row, already appended.  shared_parts: nc_attn_shared_partial_bytes() bytes.  Returns -3 without
-// launching anything when the shape does not take this path (the per-row kernel would split its keys over workgroups): the caller
-// then uses the plain entry.
+// the two parts.  One new token per row, already appended.  shared_parts: nc_attn_shared_partial_bytes() bytes.  The per-row launch
+// takes one workgroup per (row, kv head) whatever the batch: a row's own tail is short, and the merge of the shared part belongs to the
+// workgroup that has the row.
 int nc_launch_attention_shared(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens, int shared_len,
                                int window_left, bf16_t* out, int B, int H, int Hkv, int Tmax, int seqlens_include_new, void* shared_parts,
                                size_t shared_part_bytes, uint32_t* amax_ws, hipStream_t s) {
     NC_CHECK_ARG(B > 0 && H > 0 && Hkv > 0 && Tmax > 0 && H % Hkv == 0, "decode_attention_shared: bad shape");
     NC_CHECK_ARG(shared_len > 0 && shared_len < Tmax, "decode_attention_shared: shared length %d outside (0, %d)", shared_len, Tmax);
-    const int max_keys = (window_left >= 0 && window_left + 1 < Tmax) ? window_left + 1 : Tmax;
-    if (pick_splits(B, 1, Hkv, max_keys) != 1) return -3;       // (what the per-row launch below will decide for itself)
     int nchunks = 0;
     int rc = nc_launch_attention_shared_prefix(q, k_cache, v_cache, cache_seqlens, shared_len, window_left, seqlens_include_new,
                                                (float*)shared_parts, shared_part_bytes, B, H, Hkv, Tmax, &nchunks, s);
     if (rc) return rc;
+    // (one split whatever the batch: a row's own tail is short, and the merge of the shared part belongs to the workgroup that has the row)
     return launch_attention_impl(q, nullptr, 0, const_cast<bf16_t*>(k_cache), const_cast<bf16_t*>(v_cache), cache_seqlens, window_left, out, B, 1,
-                                 H, Hkv, Tmax, seqlens_include_new, nullptr, nullptr, 0, amax_ws, 0, 1, s, shared_len, (const float*)shared_parts,
+                                 H, Hkv, Tmax, seqlens_include_new, nullptr, nullptr, 0, amax_ws, 1, 1, s, shared_len, (const float*)shared_parts,
                                  nchunks);
 }
 

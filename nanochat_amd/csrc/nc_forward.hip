@@ -44,9 +44,8 @@
 // ~12-14 us together with the merge) and saves the per-row streaming of the shared keys the layer sees: rows x kv heads x keys x 512
 // bytes at ~6 TB/s.  It is taken when that is at least ~14 us: 164 000 (row, kv head, key) units -- 197 shared keys at 64 rows of 13
 // heads (a full-context layer always; a 512-key window until it has moved most of the way out of the prompt), 394 at 32 rows.
-// (and only for batches whose per-row launches never split a row's keys over workgroups, rows x kv heads >= 512: below that the
-// per-row launch is short and the three launches of the shared form were measured 2-8 % slower per step)
-#define NC_SHARED_MIN_ROW_HEADS 512
+// (measured through the harness at d26, 1792-token prompt: 8 / 16 / 32 rows 1.38 / 1.58 / 2.14 -> 1.30 / 1.43 / 1.79 ms per step)
+#define NC_SHARED_MIN_ROW_HEADS 64
 #define NC_SHARED_MIN_KEYS 128
 #define NC_SHARED_MIN_UNITS 164000L
 
@@ -327,12 +326,8 @@ static int gpt_forward_impl(const nc_model_desc* m, const nc_cache_desc* kv, con
                 else
                     TRY(nc_launch_qkv_rope_append(w.qkv, qkv_w, w.xn, E, idx, ly.ve_table, ly.ve_gate_w, m->cos, m->sin, m->rope_len,
                                                   kv->cache_seqlens, kc, vc, w.qh, B, T, H, Hkv, kv->max_seq_len, m->padded_vocab, s));
-                int rc = nc_launch_attention_shared(w.qh, kc, vc, kv->cache_seqlens, kv->shared_prefix, ly.window_left, w.y, B, H, Hkv,
-                                                    kv->max_seq_len, 0, w.shared_parts, w.shared_part_bytes, w.site(site), s);
-                if (rc == -3)      // (the per-row kernel would split its keys: the plain entry, on the q and the cache rows just written)
-                    rc = nc_launch_attention(w.qh, kc, vc, kv->cache_seqlens, ly.window_left, w.y, B, T, H, Hkv, kv->max_seq_len, 0,
-                                             w.attn_counters, w.attn_parts, w.attn_part_bytes, w.site(site), 0, 1, s);
-                if (rc) return rc;
+                TRY(nc_launch_attention_shared(w.qh, kc, vc, kv->cache_seqlens, kv->shared_prefix, ly.window_left, w.y, B, H, Hkv,
+                                               kv->max_seq_len, 0, w.shared_parts, w.shared_part_bytes, w.site(site), s));
                 shared_done = true;
             }
         }

@@ -199,6 +199,9 @@ SHARED_SHAPES = [
     (128, 16, 4, 1024, 700, 830, -1),        # four query heads per kv head (the d32 width), a shared length that is no multiple of 64
     (96, 12, 6, 512, 130, 140, -1),          # two query heads per kv head, one chunk
     (70, 8, 8, 640, 600, 601, 300),          # rows that do not fill the last block of 32
+    (8, 13, 13, 2048, 1792, 1900, -1),       # few rows: the plain per-row launch would split a row's keys, this one does not
+    (16, 13, 13, 2048, 1792, 2047, 512),
+    (3, 4, 2, 512, 300, 310, -1),
 ]
 
 
