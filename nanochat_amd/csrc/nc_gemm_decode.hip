@@ -19,12 +19,13 @@
 //                               the whole range asked for through buffer descriptors before the first wait
 //                               (9.0 / 6.7 / 9.9 / 9.7 us -> 8.2 / 5.0 / 8.3 / 8.5 us for the four linears of a
 //                               d26 layer at 64 rows; about 3.4 us of each is the weight fetch itself, 2.3 us the
-//                               launch, 1.5 us the partial sums leaving the chip);
+//                               launch, 1.5 us the partial sums leaving the chip); 65 .. 128 rows take eight
+//                               waves, two halves of 64 rows against the same weight columns (d26 at 128 rows
+//                               with the prompt read once: 39.7 k -> 43.1 k tokens/s);
 //   gemm_decode_full_kernel     17 .. 64 rows, K <= 2048, relu^2 epilogue: unsplit, 32 columns per workgroup,
 //                               the result leaves finished and the MLP activation needs no pass of its own
 //                               (10.6 us against 8.3 + 4.4 us for the split linear and its finishing pass);
-//   gemm_decode_kernel          everything else (longer K ranges walked in 512-wide chunks, more than 64 rows,
-//                               activation rows made inside the kernel from a recipe).
+//   gemm_decode_kernel          everything else (longer K ranges walked in 512-wide chunks).
 //
 // Epilogues: 0 bf16;  1 fp32 softcap*tanh(bf16(v)/softcap) (lm_head, nanochat/gpt.py:512-515);
 //            2 bf16 relu(bf16(v))^2 plus atomic amax of the result (MLP activation, gpt.py:139).
@@ -434,13 +435,16 @@ __global__ __launch_bounds__(256) void gemm_decode_kernel(DecodeGemmArgs g) {
 typedef int dg_v4i __attribute__((ext_vector_type(4)));
 // A_MODE as in gemm_decode_kernel: 0 e4m3 activations, 1 bf16 + the producer's amax, 2 / 3 rows made here from a recipe of kind 1 / 2
 // (one or two rows; the weight rows are on their way while the rows are made).
-template <int MB, int A_MODE, int NSET>
-__global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs g) {
+// WR: 1 = four waves, up to 64 rows; 2 = eight waves for 65 .. 128 rows, waves 4 .. 7 multiplying rows 64 .. 127 with the same columns.
+// The occupancy is pinned so that the scheduler keeps every load of the range in flight instead of trading them for registers.
+template <int MB, int A_MODE, int NSET, int WR = 1>
+__global__ __launch_bounds__(256 * WR) __attribute__((amdgpu_waves_per_eu(WR, 2))) void gemm_decode_onetrip_kernel(DecodeGemmArgs g) {
     constexpr bool A_BF16 = A_MODE != 0;
-    constexpr int ROWS = MB * 16;
-    constexpr int A_CH = ROWS * 32 / 256;          // 16-byte e4m3 chunks per thread per 512-wide half of the range
+    constexpr int ROWS = MB * 16 * WR, NT = 256 * WR;
+    constexpr int A_CH = ROWS * 32 / NT;           // 16-byte e4m3 chunks per thread per 512-wide half of the range
     constexpr int A_LD = A_BF16 ? 2 : 1;
-    __shared__ __align__(16) uint8_t lds[NSET][ROWS * 512];
+    extern __shared__ __align__(16) uint8_t lds_raw[];             // NSET panels of ROWS x 512 bytes
+    uint8_t (*lds)[ROWS * 512] = (uint8_t (*)[ROWS * 512])lds_raw;
     __shared__ float red[8];
     __shared__ __align__(16) bf16_t rowbuf[A_MODE == 2 ? NC_RECIPE_MAX_ROWS * 2048 : (A_MODE == 3 ? NC_RECIPE_MAX_ROWS * NC_RECIPE_MAX_K : 8)];
 
@@ -450,7 +454,8 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
     const int frow = lane & 15, kb = lane >> 4;
     const int split = blockIdx.y;
     const int M = g.M, N = g.N, K = g.K;
-    const int n0 = blockIdx.x * 64 + wave * 16;
+    const int n0 = blockIdx.x * 64 + (wave & 3) * 16;
+    const int rbase = (wave >> 2) * MB * 16;                       // first row this wave multiplies
     const int brow = n0 + frow;
 
     const int nksteps = (K + 127) >> 7;
@@ -477,7 +482,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
         for (int set = 0; set < NSET; set++)
 #pragma unroll
             for (int c = 0; c < A_CH; c++) {
-                const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+                const int id = tid + c * NT, row = id >> 5, ch = id & 31;
                 const int gk = kbase + set * 512 + ch * 16;
                 const uint32_t vo = (row < M && gk < k_hi) ? ((uint32_t)row * (uint32_t)K + (uint32_t)gk) * (A_BF16 ? 2u : 1u) : NC_DG_OOB;
 #pragma unroll
@@ -511,7 +516,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
         for (int set = 0; set < NSET; set++)
 #pragma unroll
             for (int c = 0; c < A_CH; c++) {
-                const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+                const int id = tid + c * NT, row = id >> 5, ch = id & 31;
                 const int gk = kbase + set * 512 + ch * 16;
                 const bool ok = row < M && gk < k_hi;
                 const dg_v4i* p = (const dg_v4i*)(rowbuf + (ok ? (size_t)row * K + gk : 0));
@@ -524,7 +529,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
     for (int set = 0; set < NSET; set++)
 #pragma unroll
         for (int c = 0; c < A_CH; c++) {
-            const int id = tid + c * 256, row = id >> 5, ch = id & 31;
+            const int id = tid + c * NT, row = id >> 5, ch = id & 31;
             dg_v4i v;
             if (A_BF16) {
                 const uint32_t w[8] = {(uint32_t)ra[set][c][0][0], (uint32_t)ra[set][c][0][1], (uint32_t)ra[set][c][0][2], (uint32_t)ra[set][c][0][3],
@@ -555,7 +560,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
                 const int kk = (2 * pr + q) & 3;
 #pragma unroll
                 for (int i = 0; i < MB; i++) {
-                    const int row = i * 16 + frow;
+                    const int row = rbase + i * 16 + frow;
                     const int c0 = kk * 8 + kb;
                     alo[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + ((c0 ^ (row & 15)) << 4)]);
                     ahi[q][i] = *(const dg_v4i*)(&lds[pr >> 1][row * 512 + (((c0 + 4) ^ (row & 15)) << 4)]);
@@ -584,7 +589,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
         // split-K: the raw partial tile; the consumer adds the splits
 #pragma unroll
         for (int i = 0; i < MB; i++) {
-            const int m = i * 16 + frow;
+            const int m = rbase + i * 16 + frow;
             if (m < M && n < N)
                 *(float4*)(g.partial_out + ((size_t)split * M + m) * N + n) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
         }
@@ -594,7 +599,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
     float am = 0.f;
 #pragma unroll
     for (int i = 0; i < MB; i++) {
-        const int m = i * 16 + frow;
+        const int m = rbase + i * 16 + frow;
         if (m < M && n < N) {
             const float inv_b = dg_seg_scale(g, n);
             float v[4];
@@ -625,6 +630,7 @@ __global__ __launch_bounds__(256) void gemm_decode_onetrip_kernel(DecodeGemmArgs
         __syncthreads();
         if (tid == 0) {
             am = amax_join(amax_join(red[0], red[1]), amax_join(red[2], red[3]));
+            if (WR == 2) am = amax_join(am, amax_join(amax_join(red[4], red[5]), amax_join(red[6], red[7])));
             amax_publish(g.out_amax, am);
         }
     }
@@ -1166,7 +1172,7 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
     // block (batch 8: 1.50 -> 1.35 ms per d26 step with 16 rows instead of 64)
     const int MB = (made || M <= 16) ? 1 : (M <= 32 ? 2 : (M <= 48 ? 3 : (M <= 64 ? 4 : 8)));
     const bool wide = ksplits == 1 && !full && dg_wide_form(M, N, K, made);
-    const bool onetrip = MB <= 4 && kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
+    const bool onetrip = kps <= 8 && (int64_t)N * K < ((int64_t)1 << 31);
     // the one-trip, unsplit and wide forms hand their event pair to the launch itself when the profiler is on (the kernel's own begin and end,
     // no marker packets around it); the chunk-walking kernel keeps the bracketing pair
     const bool own_events = wide || full || onetrip;
@@ -1195,12 +1201,29 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
         return 0;
     }
     dim3 grid(nblk, ksplits), block(256);
-#define OT_LAUNCH(MB_, MODE_)                                                                                          \
-    do {                                                                                                               \
-        if (kps <= 4 && ev0) hipExtLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 1>), grid, block, 0, s, ev0, ev1, 0, g); \
-        else if (kps <= 4) hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 1>), grid, block, 0, s, g);      \
-        else if (ev0) hipExtLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 2>), grid, block, 0, s, ev0, ev1, 0, g); \
-        else hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, 2>), grid, block, 0, s, g);                   \
+#define OT_LAUNCH_N(MB_, MODE_, NSET_, WR_)                                                                                    \
+    do {                                                                                                                       \
+        constexpr int lds_bytes__ = NSET_ * MB_ * 16 * WR_ * 512;                                                              \
+        if (lds_bytes__ > 65536) {                                                                                             \
+            static bool reserved__[64];                                                                                        \
+            int dev__ = 0;                                                                                                     \
+            (void)hipGetDevice(&dev__);                                                                                        \
+            if (dev__ < 0 || dev__ >= 64 || !reserved__[dev__]) {                                                              \
+                const hipError_t e__ = hipFuncSetAttribute((const void*)gemm_decode_onetrip_kernel<MB_, MODE_, NSET_, WR_>,    \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes__);           \
+                if (e__ != hipSuccess) NC_FAIL(-2, "fp8_gemm(decode): cannot reserve %d bytes of LDS: %s", lds_bytes__, hipGetErrorString(e__)); \
+                if (dev__ >= 0 && dev__ < 64) reserved__[dev__] = true;                                                        \
+            }                                                                                                                  \
+        }                                                                                                                      \
+        if (ev0)                                                                                                               \
+            hipExtLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, NSET_, WR_>), grid, dim3(256 * WR_), lds_bytes__, s, ev0, ev1, 0, g); \
+        else                                                                                                                   \
+            hipLaunchKernelGGL((gemm_decode_onetrip_kernel<MB_, MODE_, NSET_, WR_>), grid, dim3(256 * WR_), lds_bytes__, s, g); \
+    } while (0)
+#define OT_LAUNCH(MB_, MODE_)                       \
+    do {                                            \
+        if (kps <= 4) OT_LAUNCH_N(MB_, MODE_, 1, 1); \
+        else OT_LAUNCH_N(MB_, MODE_, 2, 1);         \
     } while (0)
     if (onetrip) {
         if (made) {
@@ -1215,9 +1238,18 @@ int nc_launch_gemm_decode(const void* a, int a_is_bf16, const uint32_t* a_amax, 
         } else if (MB == 3) {
             if (a_is_bf16) OT_LAUNCH(3, 1);
             else OT_LAUNCH(3, 0);
-        } else {
+        } else if (MB == 4) {
             if (a_is_bf16) OT_LAUNCH(4, 1);
             else OT_LAUNCH(4, 0);
+        } else {
+            // 65 .. 128 rows: eight waves, two row halves of 64
+            if (kps <= 4) {
+                if (a_is_bf16) OT_LAUNCH_N(4, 1, 1, 2);
+                else OT_LAUNCH_N(4, 0, 1, 2);
+            } else {
+                if (a_is_bf16) OT_LAUNCH_N(4, 1, 2, 2);
+                else OT_LAUNCH_N(4, 0, 2, 2);
+            }
         }
     } else if (MB == 1) {
         if (made && recipe->kind == 1) hipLaunchKernelGGL((gemm_decode_kernel<1, 2>), grid, block, 0, s, g);

@@ -394,7 +394,9 @@ def test_fused_small_m_linear(ops, M, N, K, ksplits):
 @pytest.mark.parametrize("M,N,K,forms", [(64, 6656, 1664, (0, 1, 2, 4)),      # unsplit (32 columns per workgroup) / chunk-walking / one trip
                                          (64, 4992, 1664, (0, 1, 3)), (64, 1664, 6656, (0, 1, 13)), (64, 1664, 1664, (0, 1, 7)),
                                          (64, 32768, 1664, (0, 2, 4)),           # wide unsplit form / one trip
-                                         (40, 6656, 1280, (0, 2, 5))])
+                                         (40, 6656, 1280, (0, 2, 5)),
+                                         (128, 6656, 1664, (0, 1, 2, 4)), (100, 1664, 6656, (0, 1, 7, 13)),   # two row halves per workgroup
+                                         (65, 4992, 1664, (0, 1, 3))])
 def test_decode_linear_forms_agree_bit_for_bit(ops, M, N, K, forms):
     """The small-M linear has several kernels (one trip per split, unsplit with the activation in the GEMM, wide unsplit, chunk-walking);
     which one runs depends on the shape and on the split count asked for.  On the same operands they must give the same bf16 bits --
