@@ -261,8 +261,17 @@ __device__ __forceinline__ void bl_epilogue(v4f (&acc)[BM / WGM / 16][BN / WGN /
             }
         }
         if (relu2) {
+            // one publication per workgroup: the waves meet once more and the first thread joins their maxima
+            __shared__ float wave_am[WGM * WGN];
             am = wave_amax(am);
-            if (lane == 0) amax_publish(ep.out_amax, am);
+            if (lane == 0) wave_am[wave] = am;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                float t = wave_am[0];
+#pragma unroll
+                for (int w = 1; w < WGM * WGN; w++) t = amax_join(t, wave_am[w]);
+                amax_publish(ep.out_amax, t);
+            }
         }
     } else {
 #pragma unroll
@@ -678,6 +687,168 @@ __global__ __launch_bounds__(512) void gemm_dl_kernel(const uint8_t* __restrict_
     bl_epilogue<256, 256, 4, 2, RELU2 ? 2 : 0>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same tile-by-tile kernel with a narrower tile: 256 rows x 32 NJ columns (NJ = 4 .. 7 blocks of 16 columns per wave).  A launch of
+// one round -- a prompt of one to two thousand rows -- lasts as long as one tile, whatever the number of CUs that got one: 1792 x 4992
+// is 140 tiles of 256 x 256 on 256 CUs, but 224 tiles of 256 x 160, each 5/8 of the matrix work.  The launch picks NJ (dl_pick_nj).
+// A wave's B pieces beyond the tile's 32 NJ rows are not loaded (the test is uniform per wave), the stage is 256 + 32 NJ rows.
+template <int NJ, int A_FMT = 0, typename F = DlNothing>
+__device__ __forceinline__ void dln_compute(v4f (&acc)[4][NJ], const uint8_t* st, const DlGeom& g, F&& behind_first_reads = F()) {
+    const uint8_t* a = st + g.wm * 64 * 128;
+    const uint8_t* b = st + 256 * 128 + g.wn * (16 * NJ) * 128;
+    v8i af[4], bf[2];
+    bf[0] = dl_frag(b, g);
+#pragma unroll
+    for (int i = 0; i < 4; i++) af[i] = dl_frag(a + i * 2048, g);
+    behind_first_reads();
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        if (j + 1 < NJ) bf[(j + 1) & 1] = dl_frag(b + (j + 1) * 2048, g);    // one group ahead of its use
+#pragma unroll
+        for (int i = 0; i < 4; i++) mfma_f8_acc_ordered<A_FMT>(acc[i][j], bf[j & 1], af[i]);
+    }
+}
+
+// Epilogue for a wave block of 64 x 16 NJ outputs, bf16 (RELU2: relu(v)^2 and its maximum): the block is parked in the wave's own
+// LDS region (rows of 32 NJ + 16 bytes) and leaves as a linear sequence of 16-byte pieces, so a store instruction writes runs of
+// 32 NJ contiguous bytes per row.
+template <int NJ, bool RELU2>
+__device__ __forceinline__ void dln_epilogue(v4f (&acc)[4][NJ], uint8_t* lds, const EpilogueArgs& ep, float inv_a, const float (&sc)[4],
+                                             const DlGeom& g, int m0, int n0, int M, int N) {
+    constexpr int WCOLS = 16 * NJ, ROWB = WCOLS * 2, PITCH = ROWB + 16, LPR = ROWB / 16, PIECES = 64 * LPR;
+    static_assert(8 * 64 * PITCH <= 2 * (256 + 32 * NJ) * 128, "epilogue staging");
+    float am = 0.f;
+    __syncthreads();                                       // every wave is done with the operand tiles
+    uint8_t* reg = lds + g.wave * 64 * PITCH;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const int n = n0 + g.wn * WCOLS + j * 16 + 4 * g.kb;
+        float inv_b = sc[0];
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+            if (i + 1 < ep.segs.nseg && n >= ep.segs.end[i]) inv_b = sc[i + 1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = i * 16 + g.frow;
+            const v4f a4 = acc[i][j];
+            float o4[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                o4[r] = (a4[r] * inv_a) * inv_b;
+                if (RELU2) o4[r] = relu2_of(o4[r]);
+            }
+            *(uint2*)(reg + row * PITCH + j * 32 + g.kb * 8) = make_uint2(pack_bf16_hw(o4[0], o4[1]), pack_bf16_hw(o4[2], o4[3]));
+        }
+    }
+    // the region is private to the wave: its own LDS writes only have to land before its reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0xc07f);                    // lgkmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const bool vec16 = (ep.ldc % 8 == 0) && (((uintptr_t)ep.out & 15) == 0);
+#pragma unroll
+    for (int it = 0; it < PIECES / 64; it++) {
+        const int id = it * 64 + g.lane, row = id / LPR, c = id % LPR;
+        const int m = m0 + g.wm * 64 + row, n = n0 + g.wn * WCOLS + c * 8;
+        const uint4 v = *(const uint4*)(reg + row * PITCH + c * 16);
+        if (m >= M || n >= N) continue;
+        if (RELU2) am = amax_join(am, max_bf16x8(v, N - n));
+        bf16_t* o = (bf16_t*)ep.out + (size_t)m * ep.ldc + n;
+        if (n + 8 <= N) {
+            if (vec16) __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, (v4i*)o);
+            else {
+                *(uint2*)o = make_uint2(v.x, v.y);
+                *(uint2*)(o + 4) = make_uint2(v.z, v.w);
+            }
+        } else {
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            for (int r = 0; r < 8 && n + r < N; r++) o[r] = (bf16_t)(w[r >> 1] >> ((r & 1) * 16));
+        }
+    }
+    if (RELU2) {
+        __shared__ float wave_am[8];
+        am = wave_amax(am);
+        if (g.lane == 0) wave_am[g.wave] = am;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = wave_am[0];
+#pragma unroll
+            for (int w = 1; w < 8; w++) t = amax_join(t, wave_am[w]);
+            amax_publish(ep.out_amax, t);
+        }
+    }
+}
+
+// the operand loads of one K-step: `st` is the wave's first 1 KB piece of the stage (uniform: the LDS address of a load goes through M0)
+template <int NJ>
+__device__ __forceinline__ void dln_fetch(const uint8_t* A, int a_bytes, const uint8_t* B, int b_bytes, uint8_t* st, const uint32_t* vo_a,
+                                          const uint32_t* vo_b, int wave_s, int k_off) {
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, b_bytes, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < 4; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (lds_ptr_t)(st + i * 8192), 16, vo_a[i], k_off, 0, 0);
+#pragma unroll
+    for (int i = 0; i < (4 * NJ + 7) / 8; i++)
+        if (wave_s + 8 * i < 4 * NJ)                      // uniform per wave
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b, (lds_ptr_t)(st + 256 * 128 + i * 8192), 16, vo_b[i], k_off, 0, 0);
+}
+
+template <int NJ, bool RELU2>
+__global__ __launch_bounds__(512) void gemm_dln_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep, int M,
+                                                       int N, int K, int tiles_m, int tiles_n) {
+    constexpr int BN = 32 * NJ, STAGE = (256 + BN) * 128, B_PIECES = BN / 8, B_ROUNDS = (B_PIECES + 7) / 8;
+    extern __shared__ __align__(16) uint8_t lds[];
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * BN;
+    const DlGeom g = dl_geom();
+    const int wave_s = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    // piece i of this wave is the 1 KB block (wave + 8 i) of its operand's part of the stage: tile rows 8 wave + 64 i + sub
+    uint32_t vo_a[4], vo_b[B_ROUNDS];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int ra = m0 + 8 * g.wave + 64 * i + g.sub;
+        vo_a[i] = ra < M ? (uint32_t)ra * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+    }
+#pragma unroll
+    for (int i = 0; i < B_ROUNDS; i++) {
+        const int rb = n0 + 8 * g.wave + 64 * i + g.sub;
+        vo_b[i] = rb < N ? (uint32_t)rb * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+    }
+    const int ksteps = K / 128;
+
+    v4f acc[4][NJ];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto fetch = [&](int t, int buf) {
+        if (t < ksteps) dln_fetch<NJ>(A, M * K, B, N * K, lds + buf * STAGE + wave_s * 1024, vo_a, vo_b, wave_s, t * 128);
+    };
+    fetch(0, 0);
+    dl_step_barrier();
+    int kt = 0;
+    for (; kt + 1 < ksteps; kt += 2) {
+        dln_compute<NJ, 0>(acc, lds, g, [&] { fetch(kt + 1, 1); });
+        dl_step_barrier();
+        dln_compute<NJ, 0>(acc, lds + STAGE, g, [&] { fetch(kt + 2, 0); });
+        dl_step_barrier();
+    }
+    if (kt < ksteps) dln_compute<NJ, 0>(acc, lds, g);
+
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) asm volatile("" : "+a"(acc[i][j]));
+    const float inv_a = *ep.inv_a;
+    float sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
+    dln_epilogue<NJ, RELU2>(acc, lds, ep, inv_a, sc, g, m0, n0, M, N);
+}
+
 // Epilogue of the persistent kernel: the wave's 64 x (128 | 64) block leaves 16 rows at a time through a 4 KB LDS region of
 // its own (past the two operand stages, so the loads of the next tile keep landing meanwhile), every store instruction
 // writing whole 128-byte lines.
@@ -904,6 +1075,65 @@ static int launch_dl_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& 
     return 0;
 }
 
+// Blocks of 16 columns per wave (tile width 32 NJ, NJ = 4 .. 8) for a launch of 256-row tiles that is not persistent.  Measured at
+// K = 1664 a round of tiles lasts about 6 + NJ units (the A side of a K-step, the launch and the epilogue cost the same at any width:
+// 16.6 / 18.5 / 19.7 / 22.0 / 23.4 us for NJ = 4 .. 8 with 80 tiles) and up to a fifth longer when every CU has a tile (28.1 us with 240
+// tiles of 256 x 256).  The full width is kept unless a narrower tile is at least 8 % cheaper by that count:
+// 1792 x 4992: 140 tiles of 256 x 256, 24.1 us -> 224 of 256 x 160, 20.6 us; 1792 x 6656: 182 tiles, 25.4 -> 245 of 256 x 192, 22.2 us.
+static double dl_cost(int nj, int M, int N, int cus, long* tiles_out) {
+    const long tiles = (long)((M + 255) / 256) * ((N + 32 * nj - 1) / (32 * nj));
+    if (tiles_out) *tiles_out = tiles;
+    double cost = 0.0;
+    for (long left = tiles; left > 0; left -= cus) cost += (6.0 + nj) * (1.0 + 0.2 * (double)(left < cus ? left : cus) / cus);
+    return cost;
+}
+static int dl_pick_nj(int M, int N) {
+    const int cus = cu_count();
+    int best = 8;
+    const double full = dl_cost(8, M, N, cus, nullptr);
+    double best_cost = 0.92 * full;
+    for (int nj = 7; nj >= 4; nj--) {
+        const double c = dl_cost(nj, M, N, cus, nullptr);
+        if (c < best_cost) best = nj, best_cost = c;
+    }
+    return best;
+}
+// whether some narrower tile gives the launch one round with at least 150 of 256 CUs busy (then the 256-row tiles beat the 128 x 128
+// ones although the 256 x 256 tiles would leave most CUs idle: 1024 x 4992 x 1664 16.6 us against 18.4)
+static bool dl_narrow_fills(int M, int N) {
+    const int cus = cu_count();
+    for (int nj = 4; nj <= 7; nj++) {
+        long tiles;
+        (void)dl_cost(nj, M, N, cus, &tiles);
+        if (tiles <= cus && 256 * tiles >= 150L * cus) return true;
+    }
+    return false;
+}
+template <int NJ, bool RELU2>
+static int launch_dln_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 32 * NJ - 1) / (32 * NJ);
+    const size_t lds_bytes = 2 * (256 + 32 * NJ) * 128;
+    const void* fn = (const void*)gemm_dln_kernel<NJ, RELU2>;
+    hipError_t e = reserve_lds(fn, (int)lds_bytes);
+    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    hipLaunchKernelGGL((gemm_dln_kernel<NJ, RELU2>), dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    return 0;
+}
+// e4m3 operands, bf16 or relu^2 output, K a multiple of 128
+static int launch_dln(int nj, const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
+    NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
+    NC_CHECK_ARG(ep.out_kind != 1, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
+    const bool r2 = ep.out_kind == 2;
+    switch (nj) {
+        case 4: return r2 ? launch_dln_as<4, true>(a, b, ep, M, N, K, s) : launch_dln_as<4, false>(a, b, ep, M, N, K, s);
+        case 5: return r2 ? launch_dln_as<5, true>(a, b, ep, M, N, K, s) : launch_dln_as<5, false>(a, b, ep, M, N, K, s);
+        case 6: return r2 ? launch_dln_as<6, true>(a, b, ep, M, N, K, s) : launch_dln_as<6, false>(a, b, ep, M, N, K, s);
+        case 7: return r2 ? launch_dln_as<7, true>(a, b, ep, M, N, K, s) : launch_dln_as<7, false>(a, b, ep, M, N, K, s);
+    }
+    NC_FAIL(-1, "fp8_gemm: tile widths of 128, 160, 192 and 224 columns only, not %d", 32 * nj);
+}
+
 // the relu^2 epilogue is a variant of its own so that the plain kernels keep their register budget
 template <int A_FMT>
 static int launch_dl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
@@ -969,7 +1199,8 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     }
 
     // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256,
-    // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent, 10 / 11 buffer-load tiles 64x128 / 96x128
+    // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent, 10 / 11 buffer-load tiles 64x128 / 96x128,
+    // 12 .. 15 direct-to-LDS tiles of 256 x 128 / 160 / 192 / 224 tile by tile
     int which = force_kernel;
     if (which == 0) {
         if (M <= 128) which = 1;
@@ -979,12 +1210,16 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
             const long rounds = (t256 + cus - 1) / cus;
             const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-            if (out_kind != 1 && K % 128 == 0 && (8 * t256 >= 5 * cus || t128 > 2 * cus)) {
+            if (out_kind != 1 && K % 128 == 0 && (8 * t256 >= 5 * cus || t128 > 2 * cus || dl_narrow_fills(M, N))) {
                 // 256x256 tiles fed straight into LDS whenever they occupy at least 5/8 of the CUs, or the 128x128 tiles, four times
                 // as many, would not fit the chip in one round of two workgroups per CU (below that the small tiles fill the chip
                 // better: 18 us against 22 for 1280 x 4992 x 1664, but 25 against 22.4 for 1792 rows); from two rounds of tiles on,
                 // the persistent form, which neither rounds the last round up nor pays a prologue per tile
                 which = (t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8;
+                if (which == 8) {
+                    const int nj = dl_pick_nj(M, N);
+                    if (nj < 8) which = 8 + nj;           // 12 .. 15
+                }
             } else {
                 // 256x256 tiles move half the bytes per flop through L2 and LDS but run one workgroup per CU: take them
                 // when their count fills whole rounds of the CUs well, else the 128x128 tiles (two workgroups per CU)
@@ -1002,7 +1237,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         }
     }
     int rc = 0;
-    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 11, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 15, "fp8_gemm: unknown kernel selector %d", force_kernel);
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
@@ -1025,6 +1260,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     else if (which == 9) rc = launch_dl<0>(a, b, ep, M, N, K, true, s);
     else if (which == 10) rc = launch_bl<64, 128, 2, 2, true>(a, b, ep, M, N, K, s);
     else if (which == 11) rc = launch_bl<96, 128, 2, 2, true>(a, b, ep, M, N, K, s);
+    else if (which >= 12) rc = launch_dln(which - 8, a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");
