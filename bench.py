@@ -210,6 +210,35 @@ def mfma_ceiling(device, operands=None, iters=30000):
     return out
 
 
+def stream_read_floor(device, lib, sizes, reps=12):
+    """What a kernel that only reads reaches here (nc_probe_hbm_read: 16-byte non-temporal loads, nothing stored), at the byte counts of
+    the decode attention launches: microseconds per launch, launch and ramp included.  Every repetition reads another region of a
+    2 GiB buffer, so nothing comes from the 256 MB last-level cache.  Returns {bytes: mean microseconds of the kernel itself}."""
+    from nanochat_amd import _lib
+    total = 2 << 30
+    buf = torch.empty(total, dtype=torch.uint8, device=device)
+    buf.fill_(1)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for size in sizes:
+        size = min(int(size), total // 2) // 4096 * 4096
+        regions = max(2, total // size)
+        read = C.c_int64()
+        for r in range(reps + 2):
+            if r == 2:
+                torch.cuda.synchronize()
+                lib.nc_profile_enable(1)             # the launches from here on carry their own event pair (kernel begin / end)
+            off = (r % regions) * size
+            _lib.check(lib.nc_probe_hbm_read(C.c_void_p(buf.data_ptr() + off), size, C.byref(read), stream))
+        torch.cuda.synchronize()
+        ms, units, n = C.c_double(), C.c_double(), C.c_int64()
+        assert lib.nc_profile_read(5, C.byref(ms), C.byref(units), C.byref(n)) == 0 and n.value == reps
+        lib.nc_profile_enable(0)
+        out[read.value] = ms.value * 1e3 / reps
+    del buf
+    return out
+
+
 def cpu_gemm_baseline(cores, budget_s=6.0):
     """The reference's own CPU call for the isolated Float8Linear shapes (torch._scaled_mm on e4m3 operands, nanochat/fp8.py:143-153)
     and the fp8-emulated fp32 matmul beside it, on a row sample of M (the work is linear in M): GFLOP/s per shape."""
@@ -440,6 +469,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--no-pattern-l", action="store_true", help="skip the second run with every layer reading the whole context")
+    ap.add_argument("--no-stream-probe", action="store_true", help="skip the read-only kernel timed beside the attention launches")
     ap.add_argument("--no-shared-prompt", action="store_true", help="skip the extra run that reads the replicated prompt once for all rows")
     ap.add_argument("--library-gemm", action="store_true", help="also time torch._scaled_mm on the M=8192 GEMM operands")
     ap.add_argument("--profile-steps", type=int, default=16)
@@ -509,6 +539,21 @@ def main():
         "step_bytes": {"weights_e4m3": r["weight_bytes_step"], "kv_read": int(r["att_bytes_step"]),
                        "frac_hbm_peak_whole_step": round((r["weight_bytes_step"] + r["att_bytes_step"]) / (r["ms_per_step"] * 1e-3) / HBM_PEAK, 4)},
     }
+    if not args.no_stream_probe:
+        # beside the published peak: the duration of a read-only kernel over the bytes of a window layer's and a full-context layer's
+        # launch; between the two sizes the time is linear in the bytes, which prices the average launch (a mix of both kinds)
+        b_small = BATCH * 2 * model.config.n_kv_head * 128 * 2 * 513
+        b_large = BATCH * 2 * model.config.n_kv_head * 128 * 2 * CONTEXT
+        torch.cuda.empty_cache()
+        fl = stream_read_floor(device, lib, (b_small, b_large))
+        (s0, t0), (s1, t1) = sorted(fl.items())
+        per_byte = (t1 - t0) / (s1 - s0)
+        floor_us = t0 + (r["att_bytes_launch"] - s0) * per_byte
+        result["roofline"]["read_only_kernel"] = {
+            "bytes": [s0, s1], "us": [round(t0, 2), round(t1, 2)], "GBps": [round(s0 / t0 / 1e3, 1), round(s1 / t1 / 1e3, 1)],
+            "us_for_bytes_per_launch": round(floor_us, 2), "frac_of_it": round(floor_us / (r["att_avg_s"] * 1e6), 4),
+            "note": "nc_probe_hbm_read, launches that carry their own event pair like the attention launches, over regions of a 2 GiB buffer: what reading the same bytes once costs "
+                    "a kernel that does nothing else; frac_of_it = that time / avg_launch_us"}
     if args.window_pattern == "SSSL" and not args.no_pattern_l:
         # the same configuration with every layer reading the whole context (22.7 GB of KV per step at context 2048): the case
         # that is bound by KV reads alone; a shorter timed window, same prompt, same 256 new tokens

@@ -319,7 +319,7 @@ int nc_gpt_forward_tapped(const nc_model_desc* model /*host*/, const nc_cache_de
 
 /* ---- measurement aid (no counterpart in the reference) --------------------------------------
  * While enabled, every launch made by this library is bracketed by a HIP event pair on its stream.
- * Classes: 0 attention (partial + combine), 1 FP8 GEMM, 2 quantize/convert, 3 row kernels, 4 sampler.
+ * Classes: 0 attention (partial + combine), 1 FP8 GEMM, 2 quantize/convert, 3 row kernels, 4 sampler, 5 nc_probe_hbm_read.
  * `units` are the algorithmic bytes (classes 0,2,3,4) or flops (class 1) of the launches.  Not thread
  * safe; at most 16384 launches are recorded per enable. */
 int nc_profile_enable(int on);
@@ -336,6 +336,12 @@ int nc_profile_read_gemm(int N, int K, double* total_ms /*host*/, double* total_
  * 8 x uint64 or NULL): for workgroups 0..3, shader-clock ticks and 100 MHz ticks spent in the loop (their ratio x 0.1 = GHz). */
 int nc_probe_fp8_mfma_ceiling(const uint8_t* operands, int64_t operand_bytes, int iters, uint64_t* clocks_out,
                               double* flops_out /*host*/, nc_stream_t stream);
+
+/* What a kernel that does nothing but read reaches on this GPU's memory (no counterpart in the reference; measurement aid): one
+ * launch streams `bytes` of `src` (device, 16-byte aligned) once with 16-byte non-temporal loads and stores nothing.  Time it with
+ * events, or enable the profiler above and read class 5 (the kernel's own begin and end); over a buffer larger than the last-level cache its duration is the floor for any kernel that reads as many bytes once.
+ * *bytes_read_out (host): the bytes the launch reads (bytes rounded down to a multiple of 16 x the workgroup count). */
+int nc_probe_hbm_read(const void* src, int64_t bytes, int64_t* bytes_read_out /*host*/, nc_stream_t stream);
 
 #ifdef __cplusplus
 }

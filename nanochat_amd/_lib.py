@@ -17,7 +17,7 @@ EXPORTS = [
     "nc_gpt_workspace_bytes", "nc_gpt_forward", "nc_profile_enable", "nc_profile_read", "nc_profile_read_gemm",
     "nc_decode_attention_append", "nc_qkv_rope_append_attention", "nc_decode_attention_plan", "nc_gpt_forward_tapped",
     "nc_decode_attention_static", "nc_decode_attention_static_max_row_heads",
-    "nc_fp8_quantize_state_bytes", "nc_fp8_quantize_tensorwise_fused", "nc_fp8_quantize_tensorwise_fused_bounded", "nc_probe_fp8_mfma_ceiling", "nc_fp8_quantize_tensorwise_transposed",
+    "nc_fp8_quantize_state_bytes", "nc_fp8_quantize_tensorwise_fused", "nc_fp8_quantize_tensorwise_fused_bounded", "nc_probe_fp8_mfma_ceiling", "nc_probe_hbm_read", "nc_fp8_quantize_tensorwise_transposed",
     "nc_decode_attention_shared", "nc_decode_attention_shared_workspace_bytes",
 ]
 
@@ -90,6 +90,7 @@ def _bind(lib):
         "nc_profile_read": (i, [i, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
         "nc_profile_read_gemm": (i, [i, i, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
         "nc_probe_fp8_mfma_ceiling": (i, [p, i64, i, p, C.POINTER(C.c_double), p]),
+        "nc_probe_hbm_read": (i, [p, i64, C.POINTER(C.c_int64), p]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)     # AttributeError if the symbol is missing

@@ -3,6 +3,7 @@
 // taken from a fixed pool (the decode attention launch, whose duration the roofline figure is made of, gives its pair to the launch
 // itself instead, see nc_prof_take).  nc_profile_read() waits for the events and sums the elapsed times.
 #include "../../include/nanochat_amd.h"
+#include <hip/hip_ext.h>
 #include "nc_common.h"
 #include "nc_kernels.h"
 
@@ -130,6 +131,43 @@ int nc_probe_fp8_mfma_ceiling(const uint8_t* operands, int64_t operand_bytes, in
                        operands ? (int)(operand_bytes / 32) : 1, iters, (unsigned long long*)clocks_out, (float*)nullptr);
     NC_CHECK_LAUNCH("probe_fp8_mfma_ceiling");
     if (flops_out) *flops_out = (double)cus * 8.0 * 32.0 * (double)iters * 65536.0;     // 2 * 16 * 16 * 128 per instruction
+    return 0;
+}
+
+// ---- what a kernel that only reads reaches on this memory ---------------------------------------------------
+// Every workgroup streams a contiguous share of the buffer with 16-byte non-temporal loads, eight per thread in flight, and folds what
+// it read into one word that is never stored: the duration of a launch over a buffer larger than the last-level cache is the floor of
+// any kernel that has to read that many bytes once, launch and ramp included.
+typedef int probe_v4i __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void stream_read_kernel(const probe_v4i* __restrict__ src, long per_wg, int* __restrict__ sink) {
+    const probe_v4i* p = src + (long)blockIdx.x * per_wg;
+    probe_v4i acc = {0, 0, 0, 0};
+    long i = threadIdx.x;
+    for (; i + 7 * 256 < per_wg; i += 8 * 256) {
+        probe_v4i v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = __builtin_nontemporal_load(p + i + u * 256);
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc ^= v[u];
+    }
+    for (; i < per_wg; i += 256) acc ^= __builtin_nontemporal_load(p + i);
+    if (sink && (acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5eed1234 && per_wg < 0) sink[0] = 1;      // never true: keeps the loads alive
+}
+
+int nc_probe_hbm_read(const void* src, int64_t bytes, int64_t* bytes_read_out, nc_stream_t stream) {
+    NC_CHECK_ARG(src && ((uintptr_t)src & 15) == 0 && bytes >= 16, "probe_hbm_read: a 16-byte aligned buffer of at least 16 bytes");
+    const int grid = 8 * nc_cu_count();
+    const long per_wg = (long)(bytes / 16) / grid;
+    NC_CHECK_ARG(per_wg >= 1, "probe_hbm_read: at least %d bytes", 16 * grid);
+    // with the profiler on, the launch carries an event pair of class 5 itself: the kernel's own begin and end, as the attention launches do
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    if (nc_prof_take(5, (double)per_wg * grid * 16, 0, &ev0, &ev1))
+        hipExtLaunchKernelGGL(stream_read_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, ev0, ev1, 0, (const probe_v4i*)src, per_wg,
+                              (int*)nullptr);
+    else
+        hipLaunchKernelGGL(stream_read_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const probe_v4i*)src, per_wg, (int*)nullptr);
+    NC_CHECK_LAUNCH("probe_hbm_read");
+    if (bytes_read_out) *bytes_read_out = (int64_t)per_wg * grid * 16;
     return 0;
 }
 }

@@ -1046,3 +1046,36 @@ def test_sample_next_token_api_on_gpu(ops):
     assert all(a[i, 0] in top[i] for i in range(8))
     exp = sample_next_token(logits[:1].expand(8, -1), r1, 1.0, None)
     assert exp.shape == (8, 1)
+
+
+def test_measurement_probes_run_and_report_their_work(ops):
+    """The two measurement aids of the C-ABI: the read-only streaming kernel says how many bytes it read (the count it was given,
+    rounded down to whole 16-byte pieces per workgroup) and refuses a misaligned buffer; with the profiler on, its launch is a record
+    of class 5 with that byte count.  The matrix-pipe loop reports 2 * 16 * 16 * 128 flops per instruction issued."""
+    import ctypes as C
+    from nanochat_amd import _lib
+    say("measurement probes")
+    lib = _lib.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    buf = torch.ones(8 << 20, dtype=torch.uint8, device=DEV)
+    read = C.c_int64()
+    _lib.check(lib.nc_probe_hbm_read(C.c_void_p(buf.data_ptr()), buf.numel() - 100, C.byref(read), stream))
+    torch.cuda.synchronize()
+    assert 0 < read.value <= buf.numel() - 100 and buf.numel() - 100 - read.value < 16 * 8 * 1024 and read.value % 16 == 0
+    assert lib.nc_probe_hbm_read(C.c_void_p(buf.data_ptr() + 4), 1 << 20, C.byref(read), stream) != 0      # misaligned
+    assert lib.nc_probe_hbm_read(C.c_void_p(buf.data_ptr()), 64, C.byref(read), stream) != 0               # less than a piece per workgroup
+    lib.nc_profile_enable(1)
+    for _ in range(3):
+        _lib.check(lib.nc_probe_hbm_read(C.c_void_p(buf.data_ptr()), buf.numel(), C.byref(read), stream))
+    torch.cuda.synchronize()
+    ms, units, n = C.c_double(), C.c_double(), C.c_int64()
+    assert lib.nc_profile_read(5, C.byref(ms), C.byref(units), C.byref(n)) == 0
+    lib.nc_profile_enable(0)
+    assert n.value == 3 and units.value == 3.0 * read.value and ms.value > 0.0
+    flops = C.c_double()
+    clocks = torch.zeros(8, dtype=torch.int64, device=DEV)
+    _lib.check(lib.nc_probe_fp8_mfma_ceiling(None, 0, 100, C.c_void_p(clocks.data_ptr()), C.byref(flops), stream))
+    torch.cuda.synchronize()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert flops.value == cus * 8 * 32 * 100 * 65536.0
+    assert (clocks[::2] > 0).all()
