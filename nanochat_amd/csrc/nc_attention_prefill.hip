@@ -116,25 +116,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // staging: thread = (16-byte chunk ch of a key, key pair kp): keys 2kp, 2kp+1 of each 32-key sub-block
     const int ch = tid & 15, kp = tid >> 4;
-    const uint32_t key_stride = (uint32_t)Hkv * 128;
-    const bf16_t* kbase = k_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + ch * 8;
-    const bf16_t* vbase = v_cache + ((size_t)b * Tmax * Hkv + hk) * 128 + ch * 8;
+    // Keys and values come through buffer descriptors that end behind key k_hi of this row: a load past the workgroup's range returns
+    // zeros without a branch or a select, and the eight loads of a stage are eight instructions (plus one add each for the stage's
+    // offset; the range check looks at the vector offset only, so the stage cannot go into the scalar offset).
+    const uint32_t key_bytes = (uint32_t)Hkv * 256;
+    const uint32_t row_bytes = (uint32_t)(k_hi + 1) * key_bytes;
+    const __amdgpu_buffer_rsrc_t desc_k = __builtin_amdgcn_make_buffer_rsrc((void*)(k_cache + (size_t)b * Tmax * Hkv * 128), 0, row_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_v = __builtin_amdgcn_make_buffer_rsrc((void*)(v_cache + (size_t)b * Tmax * Hkv * 128), 0, row_bytes, 0x00020000);
+    const uint32_t lane_off = (uint32_t)(2 * kp) * key_bytes + (uint32_t)hk * 256 + (uint32_t)ch * 16;
+    typedef int pf_v4i __attribute__((ext_vector_type(4)));
     uint4 rk[2][2], rv[2][2];
-    // Load j (0..7) of the 64 keys from kb on: sub-block j / 4, key 2 kp + (j / 2) % 2 of it, K for even j and V for odd j.  Keys past
-    // the end of the workgroup's range come as zeros.  (The conditional form is deliberate: with unconditional loads of clamped
-    // addresses the compiler issues all eight in one burst, the wave then waits in the memory pipeline's queue instead of computing,
-    // and the kernel was measured at half the speed.)
-    auto fetch_one = [&](int kb, int j) {
-        const int sb = j >> 2, i = (j >> 1) & 1;
-        const int key = kb + 32 * sb + 2 * kp + i;
-        const bool ok = key <= k_hi;
-        const uint32_t off = (uint32_t)key * key_stride;
-        if (j & 1) rv[sb][i] = ok ? *(const uint4*)(vbase + off) : make_uint4(0, 0, 0, 0);
-        else rk[sb][i] = ok ? *(const uint4*)(kbase + off) : make_uint4(0, 0, 0, 0);
-    };
+    // the 64 keys from kb on: sub-block sb, key 2 kp + i of it
     auto fetch = [&](int kb) {
+        const uint32_t base = lane_off + (uint32_t)kb * key_bytes;
 #pragma unroll
-        for (int j = 0; j < 8; j++) fetch_one(kb, j);
+        for (int sb = 0; sb < 2; sb++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const uint32_t off = base + (uint32_t)(32 * sb + i) * key_bytes;
+                const pf_v4i kv = __builtin_amdgcn_raw_buffer_load_b128(desc_k, off, 0, 0);
+                const pf_v4i vv = __builtin_amdgcn_raw_buffer_load_b128(desc_v, off, 0, 0);
+                rk[sb][i] = make_uint4((uint32_t)kv[0], (uint32_t)kv[1], (uint32_t)kv[2], (uint32_t)kv[3]);
+                rv[sb][i] = make_uint4((uint32_t)vv[0], (uint32_t)vv[1], (uint32_t)vv[2], (uint32_t)vv[3]);
+            }
     };
     auto stage = [&]() {
 #pragma unroll
