@@ -792,7 +792,7 @@ __device__ __forceinline__ void dln_fetch(const uint8_t* A, int a_bytes, const u
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b, (lds_ptr_t)(st + 256 * 128 + i * 8192), 16, vo_b[i], k_off, 0, 0);
 }
 
-template <int NJ, bool RELU2>
+template <int NJ, bool RELU2, int A_FMT = 0>
 __global__ __launch_bounds__(512) void gemm_dln_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep, int M,
                                                        int N, int K, int tiles_m, int tiles_n) {
     constexpr int BN = 32 * NJ, STAGE = (256 + BN) * 128, B_PIECES = BN / 8, B_ROUNDS = (B_PIECES + 7) / 8;
@@ -830,12 +830,12 @@ __global__ __launch_bounds__(512) void gemm_dln_kernel(const uint8_t* __restrict
     dl_step_barrier();
     int kt = 0;
     for (; kt + 1 < ksteps; kt += 2) {
-        dln_compute<NJ, 0>(acc, lds, g, [&] { fetch(kt + 1, 1); });
+        dln_compute<NJ, A_FMT>(acc, lds, g, [&] { fetch(kt + 1, 1); });
         dl_step_barrier();
-        dln_compute<NJ, 0>(acc, lds + STAGE, g, [&] { fetch(kt + 2, 0); });
+        dln_compute<NJ, A_FMT>(acc, lds + STAGE, g, [&] { fetch(kt + 2, 0); });
         dl_step_barrier();
     }
-    if (kt < ksteps) dln_compute<NJ, 0>(acc, lds, g);
+    if (kt < ksteps) dln_compute<NJ, A_FMT>(acc, lds, g);
 
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
@@ -1109,27 +1109,32 @@ static bool dl_narrow_fills(int M, int N) {
     }
     return false;
 }
-template <int NJ, bool RELU2>
+template <int NJ, bool RELU2, int A_FMT>
 static int launch_dln_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 32 * NJ - 1) / (32 * NJ);
     const size_t lds_bytes = 2 * (256 + 32 * NJ) * 128;
-    const void* fn = (const void*)gemm_dln_kernel<NJ, RELU2>;
+    const void* fn = (const void*)gemm_dln_kernel<NJ, RELU2, A_FMT>;
     hipError_t e = reserve_lds(fn, (int)lds_bytes);
     if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-    hipLaunchKernelGGL((gemm_dln_kernel<NJ, RELU2>), dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL((gemm_dln_kernel<NJ, RELU2, A_FMT>), dim3(tiles_m * tiles_n), dim3(512), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
     return 0;
 }
-// e4m3 operands, bf16 or relu^2 output, K a multiple of 128
-static int launch_dln(int nj, const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+template <int NJ>
+static int launch_dln_nj(int a_fmt, const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    if (a_fmt == 1) return launch_dln_as<NJ, false, 1>(a, b, ep, M, N, K, s);
+    return ep.out_kind == 2 ? launch_dln_as<NJ, true, 0>(a, b, ep, M, N, K, s) : launch_dln_as<NJ, false, 0>(a, b, ep, M, N, K, s);
+}
+// bf16 or (e4m3 first operand only) relu^2 output, K a multiple of 128
+static int launch_dln(int nj, int a_fmt, const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
     NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
     NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
     NC_CHECK_ARG(ep.out_kind != 1, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
-    const bool r2 = ep.out_kind == 2;
+    NC_CHECK_ARG(a_fmt == 0 || ep.out_kind == 0, "fp8_gemm: the relu^2 epilogue goes with an e4m3 first operand");
     switch (nj) {
-        case 4: return r2 ? launch_dln_as<4, true>(a, b, ep, M, N, K, s) : launch_dln_as<4, false>(a, b, ep, M, N, K, s);
-        case 5: return r2 ? launch_dln_as<5, true>(a, b, ep, M, N, K, s) : launch_dln_as<5, false>(a, b, ep, M, N, K, s);
-        case 6: return r2 ? launch_dln_as<6, true>(a, b, ep, M, N, K, s) : launch_dln_as<6, false>(a, b, ep, M, N, K, s);
-        case 7: return r2 ? launch_dln_as<7, true>(a, b, ep, M, N, K, s) : launch_dln_as<7, false>(a, b, ep, M, N, K, s);
+        case 4: return launch_dln_nj<4>(a_fmt, a, b, ep, M, N, K, s);
+        case 5: return launch_dln_nj<5>(a_fmt, a, b, ep, M, N, K, s);
+        case 6: return launch_dln_nj<6>(a_fmt, a, b, ep, M, N, K, s);
+        case 7: return launch_dln_nj<7>(a_fmt, a, b, ep, M, N, K, s);
     }
     NC_FAIL(-1, "fp8_gemm: tile widths of 128, 160, 192 and 224 columns only, not %d", 32 * nj);
 }
@@ -1188,11 +1193,17 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
         if (which == 0) {
             const int cus = cu_count();
             const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-            which = (K % 128 == 0 && 8 * t256 >= 5 * cus) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
+            which = (K % 128 == 0 && (8 * t256 >= 5 * cus || dl_narrow_fills(M, N))) ? ((t256 >= 2 * cus && dlp_eligible(M, N, K)) ? 9 : 8) : 5;
+            if (which == 8) {
+                const int nj = dl_pick_nj(M, N);
+                if (nj < 8) which = 8 + nj;               // 12 .. 15: the narrower 256-row tiles
+            }
         }
-        NC_CHECK_ARG(which == 5 || which == 8 || which == 9, "fp8_gemm: kernels 5, 8 and 9 take an e5m2 operand, not %d", force_kernel);
+        NC_CHECK_ARG(which == 5 || which == 8 || which == 9 || (which >= 12 && which <= 15),
+                     "fp8_gemm: kernels 5, 8, 9 and 12..15 take an e5m2 operand, not %d", force_kernel);
         NcProfScope prof(1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
-        int rc = which == 5 ? launch_bl<128, 128, 2, 2, true, 1>(a, b, ep, M, N, K, s) : launch_dl<1>(a, b, ep, M, N, K, which == 9, s);
+        int rc = which == 5 ? launch_bl<128, 128, 2, 2, true, 1>(a, b, ep, M, N, K, s)
+                            : (which >= 12 ? launch_dln(which - 8, 1, a, b, ep, M, N, K, s) : launch_dl<1>(a, b, ep, M, N, K, which == 9, s));
         if (rc) return rc;
         NC_CHECK_LAUNCH("fp8_gemm");
         return 0;
@@ -1260,7 +1271,7 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     else if (which == 9) rc = launch_dl<0>(a, b, ep, M, N, K, true, s);
     else if (which == 10) rc = launch_bl<64, 128, 2, 2, true>(a, b, ep, M, N, K, s);
     else if (which == 11) rc = launch_bl<96, 128, 2, 2, true>(a, b, ep, M, N, K, s);
-    else if (which >= 12) rc = launch_dln(which - 8, a, b, ep, M, N, K, s);
+    else if (which >= 12) rc = launch_dln(which - 8, 0, a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;
     NC_CHECK_LAUNCH("fp8_gemm");

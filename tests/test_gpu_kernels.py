@@ -609,6 +609,8 @@ def test_quantize_with_transposed_copy_is_the_quantizer_plus_an_exact_transpose(
     (300, 320, 256, 8), (513, 272, 1664, 8), (4100, 2100, 384, 8),
     (2048, 1664, 256, 9), (2000, 1000, 384, 9), (8192, 4992, 128, 9),
     (64, 1664, 6656, 0), (2048, 6656, 1664, 0), (1664, 6656, 2048, 0), (8192, 1664, 256, 0),
+    # the narrower 256-row tiles with an e5m2 first operand, and the shapes whose choice they are (the weight gradients of d26)
+    (300, 324, 256, 12), (1000, 1004, 512, 13), (513, 272, 1664, 14), (700, 2244, 384, 15), (4992, 1664, 2048, 0), (1664, 6656, 1024, 0),
 ])
 def test_grad_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     say(f"grad gemm M={M} N={N} K={K} kernel={kernel}")
@@ -626,7 +628,7 @@ def test_grad_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     assert err <= 2e-3, err           # same fp8 inputs: only summation order and one bf16 rounding differ
 
 
-@pytest.mark.parametrize("kernel,M", [(5, 256), (8, 256), (9, 2048)])
+@pytest.mark.parametrize("kernel,M", [(5, 256), (8, 256), (9, 2048), (13, 300), (15, 300)])
 def test_grad_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
     say(f"grad gemm exact kernel={kernel}")
     g = torch.Generator().manual_seed(10)
