@@ -849,6 +849,107 @@ __global__ __launch_bounds__(512) void gemm_dln_kernel(const uint8_t* __restrict
     dln_epilogue<NJ, RELU2>(acc, lds, ep, inv_a, sc, g, m0, n0, M, N);
 }
 
+// the operand loads of one K-step of gemm_dr_kernel: `st` is the wave's first 1 KB piece of the stage, its pieces lie 4 KB apart
+template <int A_P>
+__device__ __forceinline__ void dr_fetch(const uint8_t* A, int a_bytes, const uint8_t* B, int b_bytes, uint8_t* st, int b_part, const uint32_t* vo_a,
+                                         const uint32_t* vo_b, int k_off) {
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, b_bytes, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < A_P; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (lds_ptr_t)(st + i * 4096), 16, vo_a[i], k_off, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b, (lds_ptr_t)(st + b_part + i * 4096), 16, vo_b[i], k_off, 0, 0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Direct-to-LDS tiles for a narrow weight under a prompt: BM x 128 outputs (BM = 64, 96, 128), four waves (2 x 2, BM/2 x 64 each), and a
+// ring of FOUR operand stages.  Where the 256-row tiles would leave most CUs without one (1792 x 1664: 49 or 91 tiles), the launch is
+// one round of small tiles, one workgroup of one wave per SIMD on each CU: nothing hides the latency of a K-step's operands then but
+// the depth of the prefetch.  The register-staged tiles have two K-steps in flight and pay a ds_write phase per step; here the operands
+// of three steps ahead are on their way into LDS while one is multiplied, and a step costs its MFMAs or the L2's bandwidth, whichever
+// is longer.  Past the end of K the loads are issued all the same (the first step's operands again, into stages nobody reads), so that
+// the count the barrier waits for is the same in every step.
+template <int BM, int OUT_KIND>
+__global__ __launch_bounds__(256) void gemm_dr_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, EpilogueArgs ep, int M,
+                                                      int N, int K, int tiles_m, int tiles_n) {
+    constexpr int WTM = BM / 32, STAGE = (BM + 128) * 128, A_P = BM / 32, LOADS = A_P + 4;
+    // s_waitcnt vmcnt(2 * LOADS), other counters untouched: the loads of the two youngest steps may still be in flight
+    constexpr int WAIT2 = 0x0F70 | ((2 * LOADS) & 15) | (((2 * LOADS) >> 4) << 14);
+    extern __shared__ __align__(16) uint8_t lds[];
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * 128;
+    DlGeom g = dl_geom();
+    g.wm = g.wave >> 1, g.wn = g.wave & 1;
+    const int wave_s = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // piece i of this wave is the 1 KB block (wave + 4 i) of its operand's part of the stage: tile rows 8 wave + 32 i + sub
+    uint32_t vo_a[A_P], vo_b[4];
+#pragma unroll
+    for (int i = 0; i < A_P; i++) {
+        const int ra = m0 + 8 * g.wave + 32 * i + g.sub;
+        vo_a[i] = ra < M ? (uint32_t)ra * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int rb = n0 + 8 * g.wave + 32 * i + g.sub;
+        vo_b[i] = rb < N ? (uint32_t)rb * (uint32_t)K + g.gch * 16 : NC_BUF_OOB;
+    }
+    const int ksteps = K / 128;
+
+    v4f acc[WTM][4];
+#pragma unroll
+    for (int i = 0; i < WTM; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto fetch = [&](int t) {
+        dr_fetch<A_P>(A, M * K, B, N * K, lds + (t & 3) * STAGE + wave_s * 1024, BM * 128, vo_a, vo_b, t < ksteps ? t * 128 : 0);
+    };
+    auto compute = [&](int t) {
+        const uint8_t* st = lds + (t & 3) * STAGE;
+        const uint8_t* a = st + g.wm * (BM / 2) * 128;
+        const uint8_t* b = st + BM * 128 + g.wn * 64 * 128;
+        v8i af[WTM], bf[2];
+        bf[0] = dl_frag(b, g);
+#pragma unroll
+        for (int i = 0; i < WTM; i++) af[i] = dl_frag(a + i * 2048, g);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (j + 1 < 4) bf[(j + 1) & 1] = dl_frag(b + (j + 1) * 2048, g);
+#pragma unroll
+            for (int i = 0; i < WTM; i++) mfma_f8_acc_ordered<0>(acc[i][j], bf[j & 1], af[i]);
+        }
+    };
+    fetch(0);
+    fetch(1);
+    fetch(2);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(WAIT2);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    for (int kt = 0; kt < ksteps; kt++) {
+        fetch(kt + 3);                       // into the stage that was read in step kt - 1: everyone is past the barrier that ended it
+        compute(kt);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(WAIT2);   // the operands of step kt + 1 have landed (this wave's share; the barrier says everybody's)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
+    // the loads past the end of K are still landing in the stages: they must be done before the epilogue reuses the memory
+    dl_step_barrier();
+
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < WTM; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) asm volatile("" : "+a"(acc[i][j]));
+    const float inv_a = *ep.inv_a;
+    float sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sc[i] = ep.inv_b[i < ep.segs.nseg ? i : 0];
+    bl_epilogue<BM, 128, 2, 2, OUT_KIND>(acc, lds, ep, inv_a, sc, m0, n0, M, N);
+}
+
 // Epilogue of the persistent kernel: the wave's 64 x (128 | 64) block leaves 16 rows at a time through a 4 KB LDS region of
 // its own (past the two operand stages, so the loads of the next tile keep landing meanwhile), every store instruction
 // writing whole 128-byte lines.
@@ -1139,6 +1240,25 @@ static int launch_dln(int nj, int a_fmt, const uint8_t* a, const uint8_t* b, con
     NC_FAIL(-1, "fp8_gemm: tile widths of 128, 160, 192 and 224 columns only, not %d", 32 * nj);
 }
 
+template <int BM, int OUT_KIND>
+static int launch_dr_as(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + 127) / 128;
+    const size_t lds_bytes = 4 * (size_t)(BM + 128) * 128;
+    const void* fn = (const void*)gemm_dr_kernel<BM, OUT_KIND>;
+    hipError_t e = reserve_lds(fn, (int)lds_bytes);
+    if (e != hipSuccess) NC_FAIL(-2, "fp8_gemm: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    hipLaunchKernelGGL((gemm_dr_kernel<BM, OUT_KIND>), dim3(tiles_m * tiles_n), dim3(256), lds_bytes, s, a, b, ep, M, N, K, tiles_m, tiles_n);
+    return 0;
+}
+// e4m3 operands, bf16 or relu^2 output, K a multiple of 128
+template <int BM>
+static int launch_dr(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, hipStream_t s) {
+    NC_CHECK_ARG((long)M * K < (1L << 31) && (long)N * K < (1L << 31), "fp8_gemm: buffer-load kernels need M*K and N*K below 2^31");
+    NC_CHECK_ARG(K % 128 == 0, "fp8_gemm: the direct-to-LDS kernels need K %% 128 == 0, got %d", K);
+    NC_CHECK_ARG(ep.out_kind != 1, "fp8_gemm: the direct-to-LDS kernels write bf16 only");
+    return ep.out_kind == 2 ? launch_dr_as<BM, 2>(a, b, ep, M, N, K, s) : launch_dr_as<BM, 0>(a, b, ep, M, N, K, s);
+}
+
 // the relu^2 epilogue is a variant of its own so that the plain kernels keep their register budget
 template <int A_FMT>
 static int launch_dl(const uint8_t* a, const uint8_t* b, const EpilogueArgs& ep, int M, int N, int K, bool persistent, hipStream_t s) {
@@ -1211,7 +1331,8 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
 
     // force_kernel: 0 auto, 1 small-M, 4 plain-load tile 128x128, 5/6/7 buffer-load tiles 128x128 / 256x128 / 256x256,
     // 8 direct-to-LDS 256x256 tile by tile, 9 the same persistent, 10 / 11 buffer-load tiles 64x128 / 96x128,
-    // 12 .. 15 direct-to-LDS tiles of 256 x 128 / 160 / 192 / 224 tile by tile
+    // 12 .. 15 direct-to-LDS tiles of 256 x 128 / 160 / 192 / 224 tile by tile, 16 / 17 / 18 direct-to-LDS tiles of 64 / 96 / 128 x 128
+    // with four stages
     int which = force_kernel;
     if (which == 0) {
         if (M <= 128) which = 1;
@@ -1243,12 +1364,16 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
                     const long tn = (N + 127) / 128;
                     if ((long)((M + 63) / 64) * tn <= cus) which = 10;
                     else if ((long)((M + 95) / 96) * tn <= cus) which = 11;
+                    // the same tiles fed straight into a ring of four LDS stages where K allows it: three K-steps of operands on their
+                    // way instead of two and no ds_write phase (1792 x 1664 x 6656: 27.5 -> 25.6 us, 1024 rows: 21.9 -> 20.8 us; what is
+                    // left is the L2's bandwidth: 28 KB per K-step and CU for tiles this small)
+                    if (which >= 10 && K % 128 == 0 && out_kind == 0) which += 6;
                 }
             }
         }
     }
     int rc = 0;
-    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 15, "fp8_gemm: unknown kernel selector %d", force_kernel);
+    if (which != 1) NC_CHECK_ARG(which >= 4 && which <= 18, "fp8_gemm: unknown kernel selector %d", force_kernel);
     NcProfScope prof(which == 1 ? -1 : 1, 2.0 * M * N * K, s, ((int64_t)N << 32) | (uint32_t)K);
     if (which == 1) {
         NC_CHECK_ARG(M <= 128, "fp8_gemm: the small-M kernel needs M <= 128, got %d", M);
@@ -1271,6 +1396,9 @@ int nc_launch_gemm(const uint8_t* a, const uint8_t* b, const float* inv_a, const
     else if (which == 9) rc = launch_dl<0>(a, b, ep, M, N, K, true, s);
     else if (which == 10) rc = launch_bl<64, 128, 2, 2, true>(a, b, ep, M, N, K, s);
     else if (which == 11) rc = launch_bl<96, 128, 2, 2, true>(a, b, ep, M, N, K, s);
+    else if (which == 16) rc = launch_dr<64>(a, b, ep, M, N, K, s);
+    else if (which == 17) rc = launch_dr<96>(a, b, ep, M, N, K, s);
+    else if (which == 18) rc = launch_dr<128>(a, b, ep, M, N, K, s);
     else if (which >= 12) rc = launch_dln(which - 8, 0, a, b, ep, M, N, K, s);
     else NC_FAIL(-1, "fp8_gemm: unknown kernel selector %d", force_kernel);
     if (rc) return rc;

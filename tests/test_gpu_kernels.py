@@ -253,6 +253,9 @@ def make_operands(M, N, K, seed, outliers=True):
     # a tile, inside a wave's block and inside an 8-column piece, one / odd / even K-step counts, the shapes of the choice
     (300, 320, 256, 12), (513, 272, 1664, 12), (300, 324, 128, 13), (1000, 1004, 512, 13), (1792, 4992, 1664, 13), (257, 160, 384, 13),
     (300, 320, 256, 14), (700, 1148, 640, 14), (1792, 6656, 1664, 14), (300, 320, 256, 15), (900, 2244, 384, 15), (1792, 4992, 1664, 0),
+    # four-stage direct-to-LDS tiles of 64 / 96 / 128 x 128: fewer K-steps than stages (1, 2, 3), exactly four, many; ragged M and N
+    (300, 320, 128, 16), (129, 72, 256, 16), (513, 1664, 1664, 16), (300, 320, 384, 17), (193, 72, 512, 17), (1792, 1664, 1664, 17),
+    (1792, 1664, 6656, 17), (300, 324, 640, 18), (1000, 1004, 128, 18), (2048, 1664, 1664, 18),
 ])
 def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
     say(f"gemm M={M} N={N} K={K} kernel={kernel}")
@@ -271,7 +274,7 @@ def test_gemm_matches_emulated_matmul(ops, M, N, K, kernel):
 
 
 @pytest.mark.parametrize("kernel,M", [(1, 48), (4, 128), (5, 256), (6, 128), (7, 256), (8, 256), (9, 2048), (10, 200), (11, 200),
-                                      (12, 300), (13, 300), (14, 300), (15, 300)])
+                                      (12, 300), (13, 300), (14, 300), (15, 300), (16, 200), (17, 200), (18, 200)])
 def test_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
     say(f"gemm exact powers of two kernel={kernel}")
     g = torch.Generator().manual_seed(9)
@@ -320,7 +323,7 @@ def test_gemm_stacked_weights_use_their_own_scales(ops):
     a8b, iab, _ = fp8_ref.to_fp8(a_big)
     want_big = torch.cat([fp8_ref.scaled_mm_emulated(a8b, p, iab, inv) for p, inv, _ in q], dim=1)
     got8 = None
-    for kernel in (8, 5, 7, 9, 10, 11, 12, 13, 14, 15):
+    for kernel in (8, 5, 7, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18):
         got = ops.fp8_gemm(a8b.to(DEV), w8.to(DEV), iab.to(DEV), inv_w.to(DEV), seg_ends=[256, 384, 512], kernel=kernel).cpu()
         assert rel_l2(got, want_big) < 2e-3, kernel
         # the direct-to-LDS kernels add the K-steps in the same order whatever their tile width: the same bits
@@ -332,7 +335,8 @@ def test_gemm_stacked_weights_use_their_own_scales(ops):
 
 @pytest.mark.parametrize("M,N,K,kernel", [(300, 320, 256, 5), (513, 272, 400, 5), (300, 320, 256, 7), (300, 320, 256, 8), (1000, 1000, 512, 8),
                                           (2048, 1664, 256, 9), (2000, 1000, 384, 9), (1792, 6656, 1664, 0), (2048, 6656, 256, 0),
-                                          (300, 324, 256, 12), (1000, 1004, 512, 13), (1792, 6656, 1664, 14), (700, 2244, 384, 15)])
+                                          (300, 324, 256, 12), (1000, 1004, 512, 13), (1792, 6656, 1664, 14), (700, 2244, 384, 15),
+                                          (300, 324, 256, 16), (1000, 1004, 512, 17), (700, 2244, 384, 18)])
 def test_gemm_relu2_epilogue_and_amax(ops, M, N, K, kernel):
     say(f"gemm relu2 M={M} N={N} K={K} kernel={kernel}")
     a, w = make_operands(M, N, K, seed=M + N + K)
