@@ -92,7 +92,9 @@ int nc_fp8_transpose(const uint8_t* src, int rows, int cols, uint8_t* dst, nc_st
  * softcap*tanh(bf16(v)/softcap), i.e. lm_head followed by nanochat/gpt.py:512-515.
  * kernel: 0 auto, 1 small-M (M<=128), 4 plain-load tile 128x128 (any operand size), 5/6/7 buffer-load tiles
  * 128x128 / 256x128 / 256x256 (operands below 2 GiB each), 8 direct-to-LDS 256x256 tiles and 9 their persistent
- * form (bf16 output, K a multiple of 128; 9 also needs ceil(M/256) in {8,16,...,256}), 10 / 11 buffer-load tiles 64x128 / 96x128.
+ * form (bf16 output, K a multiple of 128; 9 also needs ceil(M/256) in {8,16,...,256}), 10 / 11 buffer-load tiles 64x128 / 96x128,
+ * 12..15 direct-to-LDS tiles of 256 x 128 / 160 / 192 / 224 (one tile per workgroup), 16 / 17 / 18 direct-to-LDS tiles of 64 / 96 / 128 x 128
+ * through four LDS stages (12..18: bf16 output, K a multiple of 128).
  * workspace (may be NULL): lets the small-M kernel split K over workgroups (fp32 partial sums, added
  * in a fixed order by a finishing kernel); size from nc_fp8_small_m_workspace_bytes(), 16-byte aligned. */
 int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b,
@@ -104,13 +106,14 @@ int nc_fp8_gemm_tn(const uint8_t* a, const uint8_t* b, const float* inv_a, const
  * its transpose), b in e4m3fn (the transposed weight or input payload saved by the forward), K contiguous in both.
  *   grad_input [B,K']  = nc_fp8_gemm_tn_grad(go[B,N'],   wT[K',N'], ...)   M=B,  N=K', K=N'
  *   grad_weight[N',K'] = nc_fp8_gemm_tn_grad(goT[N',B],  xT[K',B],  ...)   M=N', N=K', K=B
- * kernel: 0 auto, 5 (128x128 tiles, any K multiple of 16), 8 / 9 (direct-to-LDS 256x256 tiles, K multiple of 128). */
+ * kernel: 0 auto, 5 (128x128 tiles, any K multiple of 16), 8 / 9 (direct-to-LDS 256x256 tiles, K multiple of 128), 12..15 (direct-to-LDS
+ * tiles of 256 x 128 / 160 / 192 / 224, K multiple of 128). */
 int nc_fp8_gemm_tn_grad(const uint8_t* a_e5m2, const uint8_t* b, const float* inv_a, const float* inv_b, void* out, int M,
                         int N, int K, int ldc, int kernel, nc_stream_t stream);
 
 /* The MLP's first linear with its activation (nanochat/gpt.py:138-139, c_fc then relu().square()) for M > 128 rows:
  * out[M,N] = bf16(relu(bf16(v))^2), v as in nc_fp8_gemm_tn, and atomicMax(*out_amax, fp32 bits of max(out)) so that the
- * next tensorwise quantization needs no amax pass; the caller clears *out_amax.  kernel: 0 auto, 5..9. */
+ * next tensorwise quantization needs no amax pass; the caller clears *out_amax.  kernel: 0 auto, 5..9, 12..18. */
 int nc_fp8_gemm_tn_relu2(const uint8_t* a, const uint8_t* b, const float* inv_a, const float* inv_b, void* out,
                          uint32_t* out_amax, int M, int N, int K, int ldc, int kernel, nc_stream_t stream);
 
