@@ -290,6 +290,27 @@ def test_gemm_power_of_two_inputs_bit_exact(ops, kernel, M):
     assert torch.equal(got, want)
 
 
+def test_gemm_direct_to_lds_kernels_agree_bit_for_bit_on_seeded_shapes(ops):
+    """Every direct-to-LDS kernel adds the K-steps of an output in the same order, whatever its tile: on twelve seeded ragged shapes the
+    narrower 256-row tiles (12..15) and the four-stage tiles (16..18) give the bits of the 256 x 256 tile (8), which the other tests
+    hold against the oracle."""
+    say("direct-to-LDS kernels, seeded shapes")
+    import random
+    rnd = random.Random(7)
+    for _ in range(12):
+        M = rnd.choice([129, 200, 257, 500, 777, 1000, 1793])
+        N = 4 * rnd.choice([5, 18, 40, 81, 250, 416, 601])
+        K = 128 * rnd.choice([1, 2, 3, 4, 5, 8, 13])
+        a, w = make_operands(M, N, K, seed=M + 3 * N + K)
+        a8, ia, _ = fp8_ref.to_fp8(a)
+        w8, iw, _ = fp8_ref.to_fp8(w)
+        ad, wd, iad, iwd = a8.to(DEV), w8.to(DEV), ia.to(DEV), iw.reshape(1).to(DEV)
+        want = ops.fp8_gemm(ad, wd, iad, iwd, kernel=8)
+        for kernel in (12, 13, 14, 15, 16, 17, 18):
+            got = ops.fp8_gemm(ad, wd, iad, iwd, kernel=kernel)
+            assert torch.equal(got, want), (M, N, K, kernel)
+
+
 def test_gemm_one_hot_weight_is_a_gather(ops):
     say("gemm one-hot")
     M, N, K = 64, 128, 256
