@@ -44,11 +44,17 @@ __device__ __forceinline__ v8bf as_v8bf(uint4 v) { return __builtin_bit_cast(v8b
 // query), and a sub-block that all of its queries see in full takes the path without the mask arithmetic.  The running maximum only
 // triggers a rescale of the 64 output accumulators when it moved for some lane of the wave.  Tiles are handed out from the end of the
 // sequence, longest key ranges first.
+// Which (tile, head) unit the workgroup with a given linear index takes, when the launch says so (one row, every key visible, a
+// grid of at most 512 workgroups): see pf_balance_units.
+struct PfUnitMap {
+    int on;
+    uint16_t unit[512];
+};
 template <int GS, int KS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                                                            const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ cache_seqlens,
                                                            int window_left, int seqlens_include_new, bf16_t* __restrict__ out,
-                                                           uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax) {
+                                                           uint32_t* __restrict__ amax_ws, int T, int H, int Hkv, int Tmax, PfUnitMap map) {
     constexpr int QT = 128 / (GS * KS);                        // queries per workgroup
     __shared__ __align__(16) uint8_t lds[2 * PF_KBYTES + 2 * PF_VBYTES];
     __shared__ float red[4];
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     {
         const int nx = gridDim.x, total = nx * (int)gridDim.y, lid = (int)blockIdx.x + nx * (int)blockIdx.y;
         const int xcd = lid & 7, slot = lid >> 3;
-        const int unit = xcd * (total >> 3) + min(xcd, total & 7) + slot;
+        const int unit = map.on ? (int)map.unit[lid] : xcd * (total >> 3) + min(xcd, total & 7) + slot;
         hy = unit / nx;
         qb0 = (nx - 1 - unit % nx) * QT;
     }
@@ -530,6 +536,39 @@ int nc_launch_attention_shared_prefix(const bf16_t* q, const bf16_t* k_cache, co
     return 0;
 }
 
+// A causal launch over one long row has tiles of very different lengths (tile t of a head reads t + 1 blocks of keys) and more workgroups
+// than CUs, but fewer than two per CU: some CUs get two workgroups that then run at half speed each, and with the plain order (each XCD:
+// a run of units, longest first) the second workgroup of a CU lands beside one of the longest.  Here each XCD's units are dealt so that
+// the longest stay alone and the rest are paired long with short: with C CUs per XCD and P = units - C pairs, the workgroups dispatched
+// P .. C-1 (alone on their CU, if the dispatcher deals the second round in the order of the first) take the longest units, 0 .. P-1 the
+// next longest and C + k the (k+1)-th shortest.  Only the order changes, every unit is still computed by exactly one workgroup.
+// d26, 1792 tokens, full-context layers (28 tiles x 13 heads = 364 workgroups): 40 -> 33.3 us, which is the longest tile alone on its CU.
+static void pf_balance_units(PfUnitMap& map, int nx, int ny, int cus) {
+    const int total = nx * ny, C = cus / 8;
+    map.on = 0;
+    if (total > 512 || C <= 0) return;
+    for (int xcd = 0; xcd < 8; xcd++) {
+        const int per = (total >> 3) + (xcd < (total & 7) ? 1 : 0), base = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7));
+        if (per <= C || per > 2 * C) return;
+        // units of this XCD in descending length: a unit's length grows with its tile index nx - 1 - unit % nx
+        int order[128];
+        if (per > 128) return;
+        for (int i = 0; i < per; i++) order[i] = base + i;
+        for (int i = 1; i < per; i++) {              // insertion sort, stable: longest first
+            const int u = order[i], key = nx - 1 - u % nx;
+            int j = i - 1;
+            while (j >= 0 && (nx - 1 - order[j] % nx) < key) order[j + 1] = order[j], j--;
+            order[j + 1] = u;
+        }
+        const int P = per - C, S = C - P;
+        for (int slot = 0; slot < per; slot++) {
+            const int rank = slot < P ? S + slot : (slot < C ? slot - P : per - 1 - (slot - C));
+            map.unit[xcd + 8 * slot] = (uint16_t)order[rank];
+        }
+    }
+    map.on = 1;
+}
+
 int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* cache_seqlens,
                                 int window_left, bf16_t* out, int B, int T, int H, int Hkv, int Tmax, int seqlens_include_new,
                                 uint32_t* amax_ws, hipStream_t s) {
@@ -548,9 +587,13 @@ int nc_launch_attention_prefill(const bf16_t* q, const bf16_t* k_cache, const bf
     const int QT = 128 / (GS * KS);
     const dim3 grid((T + QT - 1) / QT, Hkv * (G / GS), B);
     NC_CHECK_ARG(grid.y <= 65535, "prefill_attention: too many heads in one launch");
+    PfUnitMap map;                         // passed by value
+    map.on = 0;
+    // one row whose queries see every key before them (a window of at least the cache length is none): the long prompt of a prefill
+    if (B == 1 && (window_left < 0 || window_left >= Tmax)) pf_balance_units(map, (int)grid.x, (int)grid.y, nc_cu_count());
 #define PF_LAUNCH(GG, KK)                                                                                                              \
     hipLaunchKernelGGL((attn_prefill_kernel<GG, KK>), grid, dim3(256), 0, s, q, k_cache, v_cache, cache_seqlens, window_left,          \
-                       seqlens_include_new, out, amax_ws, T, H, Hkv, Tmax)
+                       seqlens_include_new, out, amax_ws, T, H, Hkv, Tmax, map)
     if (GS == 4) PF_LAUNCH(4, 1);
     else if (GS == 2 && KS == 2) PF_LAUNCH(2, 2);
     else if (GS == 2) PF_LAUNCH(2, 1);

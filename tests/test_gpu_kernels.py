@@ -911,6 +911,17 @@ def test_attention_many_queries_per_row(ops, T, window, H, Hkv, seqlens):
     attn_case(ops, 2, T, H, Hkv, 512, seqlens, window, 0, seed=T + H)
 
 
+@pytest.mark.parametrize("T,H,window,pos0,Tmax", [(1792, 13, -1, 0, 1792), (1792, 10, 4096, 0, 1792), (1408, 13, -1, 0, 1500),
+                                                 (1700, 13, 2000, 100, 1800), (1792, 13, 512, 0, 1792)])
+def test_attention_one_long_row_in_the_balanced_order(ops, T, H, window, pos0, Tmax):
+    """One row of 1400..1800 queries that see every key before them: more workgroups than CUs and fewer than two per CU, so the launch
+    deals its (tile, head) units in the balanced order (longest alone, the rest paired long with short).  Every unit must still be
+    computed exactly once: the whole output against the oracle, with the cache position at zero and past zero; a 512-key window
+    (the plain order) beside it."""
+    say(f"attention, one long row T={T} H={H} window={window} pos0={pos0}")
+    attn_case(ops, 1, T, H, H, Tmax, [pos0], window, 0, seed=T + H + pos0)
+
+
 @pytest.mark.parametrize("B,T,H,Hkv,window", [(64, 40, 8, 8, -1), (64, 100, 8, 4, 48), (70, 33, 4, 1, -1)])
 def test_attention_many_rows_of_many_queries(ops, B, T, H, Hkv, window):
     """Enough (row, head, tile) units that every query block gets a wave of its own with the whole key range (launches with
